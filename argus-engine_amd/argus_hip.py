@@ -1,0 +1,317 @@
+"""ctypes binding of libargus_hip.so (the C ABI declared in include/argus_hip.h).
+
+This module is plumbing for tests and bench.py: it loads the in-tree shared library, mirrors
+the argument structs field for field and passes raw device pointers (torch tensors are used
+only as device memory and for the stream handle).  There is no fallback: if the library is
+missing, importing this module raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libargus_hip.so")
+
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_RUNTIME, ERR_NOMEM = 0, -1, -2, -3, -4
+F32, F16 = 0, 1
+HEAD_MAJOR, SEQ_MAJOR = 0, 1
+
+EXPORTED_SYMBOLS = [
+    "argus_hip_create", "argus_hip_destroy", "argus_hip_abi_version", "argus_hip_last_error",
+    "argus_hip_get_device_info", "argus_hip_kernel_timing_begin", "argus_hip_kernel_timing_end",
+    "argus_hip_malloc", "argus_hip_free", "argus_hip_write_buffer",
+    "argus_hip_read_buffer", "argus_hip_copy_slice", "argus_hip_synchronize",
+    "argus_hip_attention_gen", "argus_hip_flash_attention_prefill",
+    "argus_hip_has_quant_attn_kernel", "argus_hip_attention_gen_quant",
+    "argus_hip_attention_gen_quant_ex", "argus_hip_gather_update_quant", "argus_hip_quant_flush",
+    "argus_hip_score_reduce", "argus_hip_score_reduce_per_layer",
+    "argus_hip_kv_scatter_f32_to_f16", "argus_hip_kv_scatter_f32_to_f16_batch",
+    "argus_hip_kv_scatter_f32_batch",
+]
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libargus_hip.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
+        "(or `make -C argus-engine_amd/csrc`) first; there is no CPU fallback")
+
+# torch bundles its own HIP runtime under the same soname as /opt/rocm's; whichever is loaded
+# first serves the whole process.  Import torch first so the tensors handed to the library and
+# the library's own launches go through one runtime.
+import torch  # noqa: E402,F401
+
+lib = C.CDLL(LIB_PATH)
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("compute_units", C.c_int32), ("clock_mhz", C.c_int32),
+                ("wavefront_size", C.c_int32), ("lds_bytes_per_block", C.c_int32),
+                ("hbm_bytes", C.c_int64), ("name", C.c_char * 128), ("gcn_arch", C.c_char * 64)]
+
+
+class AttentionGenArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("q", C.c_void_p), ("k_cache", C.c_void_p),
+                ("v_cache", C.c_void_p), ("out", C.c_void_p), ("scores_out", C.c_void_p),
+                ("kv_index", C.c_void_p),
+                ("num_heads_q", C.c_int32), ("num_heads_kv", C.c_int32), ("head_dim", C.c_int32),
+                ("cache_seq_len", C.c_int32), ("capacity", C.c_int32), ("kv_start", C.c_int32),
+                ("layout", C.c_int32), ("kv_dtype", C.c_int32), ("batch", C.c_int32),
+                ("score_stride", C.c_int32),
+                ("q_batch_stride", C.c_int64), ("out_batch_stride", C.c_int64),
+                ("kv_batch_stride", C.c_int64), ("score_batch_stride", C.c_int64),
+                ("index_batch_stride", C.c_int64),
+                ("softcap", C.c_float), ("scale", C.c_float)]
+
+
+class PrefillArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("q", C.c_void_p), ("k_cache", C.c_void_p),
+                ("v_cache", C.c_void_p), ("out", C.c_void_p),
+                ("n_heads_q", C.c_int32), ("n_heads_kv", C.c_int32), ("seq_len", C.c_int32),
+                ("cache_seq_len", C.c_int32), ("head_dim", C.c_int32), ("kv_capacity", C.c_int32),
+                ("batch_size", C.c_int32), ("is_head_major", C.c_int32), ("q_dtype", C.c_int32),
+                ("kv_dtype", C.c_int32), ("out_dtype", C.c_int32), ("window", C.c_int32)]
+
+
+class QuantAttnArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("q_mem", C.c_uint64), ("qk_mem", C.c_uint64),
+                ("qv_mem", C.c_uint64), ("res_k_mem", C.c_uint64), ("res_v_mem", C.c_uint64),
+                ("out_mem", C.c_uint64), ("scores_out", C.c_void_p), ("scores_len", C.c_size_t),
+                ("num_heads_q", C.c_size_t), ("num_heads_kv", C.c_size_t), ("head_dim", C.c_size_t),
+                ("q_tokens", C.c_size_t), ("res_tokens", C.c_size_t), ("res_cap", C.c_size_t),
+                ("scale", C.c_float), ("bits", C.c_uint8)]
+
+
+class QuantAttnExt(C.Structure):
+    _fields_ = [("scores_dev", C.c_uint64), ("score_stride", C.c_size_t),
+                ("res_dtype", C.c_int32), ("softcap", C.c_float)]
+
+
+class QuantGatherArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("input_mem", C.c_uint64), ("residual_mem", C.c_uint64),
+                ("kv_heads", C.c_size_t), ("res_cap", C.c_size_t), ("head_dim", C.c_size_t),
+                ("seq_len", C.c_size_t), ("res_pos", C.c_size_t)]
+
+
+class QuantFlushArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("res_k_mem", C.c_uint64), ("res_v_mem", C.c_uint64),
+                ("qk_mem", C.c_uint64), ("qv_mem", C.c_uint64), ("kv_heads", C.c_size_t),
+                ("res_cap", C.c_size_t), ("head_dim", C.c_size_t), ("flush_tokens", C.c_size_t),
+                ("k_block_start", C.c_size_t), ("v_block_start", C.c_size_t), ("bits", C.c_uint8)]
+
+
+class ScoreReduceArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("score_buf", C.c_uint64), ("importance", C.c_uint64),
+                ("head_importance", C.c_uint64), ("decay_factor", C.c_float),
+                ("n_layers", C.c_size_t), ("n_heads_q", C.c_size_t), ("n_kv_heads", C.c_size_t),
+                ("cache_seq_len", C.c_size_t), ("score_stride", C.c_size_t),
+                ("max_seq_len", C.c_size_t), ("layer_flat_importance", C.c_uint64)]
+
+
+def _bind():
+    vp, i32 = C.c_void_p, C.c_int32
+    lib.argus_hip_create.argtypes = [C.c_int, C.POINTER(vp)]
+    lib.argus_hip_destroy.argtypes = [vp]
+    lib.argus_hip_abi_version.argtypes = []
+    lib.argus_hip_last_error.argtypes = [vp]
+    lib.argus_hip_last_error.restype = C.c_char_p
+    lib.argus_hip_get_device_info.argtypes = [vp, C.POINTER(DeviceInfo)]
+    lib.argus_hip_kernel_timing_begin.argtypes = [vp, i32]
+    lib.argus_hip_kernel_timing_end.argtypes = [vp, C.POINTER(C.c_float), i32, C.POINTER(i32)]
+    lib.argus_hip_malloc.argtypes = [vp, C.c_size_t, C.POINTER(vp)]
+    lib.argus_hip_free.argtypes = [vp, vp]
+    lib.argus_hip_write_buffer.argtypes = [vp, vp, vp, vp, C.c_size_t]
+    lib.argus_hip_read_buffer.argtypes = [vp, vp, vp, vp, C.c_size_t]
+    lib.argus_hip_copy_slice.argtypes = [vp, vp, vp, vp, C.c_size_t]
+    lib.argus_hip_synchronize.argtypes = [vp, vp]
+    lib.argus_hip_attention_gen.argtypes = [vp, C.POINTER(AttentionGenArgs)]
+    lib.argus_hip_flash_attention_prefill.argtypes = [vp, C.POINTER(PrefillArgs)]
+    lib.argus_hip_has_quant_attn_kernel.argtypes = [vp, C.c_uint8]
+    lib.argus_hip_attention_gen_quant.argtypes = [vp, C.POINTER(QuantAttnArgs)]
+    lib.argus_hip_attention_gen_quant_ex.argtypes = [vp, C.POINTER(QuantAttnArgs), C.POINTER(QuantAttnExt)]
+    lib.argus_hip_gather_update_quant.argtypes = [vp, C.POINTER(QuantGatherArgs)]
+    lib.argus_hip_quant_flush.argtypes = [vp, C.POINTER(QuantFlushArgs)]
+    lib.argus_hip_score_reduce.argtypes = [vp, C.POINTER(ScoreReduceArgs)]
+    lib.argus_hip_score_reduce_per_layer.argtypes = [vp, C.POINTER(ScoreReduceArgs)]
+    sc16 = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32]
+    lib.argus_hip_kv_scatter_f32_to_f16.argtypes = sc16
+    lib.argus_hip_kv_scatter_f32_to_f16_batch.argtypes = sc16 + [i32]
+    lib.argus_hip_kv_scatter_f32_batch.argtypes = sc16 + [i32]
+    for name in EXPORTED_SYMBOLS:
+        if name != "argus_hip_last_error":
+            getattr(lib, name).restype = C.c_int
+
+
+_bind()
+
+
+class ArgusHipError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("argus_hip rc=%d: %s" % (code, msg))
+        self.code = code
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _kv_dtype(t):
+    import torch
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.float32:
+        return F32
+    raise TypeError("unsupported KV dtype %s" % t.dtype)
+
+
+class Context:
+    """Owns one argus_hip_ctx.  Methods take torch CUDA tensors and return the C return code
+    (raising ArgusHipError on a negative one unless check=False)."""
+
+    def __init__(self, device=0):
+        h = C.c_void_p()
+        rc = lib.argus_hip_create(device, C.byref(h))
+        if rc != OK:
+            raise ArgusHipError(rc, "argus_hip_create failed (no HIP device?)")
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            lib.argus_hip_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def last_error(self):
+        return lib.argus_hip_last_error(self.handle).decode()
+
+    def _check(self, rc, check=True):
+        if rc < 0 and check:
+            raise ArgusHipError(rc, self.last_error())
+        return rc
+
+    def device_info(self):
+        info = DeviceInfo()
+        self._check(lib.argus_hip_get_device_info(self.handle, C.byref(info)))
+        return info
+
+    def kernel_timing_begin(self, max_launches):
+        self._check(lib.argus_hip_kernel_timing_begin(self.handle, max_launches))
+
+    def kernel_timing_end(self, capacity=4096):
+        """Per-launch durations (ms) of the dominant kernel since kernel_timing_begin."""
+        buf = (C.c_float * capacity)()
+        n = C.c_int32(0)
+        self._check(lib.argus_hip_kernel_timing_end(self.handle, buf, capacity, C.byref(n)))
+        return [buf[i] for i in range(min(n.value, capacity))]
+
+    # -- (a-1) ---------------------------------------------------------------------------
+    def attention_gen(self, q, k, v, out, num_heads_kv, cache_seq_len, capacity=0,
+                      layout=HEAD_MAJOR, scores=None, score_stride=0, kv_index=None, kv_start=0,
+                      batch=1, kv_batch_stride=0, index_batch_stride=0, softcap=0.0, scale=0.0,
+                      check=True):
+        """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride]."""
+        hq, d = q.shape[-2], q.shape[-1]
+        a = AttentionGenArgs(
+            stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),
+            scores_out=_ptr(scores), kv_index=_ptr(kv_index), num_heads_q=hq,
+            num_heads_kv=num_heads_kv, head_dim=d, cache_seq_len=cache_seq_len, capacity=capacity,
+            kv_start=kv_start, layout=layout, kv_dtype=_kv_dtype(k), batch=batch,
+            score_stride=score_stride, q_batch_stride=0, out_batch_stride=0,
+            kv_batch_stride=kv_batch_stride, score_batch_stride=0,
+            index_batch_stride=index_batch_stride, softcap=softcap, scale=scale)
+        return self._check(lib.argus_hip_attention_gen(self.handle, C.byref(a)), check)
+
+    # -- (a-2) ---------------------------------------------------------------------------
+    def flash_attention_prefill(self, q, k, v, out, n_heads_q, n_heads_kv, seq_len, cache_seq_len,
+                                head_dim, kv_capacity, batch_size=1, is_head_major=True, window=0,
+                                check=True):
+        a = PrefillArgs(
+            stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),
+            n_heads_q=n_heads_q, n_heads_kv=n_heads_kv, seq_len=seq_len,
+            cache_seq_len=cache_seq_len, head_dim=head_dim, kv_capacity=kv_capacity,
+            batch_size=batch_size, is_head_major=int(is_head_major), q_dtype=_kv_dtype(q),
+            kv_dtype=_kv_dtype(k), out_dtype=_kv_dtype(out), window=window)
+        return self._check(lib.argus_hip_flash_attention_prefill(self.handle, C.byref(a)), check)
+
+    # -- (a-3) ---------------------------------------------------------------------------
+    def has_quant_attn_kernel(self, bits):
+        return lib.argus_hip_has_quant_attn_kernel(self.handle, bits) == 1
+
+    def attention_gen_quant(self, q, qk, qv, res_k, res_v, out, num_heads_kv, q_tokens, res_tokens,
+                            res_cap, scale, bits, scores_host=None, scores_dev=None,
+                            score_stride=0, softcap=0.0, check=True):
+        """scores_host: numpy float32 array (host readback, reference contract);
+        scores_dev: torch tensor (device)."""
+        import torch
+        hq, d = q.shape
+        a = QuantAttnArgs(
+            stream=_stream(), q_mem=_ptr(q), qk_mem=_ptr(qk), qv_mem=_ptr(qv),
+            res_k_mem=_ptr(res_k), res_v_mem=_ptr(res_v), out_mem=_ptr(out),
+            scores_out=(scores_host.ctypes.data if scores_host is not None else None),
+            scores_len=(scores_host.size if scores_host is not None else 0), num_heads_q=hq,
+            num_heads_kv=num_heads_kv, head_dim=d, q_tokens=q_tokens, res_tokens=res_tokens,
+            res_cap=res_cap, scale=scale, bits=bits)
+        res_dtype = F16 if res_k.dtype == torch.float16 else F32
+        if scores_dev is None and res_dtype == F32 and softcap == 0.0:
+            return self._check(lib.argus_hip_attention_gen_quant(self.handle, C.byref(a)), check)
+        e = QuantAttnExt(scores_dev=_ptr(scores_dev), score_stride=score_stride,
+                         res_dtype=res_dtype, softcap=softcap)
+        return self._check(lib.argus_hip_attention_gen_quant_ex(self.handle, C.byref(a), C.byref(e)), check)
+
+    def gather_update_quant(self, inp, residual, kv_heads, res_cap, head_dim, seq_len, res_pos,
+                            check=True):
+        a = QuantGatherArgs(stream=_stream(), input_mem=_ptr(inp), residual_mem=_ptr(residual),
+                            kv_heads=kv_heads, res_cap=res_cap, head_dim=head_dim, seq_len=seq_len,
+                            res_pos=res_pos)
+        return self._check(lib.argus_hip_gather_update_quant(self.handle, C.byref(a)), check)
+
+    def quant_flush(self, res_k, res_v, qk, qv, kv_heads, res_cap, head_dim, flush_tokens,
+                    k_block_start, v_block_start, bits, check=True):
+        a = QuantFlushArgs(stream=_stream(), res_k_mem=_ptr(res_k), res_v_mem=_ptr(res_v),
+                           qk_mem=_ptr(qk), qv_mem=_ptr(qv), kv_heads=kv_heads, res_cap=res_cap,
+                           head_dim=head_dim, flush_tokens=flush_tokens,
+                           k_block_start=k_block_start, v_block_start=v_block_start, bits=bits)
+        return self._check(lib.argus_hip_quant_flush(self.handle, C.byref(a)), check)
+
+    # -- (a-4) ---------------------------------------------------------------------------
+    def _score_args(self, scores, importance, head_importance, decay_factor, n_layers, n_heads_q,
+                    n_kv_heads, cache_seq_len, score_stride, max_seq_len, layer_flat):
+        return ScoreReduceArgs(
+            stream=_stream(), score_buf=_ptr(scores), importance=_ptr(importance),
+            head_importance=_ptr(head_importance), decay_factor=decay_factor, n_layers=n_layers,
+            n_heads_q=n_heads_q, n_kv_heads=n_kv_heads, cache_seq_len=cache_seq_len,
+            score_stride=score_stride, max_seq_len=max_seq_len,
+            layer_flat_importance=_ptr(layer_flat))
+
+    def score_reduce(self, scores, importance, head_importance, decay_factor, n_layers, n_heads_q,
+                     n_kv_heads, cache_seq_len, score_stride, max_seq_len, check=True):
+        a = self._score_args(scores, importance, head_importance, decay_factor, n_layers, n_heads_q,
+                             n_kv_heads, cache_seq_len, score_stride, max_seq_len, None)
+        return self._check(lib.argus_hip_score_reduce(self.handle, C.byref(a)), check)
+
+    def score_reduce_per_layer(self, scores, layer_flat, decay_factor, n_layers, n_heads_q,
+                               n_kv_heads, cache_seq_len, score_stride, max_seq_len, check=True):
+        a = self._score_args(scores, None, None, decay_factor, n_layers, n_heads_q, n_kv_heads,
+                             cache_seq_len, score_stride, max_seq_len, layer_flat)
+        return self._check(lib.argus_hip_score_reduce_per_layer(self.handle, C.byref(a)), check)
+
+    # -- (f-1) ---------------------------------------------------------------------------
+    def kv_scatter(self, k_src, v_src, k_dst, v_dst, kv_heads, head_dim, capacity, write_pos,
+                   seq_len=None, check=True):
+        import torch
+        args = [self.handle, _stream(), _ptr(k_src), _ptr(v_src), _ptr(k_dst), _ptr(v_dst),
+                kv_heads, head_dim, capacity, write_pos]
+        if k_dst.dtype == torch.float32:
+            rc = lib.argus_hip_kv_scatter_f32_batch(*args, 1 if seq_len is None else seq_len)
+        elif seq_len is None:
+            rc = lib.argus_hip_kv_scatter_f32_to_f16(*args)
+        else:
+            rc = lib.argus_hip_kv_scatter_f32_to_f16_batch(*args, seq_len)
+        return self._check(rc, check)

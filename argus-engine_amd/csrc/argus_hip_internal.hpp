@@ -1,0 +1,111 @@
+// Internal helpers shared by the gfx950 kernels and the C-ABI glue.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+#include "../../include/argus_hip.h"
+
+#define ARGUS_API extern "C" __attribute__((visibility("default")))
+
+struct argus_hip_ctx {
+  int device = 0;
+  int compute_units = 0;
+  hipDeviceProp_t props;
+  // Split-KV partial workspace: per (sequence, Q head, split) one (m, l) pair and one
+  // un-normalised output row.  Grown on demand, never shrunk.
+  float *ws = nullptr;
+  size_t ws_bytes = 0;
+  // Event pairs of argus_hip_kernel_timing_begin/_end; ev_used counts events handed out.
+  std::vector<hipEvent_t> ev;
+  size_t ev_used = 0;
+  bool timing = false;
+  char err[512] = {0};
+};
+
+// Brackets the launches issued during its lifetime with one event pair when timing is armed.
+struct KernelTimer {
+  argus_hip_ctx *ctx;
+  hipStream_t stream;
+  bool on;
+  KernelTimer(argus_hip_ctx *c, hipStream_t s) : ctx(c), stream(s), on(false) {
+    if (c->timing && c->ev_used + 2 <= c->ev.size()) {
+      on = true;
+      (void)hipEventRecord(c->ev[c->ev_used], s);
+    }
+  }
+  ~KernelTimer() {
+    if (on) {
+      (void)hipEventRecord(ctx->ev[ctx->ev_used + 1], stream);
+      ctx->ev_used += 2;
+    }
+  }
+};
+
+inline int argus_fail(argus_hip_ctx *ctx, int code, const char *fmt, ...) {
+  if (ctx) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ctx->err, sizeof(ctx->err), fmt, ap);
+    va_end(ap);
+  }
+  return code;
+}
+
+#define ARGUS_HIP_CHECK(ctx, expr)                                                          \
+  do {                                                                                      \
+    hipError_t e_ = (expr);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      return argus_fail((ctx), ARGUS_HIP_ERR_RUNTIME, "%s: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+// Ensures the context workspace holds at least `bytes`; reallocation frees the old buffer
+// (hipFree synchronises the device, so no launch still reads it).
+int argus_ws_reserve(argus_hip_ctx *ctx, size_t bytes);
+
+#if defined(__HIPCC__)
+// ---- wave64 cross-lane helpers ------------------------------------------------------------
+// DPP moves stay inside a row of 16 lanes, which is all the 8/16-lane row groups need.
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+// All-reduce (sum) over aligned groups of LANES consecutive lanes; every lane gets the total.
+template <int LANES>
+__device__ __forceinline__ float group_allreduce_sum(float x) {
+  if constexpr (LANES >= 2) x += dpp_mov<0xB1>(x);   // quad_perm [1,0,3,2]
+  if constexpr (LANES >= 4) x += dpp_mov<0x4E>(x);   // quad_perm [2,3,0,1]
+  if constexpr (LANES >= 8) x += dpp_mov<0x141>(x);  // row_half_mirror
+  if constexpr (LANES >= 16) x += dpp_mov<0x140>(x); // row_mirror
+  if constexpr (LANES >= 32) x += __shfl_xor(x, 16, 64);
+  if constexpr (LANES >= 64) x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+template <int LANES>
+__device__ __forceinline__ float group_allreduce_max(float x) {
+  if constexpr (LANES >= 2) x = fmaxf(x, dpp_mov<0xB1>(x));
+  if constexpr (LANES >= 4) x = fmaxf(x, dpp_mov<0x4E>(x));
+  if constexpr (LANES >= 8) x = fmaxf(x, dpp_mov<0x141>(x));
+  if constexpr (LANES >= 16) x = fmaxf(x, dpp_mov<0x140>(x));
+  if constexpr (LANES >= 32) x = fmaxf(x, __shfl_xor(x, 16, 64));
+  if constexpr (LANES >= 64) x = fmaxf(x, __shfl_xor(x, 32, 64));
+  return x;
+}
+
+__device__ __forceinline__ float wave_allreduce_sum(float x) { return group_allreduce_sum<64>(x); }
+__device__ __forceinline__ float wave_allreduce_max(float x) { return group_allreduce_max<64>(x); }
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr float kNegInf = -__builtin_huge_valf();
+#endif

@@ -1,0 +1,428 @@
+// Split-KV flash-decode for single-query GQA attention on gfx950.
+//
+// Stands in for Backend::attention_gen (engine/src/backend.rs:284-295; CPU semantics
+// engine/src/backend/cpu/x86.rs:178-357 and common.rs:359-675).
+//
+// Design (HBM-bound: every K/V byte is read exactly once per call):
+//  * One workgroup (4 waves) owns one (sequence, KV head, KV split).  All Hq/Hkv query heads of
+//    the group share the single pass over K and V, so GQA does not multiply traffic.
+//  * A wave reads K/V rows with 16-byte loads; LPR = row_bytes/16 consecutive lanes cover one
+//    row, so each load instruction of a wave covers 64/LPR whole rows = 1 KiB of contiguous
+//    memory.  U such loads for K and U for V are in flight per wave before any use.
+//  * q.k partial sums are reduced over the LPR lanes with DPP adds (no LDS); afterwards every
+//    lane of a row group holds that row's logit, which is exactly the weight it needs for its
+//    slice of the V row.  Each row group keeps a private online-softmax state (m, l, acc) that is
+//    merged once at the end: shuffles across row groups, LDS across the 4 waves.
+//  * Each workgroup writes one partial (m, l, un-normalised out) per Q head; a second kernel
+//    combines the splits with a log-sum-exp merge, writes `out`, and -- when post-softmax scores
+//    were requested -- turns the logits the first pass stored in `scores_out` into probabilities
+//    in place (exact global max / sum are only known there).
+#include "argus_hip_internal.hpp"
+
+#include <algorithm>
+
+namespace {
+
+struct DecodeParams {
+  const float *q;
+  const void *k;
+  const void *v;
+  float *out;
+  float *scores;
+  const int32_t *kv_index;
+  float *ws_ml;  // [batch, Hq, nsplit, 2]
+  float *ws_o;   // [batch, Hq, nsplit, D]
+  int32_t n_heads_q, n_heads_kv, group;  // group = Hq / Hkv
+  int32_t len, kv_start, chunk, nsplit;
+  int32_t score_stride;
+  int64_t row_stride;   // elements between consecutive token rows of one KV head
+  int64_t head_stride;  // elements between KV heads
+  int64_t q_bs, out_bs, kv_bs, score_bs, index_bs;
+  float scale, softcap;
+  int32_t direct;  // nsplit == 1 and no scores: first pass writes `out` itself
+};
+
+template <typename KV_T>
+struct KvVec;
+template <>
+struct KvVec<_Float16> {
+  static constexpr int E = 8;
+  using vec = half8_t;
+};
+template <>
+struct KvVec<float> {
+  static constexpr int E = 4;
+  using vec = float4_t;
+};
+
+__device__ __forceinline__ float apply_softcap(float s, float cap) {
+  return cap > 0.0f ? cap * tanhf(s / cap) : s;
+}
+
+// Uniform-weights fallback of common.rs:561-577: out = mean of the attended V rows, every
+// probability 1/len.  Only reached when no logit is finite, so speed is irrelevant.
+template <typename KV_T>
+__device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
+  const int kvh = h / p.group;
+  const KV_T *vb = (const KV_T *)p.v + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;
+  const int32_t *idx = p.kv_index ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
+  const float u = 1.0f / (float)p.len;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) {
+    float acc = 0.0f;
+    for (int t = 0; t < p.len; ++t) {
+      const int64_t slot = idx ? idx[t] : (p.kv_start + t);
+      acc += u * (float)vb[slot * p.row_stride + c];
+    }
+    p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = acc;
+  }
+  if (p.scores) {
+    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
+    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = u;
+  }
+}
+
+template <int D, int GT, typename KV_T, int U>
+__global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p) {
+  constexpr int E = KvVec<KV_T>::E;
+  using vec_t = typename KvVec<KV_T>::vec;
+  constexpr int LPR = D / E;       // lanes per K/V row
+  constexpr int RPW = 64 / LPR;    // rows per wave load instruction
+  constexpr int TILE = RPW * U;    // rows per wave iteration
+  static_assert(LPR >= GT && LPR <= 64, "row group must cover the query-head tile");
+
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = lane / LPR, sub = lane % LPR;
+  const int c0 = sub * E;
+
+  const int t_begin = split * p.chunk;
+  const int t_end = min(p.len, t_begin + p.chunk);
+
+  const KV_T *kb = (const KV_T *)p.k + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride + c0;
+  const KV_T *vb = (const KV_T *)p.v + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride + c0;
+  const int32_t *idx = p.kv_index ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
+
+  // This lane's slice of every query head of the group (heads beyond the group are clamped
+  // duplicates whose results are never written).
+  float q[GT][E];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    const int h = kvh * p.group + min(g, p.group - 1);
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)h * D + c0;
+#pragma unroll
+    for (int e = 0; e < E; ++e) q[g][e] = qp[e] * p.scale;
+  }
+
+  float m[GT], l[GT], acc[GT][E];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    m[g] = kNegInf;
+    l[g] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[g][e] = 0.0f;
+  }
+
+  for (int base = t_begin + wave * TILE; base < t_end; base += 4 * TILE) {
+    vec_t kr[U], vr[U];
+    bool valid[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = base + u * RPW + grp;
+      valid[u] = t < t_end;
+      const int tc = valid[u] ? t : (t_end - 1);
+      const int64_t slot = idx ? (int64_t)idx[tc] : (int64_t)(p.kv_start + tc);
+      kr[u] = *(const vec_t *)(kb + slot * p.row_stride);
+      vr[u] = *(const vec_t *)(vb + slot * p.row_stride);
+    }
+
+    float s[U][GT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int g = 0; g < GT; ++g) {
+        float part = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) part = fmaf(q[g][e], (float)kr[u][e], part);
+        float sv = group_allreduce_sum<LPR>(part);
+        sv = apply_softcap(sv, p.softcap);
+        sv = (sv != sv) ? kNegInf : sv;  // NaN logit counts as -inf (common.rs:555-560)
+        s[u][g] = valid[u] ? sv : kNegInf;
+      }
+    }
+
+    if (p.scores) {
+      // Store the logits; the combine pass rewrites them as probabilities.
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = base + u * RPW + grp;
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          if (sub == g && g < p.group && valid[u])
+            p.scores[(int64_t)b * p.score_bs + (int64_t)(kvh * p.group + g) * p.score_stride + t] = s[u][g];
+        }
+      }
+    }
+
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      float mt = s[0][g];
+#pragma unroll
+      for (int u = 1; u < U; ++u) mt = fmaxf(mt, s[u][g]);
+      const float m_new = fmaxf(m[g], mt);
+      const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+      const float alpha = __expf(m[g] - m_ref);
+      m[g] = m_new;
+      float lsum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[g][e] *= alpha;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float pw = __expf(s[u][g] - m_ref);
+        lsum += pw;
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[g][e] = fmaf(pw, (float)vr[u][e], acc[g][e]);
+      }
+      l[g] = l[g] * alpha + lsum;
+    }
+  }
+
+  // ---- merge the RPW row groups of this wave --------------------------------------------
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    float mw = m[g];
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
+    const float m_ref = (mw == kNegInf) ? 0.0f : mw;
+    const float f = __expf(m[g] - m_ref);
+    float lw = l[g] * f;
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) lw += __shfl_xor(lw, off, 64);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      float a = acc[g][e] * f;
+#pragma unroll
+      for (int off = LPR; off < 64; off <<= 1) a += __shfl_xor(a, off, 64);
+      acc[g][e] = a;
+    }
+    m[g] = mw;
+    l[g] = lw;
+  }
+
+  // ---- merge the 4 waves through LDS ------------------------------------------------------
+  __shared__ float lds_m[4][GT], lds_l[4][GT];
+  __shared__ float lds_acc[4][GT][D];
+  if (grp == 0) {
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      if (sub == 0) {
+        lds_m[wave][g] = m[g];
+        lds_l[wave][g] = l[g];
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) lds_acc[wave][g][c0 + e] = acc[g][e];
+    }
+  }
+  __syncthreads();
+
+  for (int i = threadIdx.x; i < p.group * D; i += 256) {
+    const int g = i / D, c = i % D;
+    const int h = kvh * p.group + g;
+    float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
+    const float m_ref = (mm == kNegInf) ? 0.0f : mm;
+    float o = 0.0f, ll = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = __expf(lds_m[w][g] - m_ref);
+      o += lds_acc[w][g][c] * f;
+      ll += lds_l[w][g] * f;
+    }
+    if (p.direct) {
+      // Single split, no scores: finish here.  A row without any finite logit is left to the
+      // fallback below.
+      if (ll > 0.0f && ll < __builtin_huge_valf()) p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = o / ll;
+    } else {
+      const int64_t pidx = ((int64_t)b * p.n_heads_q + h) * p.nsplit + split;
+      p.ws_o[pidx * D + c] = o;
+      if (c == 0) {
+        p.ws_ml[pidx * 2 + 0] = mm;
+        p.ws_ml[pidx * 2 + 1] = ll;
+      }
+    }
+  }
+  if (p.direct) {
+    for (int g = 0; g < p.group; ++g) {
+      const float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
+      const float m_ref = (mm == kNegInf) ? 0.0f : mm;
+      float ll = 0.0f;
+      for (int w = 0; w < 4; ++w) ll += lds_l[w][g] * __expf(lds_m[w][g] - m_ref);
+      if (!(ll > 0.0f && ll < __builtin_huge_valf())) uniform_fallback<KV_T>(p, b, kvh * p.group + g, D);
+    }
+  }
+}
+
+// Second pass: log-sum-exp merge of the splits of one (sequence, Q head); optional in-place
+// logits -> probabilities rewrite of the score row.
+template <typename KV_T>
+__global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams p, int D) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int64_t pbase = ((int64_t)b * p.n_heads_q + h) * p.nsplit;
+  __shared__ float sh_m, sh_l;
+  if (threadIdx.x < 64) {
+    float mm = kNegInf;
+    for (int s = threadIdx.x; s < p.nsplit; s += 64) mm = fmaxf(mm, p.ws_ml[(pbase + s) * 2]);
+    mm = wave_allreduce_max(mm);
+    const float m_ref = (mm == kNegInf) ? 0.0f : mm;
+    float ll = 0.0f;
+    for (int s = threadIdx.x; s < p.nsplit; s += 64)
+      ll += p.ws_ml[(pbase + s) * 2 + 1] * __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
+    ll = wave_allreduce_sum(ll);
+    if (threadIdx.x == 0) {
+      sh_m = mm;
+      sh_l = ll;
+    }
+  }
+  __syncthreads();
+  const float mm = sh_m, ll = sh_l;
+  if (!(ll > 0.0f && ll < __builtin_huge_valf())) {
+    uniform_fallback<KV_T>(p, b, h, D);
+    return;
+  }
+  const float m_ref = mm;
+  const float inv = 1.0f / ll;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    float o = 0.0f;
+    for (int s = 0; s < p.nsplit; ++s)
+      o += p.ws_o[(pbase + s) * D + c] * __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
+    p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = o * inv;
+  }
+  if (p.scores) {
+    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
+    for (int t = threadIdx.x; t < p.len; t += 256) srow[t] = __expf(srow[t] - m_ref) * inv;
+  }
+}
+
+template <int D, int GT, typename KV_T>
+constexpr int unroll_for() {
+  // Keep q + acc + in-flight K/V rows inside the register file at >= 2 waves per SIMD.
+  return GT >= 8 ? 2 : (GT >= 4 ? 4 : 8);
+}
+
+template <int D, int GT, typename KV_T>
+int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scores, hipStream_t stream) {
+  constexpr int U = unroll_for<D, GT, KV_T>();
+  constexpr int E = KvVec<KV_T>::E;
+  constexpr int tile_rows = 4 * (64 / (D / E)) * U;  // rows one workgroup consumes per iteration
+
+  const int pairs = batch * p.n_heads_kv;
+  const int target_wgs = ctx->compute_units * 4;
+  const int max_splits = (p.len + tile_rows - 1) / tile_rows;
+  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, 512}));
+  int chunk = (p.len + nsplit - 1) / nsplit;
+  chunk = (chunk + tile_rows - 1) / tile_rows * tile_rows;
+  nsplit = (p.len + chunk - 1) / chunk;
+  p.chunk = chunk;
+  p.nsplit = nsplit;
+  p.direct = (nsplit == 1 && !want_scores) ? 1 : 0;
+
+  if (!p.direct) {
+    const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
+    const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
+    int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+    if (rc != ARGUS_HIP_OK) return rc;
+    p.ws_ml = ctx->ws;
+    p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
+  }
+
+  dim3 grid(nsplit, p.n_heads_kv, batch);
+  {
+    KernelTimer timer(ctx, stream);
+    hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U>), grid, dim3(256), 0, stream, p);
+  }
+  ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  if (!p.direct) {
+    hipLaunchKernelGGL((decode_combine_kernel<KV_T>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p, D);
+    ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  }
+  return ARGUS_HIP_OK;
+}
+
+template <int D, typename KV_T>
+int dispatch_group(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scores, hipStream_t stream) {
+  if (p.group <= 1) return launch_decode<D, 1, KV_T>(ctx, p, batch, want_scores, stream);
+  if (p.group <= 2) return launch_decode<D, 2, KV_T>(ctx, p, batch, want_scores, stream);
+  if (p.group <= 4) return launch_decode<D, 4, KV_T>(ctx, p, batch, want_scores, stream);
+  if (p.group <= 8) return launch_decode<D, 8, KV_T>(ctx, p, batch, want_scores, stream);
+  return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "GQA group %d > 8 not supported", p.group);
+}
+
+template <typename KV_T>
+int dispatch_dim(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, bool want_scores, hipStream_t stream) {
+  switch (D) {
+    case 64: return dispatch_group<64, KV_T>(ctx, p, batch, want_scores, stream);
+    case 128: return dispatch_group<128, KV_T>(ctx, p, batch, want_scores, stream);
+    case 256: return dispatch_group<256, KV_T>(ctx, p, batch, want_scores, stream);
+    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "head_dim %d not in {64,128,256}", D);
+  }
+}
+
+}  // namespace
+
+ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *a) {
+  if (!ctx || !a) return ARGUS_HIP_ERR_INVALID;
+  if (!a->q || !a->k_cache || !a->v_cache || !a->out)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: null tensor pointer");
+  if (a->num_heads_q <= 0 || a->num_heads_kv <= 0 || a->num_heads_q % a->num_heads_kv)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: heads %d/%d", a->num_heads_q, a->num_heads_kv);
+  if (a->cache_seq_len <= 0 || a->batch <= 0 || a->kv_start < 0)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: cache_seq_len %d batch %d kv_start %d",
+                      a->cache_seq_len, a->batch, a->kv_start);
+  if (a->layout != ARGUS_HIP_HEAD_MAJOR && a->layout != ARGUS_HIP_SEQ_MAJOR)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: layout %d", a->layout);
+  if (a->layout == ARGUS_HIP_HEAD_MAJOR && !a->kv_index && a->kv_start + a->cache_seq_len > a->capacity)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: kv_start %d + len %d exceeds capacity %d",
+                      a->kv_start, a->cache_seq_len, a->capacity);
+  if (a->scores_out && a->score_stride < a->cache_seq_len)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: score_stride %d < cache_seq_len %d",
+                      a->score_stride, a->cache_seq_len);
+  if (a->batch > 65535 || a->num_heads_kv > 65535)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: batch / kv heads beyond grid limits");
+
+  const int D = a->head_dim;
+  DecodeParams p{};
+  p.q = a->q;
+  p.k = a->k_cache;
+  p.v = a->v_cache;
+  p.out = a->out;
+  p.scores = a->scores_out;
+  p.kv_index = a->kv_index;
+  p.n_heads_q = a->num_heads_q;
+  p.n_heads_kv = a->num_heads_kv;
+  p.group = a->num_heads_q / a->num_heads_kv;
+  p.len = a->cache_seq_len;
+  p.kv_start = a->kv_index ? 0 : a->kv_start;
+  p.score_stride = a->score_stride;
+  if (a->layout == ARGUS_HIP_HEAD_MAJOR) {
+    p.row_stride = D;
+    p.head_stride = (int64_t)a->capacity * D;
+  } else {
+    p.row_stride = (int64_t)a->num_heads_kv * D;
+    p.head_stride = D;
+  }
+  p.q_bs = a->q_batch_stride ? a->q_batch_stride : (int64_t)a->num_heads_q * D;
+  p.out_bs = a->out_batch_stride ? a->out_batch_stride : (int64_t)a->num_heads_q * D;
+  p.kv_bs = a->kv_batch_stride;
+  p.score_bs = a->score_batch_stride ? a->score_batch_stride : (int64_t)a->num_heads_q * a->score_stride;
+  p.index_bs = a->index_batch_stride;
+  p.scale = a->scale != 0.0f ? a->scale : 1.0f / sqrtf((float)D);
+  p.softcap = a->softcap;
+  if (a->batch > 1 && p.kv_bs == 0)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: batch > 1 needs kv_batch_stride");
+
+  hipStream_t stream = (hipStream_t)a->stream;
+  const bool want_scores = a->scores_out != nullptr;
+  switch (a->kv_dtype) {
+    case ARGUS_HIP_F16: return dispatch_dim<_Float16>(ctx, p, D, a->batch, want_scores, stream);
+    case ARGUS_HIP_F32: return dispatch_dim<float>(ctx, p, D, a->batch, want_scores, stream);
+    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: kv dtype %d", a->kv_dtype);
+  }
+}

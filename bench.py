@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X attention hot path (one GPU).
+
+Primary line (the metric BASELINE.json names): split-KV decode attention, Llama-3.1-8B head
+shape (32 query heads, 8 KV heads, head_dim 128), F16 KV cache, KV length 32768, batch 16
+independent sequences -- 2 GiB of KV per step, far beyond the 256 MB Infinity Cache, so the
+rate is an HBM rate.  A "step" is one attention call over the whole batch with Q/K/V already
+resident in HBM.  `value` is algorithmic bytes / wall time of the timed region.
+
+`roofline` is computed from the dominant kernel's own duration (HIP events recorded by the
+library on the launch stream around the split-KV kernel of every timed step).
+`cpu_baseline` times the restated reference CPU backend (AVX2+FMA+F16C, one task per Q head) on
+a bounded sample (one of the 16 sequences) on the host cores of the same box.
+`extras` reports the other BASELINE configurations with the same accounting.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "argus-engine_amd"), os.path.join(ROOT, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16 MFMA
+
+
+def decode_bytes(hq, hkv, d, L, batch, kv_elem_bytes=2, scores=False):
+    """Algorithmic bytes of one decode call: K+V over the valid length, Q in, out (+ scores)."""
+    per_seq = 2 * hkv * L * d * kv_elem_bytes + hq * d * 4 * 2
+    if scores:
+        per_seq += hq * L * 4
+    return per_seq * batch
+
+
+def time_region(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores=False, softcap=0.0,
+                 rotate=1, seed=137):
+    """Returns dict(ms_per_step, kernel_ms, bytes).  `rotate` distinct KV buffers are cycled so a
+    cache smaller than the rotation set cannot serve repeated reads."""
+    import torch
+    cap = capacity or L
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    ks, vs = [], []
+    for _ in range(rotate):
+        ks.append(torch.randn((batch, hkv, cap, d), generator=g, device="cuda", dtype=torch.float32).half())
+        vs.append(torch.randn((batch, hkv, cap, d), generator=g, device="cuda", dtype=torch.float32).half())
+    q = torch.randn((batch, hq, d), generator=g, device="cuda", dtype=torch.float32)
+    out = torch.empty((batch, hq, d), device="cuda", dtype=torch.float32)
+    sc = torch.empty((batch, hq, cap), device="cuda", dtype=torch.float32) if scores else None
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] % rotate
+        state["i"] += 1
+        ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, cap, scores=sc, score_stride=cap if scores else 0,
+                          batch=batch, kv_batch_stride=hkv * cap * d, softcap=softcap)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ctx.kernel_timing_begin(steps)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    kms = ctx.kernel_timing_end(steps)
+    nbytes = decode_bytes(hq, hkv, d, L, batch, 2, scores)
+    kernel_ms = sum(kms) / max(len(kms), 1)
+    return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes,
+                gbps_wall=nbytes / wall / 1e9, gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None)
+
+
+def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
+    """Restated CpuBackendAVX2::attention_gen on one sequence of the primary workload."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(137)
+    q = rng.standard_normal((hq, d), dtype=np.float32)
+    k = rng.standard_normal((hkv, L, d), dtype=np.float32).astype(np.float16)
+    v = rng.standard_normal((hkv, L, d), dtype=np.float32).astype(np.float16)
+    cores = min(hq, int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1), 16)
+    oracle.attention_gen(q, k, v, hkv, L, L, impl="avx2", n_threads=cores)  # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 20 or (time.perf_counter() - t_start < budget_s and len(times) < 400):
+        t0 = time.perf_counter()
+        oracle.attention_gen(q, k, v, hkv, L, L, impl="avx2", n_threads=cores)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > 2.5 * budget_s:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    nbytes = decode_bytes(hq, hkv, d, L, 1)
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "1 of the 16 sequences (Hq32 Hkv8 d128 L32768 F16 KV), median of %d calls, %.1f us/call; "
+                      "restated CpuBackendAVX2::attention_gen, one task per Q head" % (len(times), med * 1e6)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (every box has one GPU; the path shards by "
+              "sequence / KV head without exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import argus_hip
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    ctx = argus_hip.Context(0)
+    info = ctx.device_info()
+
+    hq, hkv, d, L, batch = 32, 8, 128, 32768, 16
+    r = bench_decode(ctx, hq, hkv, d, L, batch, args.steps, args.warmup)
+    line = {
+        "metric": "decode_attn_hbm_gbps_32k_kv",
+        "value": round(r["gbps_wall"], 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(r["ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 3: split-KV decode attention, Llama-3.1-8B shape "
+                               "(Hq32 Hkv8 d128), F16 KV, KV length 32768, batch 16, seeded N(0,1)",
+                   "kv_dtype": "f16", "accumulate": "f32", "batch": batch, "kv_len": L,
+                   "us_per_call": round(r["ms_per_step"] * 1e3, 2),
+                   "tokens_per_s": round(batch / (r["ms_per_step"] * 1e-3), 1)},
+        "roofline": {"bound": "hbm", "achieved": round(r["gbps_kernel"], 2), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(r["gbps_kernel"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "decode_split_kernel<128,4,f16>", "kernel_ms": round(r["kernel_ms"], 5),
+                     "algorithmic_bytes": r["bytes"]},
+        "device": {"name": info.name.decode(), "arch": info.gcn_arch.decode(), "cus": info.compute_units,
+                   "clock_mhz": info.clock_mhz},
+    }
+
+    if not args.no_extras:
+        ex = {}
+        es, ew = max(20, args.steps), max(3, args.warmup)
+
+        def add(name, res, note=""):
+            ex[name] = {"us_per_call": round(res["ms_per_step"] * 1e3, 2),
+                        "kernel_us": round(res["kernel_ms"] * 1e3, 2),
+                        "gbps_kernel": round(res["gbps_kernel"], 1),
+                        "hbm_frac_kernel": round(res["gbps_kernel"] / HBM_PEAK_GBPS, 4),
+                        "bytes": res["bytes"], "note": note}
+
+        add("cfg3_L32768_b1", bench_decode(ctx, 32, 8, 128, 32768, 1, es, ew, rotate=4),
+            "4 KV buffer sets rotated (512 MiB > Infinity Cache)")
+        add("cfg3_L4096_b16", bench_decode(ctx, 32, 8, 128, 4096, 16, es, ew, rotate=2), "2 sets rotated")
+        add("cfg3_L4096_b1", bench_decode(ctx, 32, 8, 128, 4096, 1, es, ew, rotate=16), "16 sets rotated")
+        add("cfg1_qwen_L1024_b1", bench_decode(ctx, 14, 2, 64, 1024, 1, es, ew), "latency-bound (0.5 MiB)")
+        add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
+            bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=4),
+            "scores emitted; kernel time covers the split pass only")
+        line["extras"] = ex
+
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_decode(hq, hkv, d, L)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,277 @@
+/*
+ * argus_hip.h -- C ABI of the MI355X (gfx950) attention backend for the Argus engine.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers / integers, returns an
+ * `int` (0 = ok, negative = error, never throws or aborts: the engine's release
+ * profile is panic=abort, crates/argus-extension-api/src/lib.rs:1680) and runs on
+ * the single in-order stream the engine lends (NULL = the default stream,
+ * engine/src/kv/quant_window_cuda.rs:38-46).  The engine owns every Q / KV / out /
+ * score buffer and lends raw device pointers for the duration of one call; the
+ * library never frees or retains them (crates/argus-extension-api/src/lib.rs:1593).
+ *
+ * Each declaration cites the reference interface it stands in for; paths are
+ * relative to the reference repository root.
+ */
+#ifndef ARGUS_HIP_H
+#define ARGUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARGUS_HIP_ABI_VERSION 1
+
+/* Return codes. */
+#define ARGUS_HIP_OK 0
+#define ARGUS_HIP_ERR_INVALID (-1)     /* bad argument (null pointer, non-dividing heads, ...) */
+#define ARGUS_HIP_ERR_UNSUPPORTED (-2) /* shape / dtype outside the kernels' coverage */
+#define ARGUS_HIP_ERR_RUNTIME (-3)     /* HIP runtime error; see argus_hip_last_error */
+#define ARGUS_HIP_ERR_NOMEM (-4)       /* workspace allocation failed */
+
+/* DType subset of engine/src/buffer.rs:25-47 that the attention path touches. */
+#define ARGUS_HIP_F32 0
+#define ARGUS_HIP_F16 1
+
+/* KVLayout, engine/src/kv/kv_cache_ops.rs:18-21. */
+#define ARGUS_HIP_HEAD_MAJOR 0 /* [batch, kv_heads, capacity, head_dim] */
+#define ARGUS_HIP_SEQ_MAJOR 1  /* [batch, seq, kv_heads, head_dim]     */
+
+typedef struct argus_hip_ctx argus_hip_ctx;
+
+/* ---- context: what `HipBackend::new` / `Drop` bind -------------------------------------- */
+/* Counterpart of CudaBackend construction in engine/src/session/init.rs:351-428: selects the
+ * device, reads its CU count and allocates the split-KV partial workspace.  Fails with
+ * ARGUS_HIP_ERR_RUNTIME (and *out = NULL) when no HIP device is present. */
+int argus_hip_create(int device, argus_hip_ctx **out);
+int argus_hip_destroy(argus_hip_ctx *ctx);
+int argus_hip_abi_version(void);
+/* Last error text of this context (single inference thread, like the reference backends). */
+const char *argus_hip_last_error(const argus_hip_ctx *ctx);
+
+typedef struct argus_hip_device_info {
+  int32_t compute_units;
+  int32_t clock_mhz;
+  int32_t wavefront_size;
+  int32_t lds_bytes_per_block;
+  int64_t hbm_bytes;
+  char name[128];
+  char gcn_arch[64];
+} argus_hip_device_info;
+int argus_hip_get_device_info(const argus_hip_ctx *ctx, argus_hip_device_info *info);
+
+/* ---- per-kernel event timing ------------------------------------------------------------- */
+/* Counterpart of the event-based GPU profiling switch Backend::profile_events_enabled /
+ * set_op_label (engine/src/backend.rs:1296-1306).  Between _begin and _end the dominant kernel
+ * of every attention call (decode split pass, prefill, KIVI decode) is bracketed by a HIP event
+ * pair recorded on the stream it is launched on; _end waits for the last one and returns the
+ * per-launch durations in milliseconds (at most `capacity`; *n_out = launches recorded). */
+int argus_hip_kernel_timing_begin(argus_hip_ctx *ctx, int32_t max_launches);
+int argus_hip_kernel_timing_end(argus_hip_ctx *ctx, float *ms_out, int32_t capacity, int32_t *n_out);
+
+/* ---- memory helpers for the Rust `Memory` / `Buffer` impls ------------------------------- */
+/* Backend::{read_buffer, write_buffer, write_buffer_range, copy_slice, buffer_shift,
+ * synchronize}: engine/src/backend.rs:610, 710, 736, 1085, 1119, 762. */
+int argus_hip_malloc(argus_hip_ctx *ctx, size_t bytes, void **dev_ptr);
+int argus_hip_free(argus_hip_ctx *ctx, void *dev_ptr);
+int argus_hip_write_buffer(argus_hip_ctx *ctx, void *stream, void *dst_dev, const void *src_host, size_t bytes);
+int argus_hip_read_buffer(argus_hip_ctx *ctx, void *stream, void *dst_host, const void *src_dev, size_t bytes);
+int argus_hip_copy_slice(argus_hip_ctx *ctx, void *stream, void *dst_dev, const void *src_dev, size_t bytes);
+int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream);
+
+/* ---- (a-1) single-query GQA decode attention ---------------------------------------------- */
+/* Backend::attention_gen, engine/src/backend.rs:284-295 (CPU: backend/cpu/x86.rs:178-357,
+ * backend/cpu/common.rs:359-675; CUDA host: backend/cuda_pc.rs:1693-1885).
+ *   s_t = (q . k_t) * scale;  [soft-cap];  p = softmax_t(s);  out = sum_t p_t v_t
+ * Layout rule of x86.rs:195-198: HeadMajor offset (kv_h*capacity + t)*d, SeqMajor
+ * (t*Hkv + kv_h)*d.  `scores_out[h*score_stride + t] = p_t` like x86.rs:302-310, but the
+ * pointer is a DEVICE pointer here (the host-slice contract of the trait, with its
+ * synchronize + copy-back, lives in the host mirror `HipBackend::attention_gen`).
+ * NaN logits count as -inf and an all -inf row falls back to uniform weights, as in
+ * common.rs:555-584.
+ * Beyond the reference trait (all default to the reference behaviour when zero / NULL):
+ *   batch / *_batch_stride : `batch` independent sequences in one launch (the reference
+ *                            loops, engine/src/backend.rs:277-295);
+ *   kv_start               : first attended slot (windowed layers pass cache_len - window);
+ *   kv_index               : logical token t lives in slot kv_index[t]
+ *                            (SelectiveRead gather, engine/src/kv/standard_format.rs:2052-2184);
+ *   softcap                : cap*tanh(s/cap) after scaling
+ *                            (engine/kernels/flash_attn_f32_f16.cl:563-565; host passes 0);
+ *   scale                  : 0 selects 1/sqrt(head_dim) (x86.rs:192). */
+typedef struct argus_hip_attention_gen_args {
+  void *stream;
+  const float *q;       /* [batch, num_heads_q, head_dim] F32 */
+  const void *k_cache;  /* F16 or F32, layout per `layout` */
+  const void *v_cache;
+  float *out;           /* [batch, num_heads_q, head_dim] F32 */
+  float *scores_out;    /* device, [batch, num_heads_q, score_stride] F32, or NULL */
+  const int32_t *kv_index; /* device, [cache_seq_len] (per sequence if index_batch_stride != 0), or NULL */
+  int32_t num_heads_q;
+  int32_t num_heads_kv;
+  int32_t head_dim;      /* 64, 128 or 256 */
+  int32_t cache_seq_len; /* valid tokens attended */
+  int32_t capacity;      /* HeadMajor rows per head; ignored for SeqMajor */
+  int32_t kv_start;
+  int32_t layout;        /* ARGUS_HIP_HEAD_MAJOR / ARGUS_HIP_SEQ_MAJOR */
+  int32_t kv_dtype;      /* ARGUS_HIP_F16 / ARGUS_HIP_F32 */
+  int32_t batch;         /* >= 1 */
+  int32_t score_stride;  /* floats per head row of scores_out, >= cache_seq_len */
+  int64_t q_batch_stride;     /* elements; 0 = num_heads_q*head_dim */
+  int64_t out_batch_stride;   /* elements; 0 = num_heads_q*head_dim */
+  int64_t kv_batch_stride;    /* elements between consecutive sequences' caches */
+  int64_t score_batch_stride; /* elements; 0 = num_heads_q*score_stride */
+  int64_t index_batch_stride; /* elements; 0 = one index list shared by the batch */
+  float softcap;
+  float scale;
+} argus_hip_attention_gen_args;
+int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args);
+
+/* ---- (a-2) causal GQA flash-attention prefill ---------------------------------------------- */
+/* Backend::flash_attention_prefill, engine/src/backend.rs:1011-1027 (CUDA host
+ * backend/cuda_pc.rs:830-926, CPU layers/attention.rs:78-351).  Key c is visible to query
+ * row r iff c <= r + q_start_pos (and c + window > r + q_start_pos when window > 0), with
+ * q_start_pos = cache_seq_len - seq_len; fully masked rows give zeros.
+ * Returns 1 when dispatched (trait: Ok(true)), 0 when declined so the caller runs its CPU
+ * path (Ok(false): SeqMajor, head_dim outside {64,128,256}, unsupported dtype -- the same
+ * cases cuda_pc.rs:851-860 declines), negative on error.
+ * Q/out [batch, seq_len, n_heads_q, head_dim], K/V HeadMajor [batch, n_heads_kv, capacity,
+ * head_dim].  The reference shape is F32 Q/out with F16 KV; F16 Q/out is the all-f16 form. */
+typedef struct argus_hip_prefill_args {
+  void *stream;
+  const void *q;
+  const void *k_cache;
+  const void *v_cache;
+  void *out;
+  int32_t n_heads_q;
+  int32_t n_heads_kv;
+  int32_t seq_len;
+  int32_t cache_seq_len;
+  int32_t head_dim;
+  int32_t kv_capacity;
+  int32_t batch_size;
+  int32_t is_head_major;
+  int32_t q_dtype;   /* ARGUS_HIP_F32 / ARGUS_HIP_F16 */
+  int32_t kv_dtype;  /* ARGUS_HIP_F16 / ARGUS_HIP_F32 */
+  int32_t out_dtype; /* ARGUS_HIP_F32 / ARGUS_HIP_F16 */
+  int32_t window;    /* 0 = none */
+} argus_hip_prefill_args;
+int argus_hip_flash_attention_prefill(argus_hip_ctx *ctx, const argus_hip_prefill_args *args);
+
+/* ---- (a-3) KIVI fused dequant + decode attention ------------------------------------------- */
+/* Field-for-field twin of CudaQuantAttnArgs, crates/argus-extension-api/src/lib.rs:3000-3026,
+ * so the Rust side is a cast.  `scores_out` is a HOST pointer filled by a blocking copy, as in
+ * crates/techniques/kivi/src/gpu_kivi_cuda.rs:204-212.  Block layouts and index math:
+ * crates/techniques/kivi/src/kivi_attn.cu:71-82, 256-262 (K per channel), 173-177, 357-361
+ * (V per token); codec crates/argus-kv-codec/src/lib.rs:26-203. */
+typedef struct argus_hip_quant_attn_args {
+  void *stream;
+  uint64_t q_mem;     /* [num_heads_q, head_dim] F32 */
+  uint64_t qk_mem;    /* quantised key blocks, per channel, flush-interleaved */
+  uint64_t qv_mem;    /* quantised value blocks, per token, flush-interleaved */
+  uint64_t res_k_mem; /* residual keys [kv_heads, res_cap, head_dim] */
+  uint64_t res_v_mem;
+  uint64_t out_mem;   /* [num_heads_q, head_dim] F32 */
+  float *scores_out;  /* host, may be NULL */
+  size_t scores_len;
+  size_t num_heads_q;
+  size_t num_heads_kv;
+  size_t head_dim;
+  size_t q_tokens;
+  size_t res_tokens;
+  size_t res_cap;
+  float scale;
+  uint8_t bits; /* 2, 4 or 8 */
+} argus_hip_quant_attn_args;
+
+/* Optional extras that have no field in the reference POD. */
+typedef struct argus_hip_quant_attn_ext {
+  uint64_t scores_dev;   /* device score buffer [num_heads_q, score_stride]; 0 = none */
+  size_t score_stride;
+  int32_t res_dtype;     /* ARGUS_HIP_F32 (reference, engine/src/kv/quant_window_cache.rs:171-177) or ARGUS_HIP_F16 */
+  float softcap;
+} argus_hip_quant_attn_ext;
+
+/* CudaQuantAttnBackend::{has_quant_attn_kernel, attention_gen_quant, gather_update_quant},
+ * crates/argus-extension-api/src/lib.rs:3087-3104. */
+int argus_hip_has_quant_attn_kernel(const argus_hip_ctx *ctx, uint8_t bits);
+int argus_hip_attention_gen_quant(argus_hip_ctx *ctx, const argus_hip_quant_attn_args *args);
+int argus_hip_attention_gen_quant_ex(argus_hip_ctx *ctx, const argus_hip_quant_attn_args *args,
+                                     const argus_hip_quant_attn_ext *ext);
+
+/* Twin of CudaQuantAttnGatherArgs, crates/argus-extension-api/src/lib.rs:3031-3046; kernel
+ * semantics crates/techniques/kivi/src/kivi_q2.cu:117-138 (residual ring append). */
+typedef struct argus_hip_quant_gather_args {
+  void *stream;
+  uint64_t input_mem;    /* [seq_len, kv_heads, head_dim] F32 */
+  uint64_t residual_mem; /* [kv_heads, res_cap, head_dim] F32, written */
+  size_t kv_heads;
+  size_t res_cap;
+  size_t head_dim;
+  size_t seq_len;
+  size_t res_pos;
+} argus_hip_quant_gather_args;
+int argus_hip_gather_update_quant(argus_hip_ctx *ctx, const argus_hip_quant_gather_args *args);
+
+/* On-device quantise-at-flush: the CPU loop of QuantizedRecentWindowCache::flush_residual,
+ * engine/src/kv/quant_window_cache.rs:919-946, producing bit-identical blocks appended at
+ * block offsets k_block_start / v_block_start (the reference quantises on the CPU even in GPU
+ * mode, quant_window_cache.rs:1700-1722). */
+typedef struct argus_hip_quant_flush_args {
+  void *stream;
+  uint64_t res_k_mem; /* [kv_heads, res_cap, head_dim] F32 */
+  uint64_t res_v_mem;
+  uint64_t qk_mem;    /* destination block stream */
+  uint64_t qv_mem;
+  size_t kv_heads;
+  size_t res_cap;
+  size_t head_dim;
+  size_t flush_tokens; /* multiple of 32, <= res_cap */
+  size_t k_block_start;
+  size_t v_block_start;
+  uint8_t bits;
+} argus_hip_quant_flush_args;
+int argus_hip_quant_flush(argus_hip_ctx *ctx, const argus_hip_quant_flush_args *args);
+
+/* ---- (a-4) attention-score reduce for H2O / D2O --------------------------------------------- */
+/* Field-for-field twin of CudaScoreReduceArgs, crates/argus-extension-api/src/lib.rs:2909-2933;
+ * CudaScoreReduceBackend::{reduce, reduce_per_layer} 2938-2948; kernel semantics
+ * crates/techniques/attn-score/src/score_reduce.cu:13-62, 64-91. */
+typedef struct argus_hip_score_reduce_args {
+  void *stream;
+  uint64_t score_buf;       /* [n_layers, n_heads_q, score_stride] F32 */
+  uint64_t importance;      /* [max_seq_len] F32, in place */
+  uint64_t head_importance; /* [n_kv_heads * max_seq_len] F32, in place */
+  float decay_factor;
+  size_t n_layers;
+  size_t n_heads_q;
+  size_t n_kv_heads; /* <= 16 */
+  size_t cache_seq_len;
+  size_t score_stride;
+  size_t max_seq_len;
+  uint64_t layer_flat_importance; /* [n_layers * max_seq_len] or 0 */
+} argus_hip_score_reduce_args;
+int argus_hip_score_reduce(argus_hip_ctx *ctx, const argus_hip_score_reduce_args *args);
+int argus_hip_score_reduce_per_layer(argus_hip_ctx *ctx, const argus_hip_score_reduce_args *args);
+
+/* ---- (f-1) KV write path ---------------------------------------------------------------------- */
+/* Backend::kv_scatter_f32_to_f16 / _batch / _f32_batch, engine/src/backend.rs:425-545; device
+ * semantics engine/src/backend/cuda_pc/kernels.cu:305-360.  src [seq_len, kv_heads, head_dim]
+ * F32 -> dst HeadMajor [kv_heads, capacity, head_dim] at rows write_pos_start + s. */
+int argus_hip_kv_scatter_f32_to_f16(argus_hip_ctx *ctx, void *stream, const float *k_src,
+                                    const float *v_src, void *k_dst, void *v_dst, int32_t kv_heads,
+                                    int32_t head_dim, int32_t capacity, int32_t write_pos);
+int argus_hip_kv_scatter_f32_to_f16_batch(argus_hip_ctx *ctx, void *stream, const float *k_src,
+                                          const float *v_src, void *k_dst, void *v_dst,
+                                          int32_t kv_heads, int32_t head_dim, int32_t capacity,
+                                          int32_t write_pos_start, int32_t seq_len);
+int argus_hip_kv_scatter_f32_batch(argus_hip_ctx *ctx, void *stream, const float *k_src,
+                                   const float *v_src, float *k_dst, float *v_dst, int32_t kv_heads,
+                                   int32_t head_dim, int32_t capacity, int32_t write_pos_start,
+                                   int32_t seq_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARGUS_HIP_H */

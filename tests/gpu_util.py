@@ -1,0 +1,50 @@
+"""Shared helpers for the GPU parity tests: one context per session, numpy <-> device moves."""
+import numpy as np
+import pytest
+
+_ctx = None
+
+
+def ctx():
+    """The process-wide argus_hip context (created on first use; needs a GPU)."""
+    global _ctx
+    if _ctx is None:
+        import argus_hip
+        _ctx = argus_hip.Context(0)
+    return _ctx
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    import torch
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def normal(shape, seed, dtype=np.float32):
+    return np.random.default_rng(seed).standard_normal(shape, dtype=np.float32).astype(dtype)
+
+
+def check_attention_out(got, ref, what=""):
+    """BASELINE tolerance for attention outputs: <= 2e-3 max-abs and <= 1e-3 mean-abs."""
+    diff = np.abs(np.asarray(got, np.float64) - np.asarray(ref, np.float64))
+    assert np.all(np.isfinite(got)), what
+    assert diff.max() <= 2e-3, "%s max-abs %g" % (what, diff.max())
+    assert diff.mean() <= 1e-3, "%s mean-abs %g" % (what, diff.mean())
+    return diff.max()
+
+
+def check_scores(got, ref, what=""):
+    """BASELINE tolerance for H2O score vectors: <= 1e-4 relative (element-wise, with an
+    absolute floor at the f32 underflow scale of a softmax over <= 64K tokens)."""
+    got = np.asarray(got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    err = np.abs(got - ref)
+    tol = 1e-4 * np.abs(ref) + 1e-12
+    bad = err > tol
+    assert not bad.any(), "%s: %d scores off, worst rel %g" % (
+        what, bad.sum(), (err / np.maximum(np.abs(ref), 1e-30)).max())

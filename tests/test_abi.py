@@ -1,0 +1,65 @@
+"""CPU-side checks of the C ABI: the library loads, exports every declared symbol, and
+degrades to error codes (never a crash) without a device or with null arguments."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "argus_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(argus_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import argus_hip as A
+    declared = _declared_symbols()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(A.lib, name), "missing export " + name
+    assert sorted(A.EXPORTED_SYMBOLS) == declared
+    assert A.lib.argus_hip_abi_version() == 1
+
+
+def test_struct_layouts_match_header_field_order():
+    # the ctypes mirrors must list the same fields in the same order as the header structs
+    import argus_hip as A
+    text = open(os.path.join(ROOT, "include", "argus_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    pairs = {"argus_hip_attention_gen_args": A.AttentionGenArgs, "argus_hip_prefill_args": A.PrefillArgs,
+             "argus_hip_quant_attn_args": A.QuantAttnArgs, "argus_hip_quant_attn_ext": A.QuantAttnExt,
+             "argus_hip_quant_gather_args": A.QuantGatherArgs, "argus_hip_quant_flush_args": A.QuantFlushArgs,
+             "argus_hip_score_reduce_args": A.ScoreReduceArgs, "argus_hip_device_info": A.DeviceInfo}
+    for cname, cls in pairs.items():
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), text, re.S).group(1)
+        fields = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            for part in decl.split(","):
+                fields.append(re.findall(r"([A-Za-z_][A-Za-z0-9_]*)\s*(?:\[\d+\])?\s*$", part.strip())[0])
+        assert fields == [f[0] for f in cls._fields_], cname
+
+
+def test_degraded_without_device_or_context():
+    # mirrors engine/tests/gate_c_kivi_backend_cap.rs:90-146: with no GPU every op returns a
+    # negative code without crashing.
+    import argus_hip as A
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a device is present; the no-device path is exercised on CPU-only hosts")
+    h = C.c_void_p()
+    assert A.lib.argus_hip_create(0, C.byref(h)) == A.ERR_RUNTIME and not h.value
+    assert A.lib.argus_hip_attention_gen(None, None) == A.ERR_INVALID
+    assert A.lib.argus_hip_score_reduce(None, None) == A.ERR_INVALID
+    assert A.lib.argus_hip_attention_gen_quant(None, None) < 0
+    assert A.lib.argus_hip_flash_attention_prefill(None, None) < 0
+    assert A.lib.argus_hip_kv_scatter_f32_to_f16(None, None, None, None, None, None, 1, 64, 8, 0) == A.ERR_INVALID
+    assert A.lib.argus_hip_destroy(None) == A.ERR_INVALID
+    with pytest.raises(A.ArgusHipError):
+        A.Context(0)

@@ -1,0 +1,226 @@
+"""GPU parity: argus_hip_attention_gen (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle as O
+import textbook as T
+from gpu_util import check_attention_out, check_scores, ctx, dev, host, normal
+
+pytestmark = pytest.mark.gpu
+
+
+def run_decode(q, k, v, hkv, L, capacity, layout=0, scores=False, score_stride=None, **kw):
+    import torch
+    import argus_hip as A
+    qd, kd, vd = dev(q), dev(k), dev(v)
+    out = torch.full(q.shape, float("nan"), dtype=torch.float32, device="cuda")
+    sc = None
+    stride = 0
+    if scores:
+        stride = score_stride or L
+        sc = torch.full(q.shape[:-1] + (stride,), -7.0, dtype=torch.float32, device="cuda")
+    ctx().attention_gen(qd, kd, vd, out, hkv, L, capacity, layout=layout, scores=sc,
+                        score_stride=stride, **kw)
+    return (host(out), host(sc)) if scores else host(out)
+
+
+def f16(x):
+    return O.f32_to_f16_bits(x).view(np.float16)
+
+
+@pytest.mark.parametrize("kv", ["f32", "f16"])
+def test_reference_unit_case(kv):
+    # engine/src/backend/cpu/x86.rs:1811-1973 inputs (LCG seeds 42/137/53), its own tolerances.
+    hq, hkv, d, L, cap = 4, 2, 64, 16, 32
+    q = O.gen_data(hq * d, 42).reshape(hq, d)
+    k = O.gen_data(hkv * cap * d, 137).reshape(hkv, cap, d)
+    v = O.gen_data(hkv * cap * d, 53).reshape(hkv, cap, d)
+    if kv == "f16":
+        k, v = f16(k), f16(v)
+    got = run_decode(q, k, v, hkv, L, cap)
+    ref = O.attention_gen(q, k, v, hkv, L, cap)
+    assert np.abs(got - ref).max() < (1e-4 if kv == "f32" else 1e-3)
+    check_attention_out(got, O.attention_gen(q, k, v, hkv, L, cap, impl="avx2"))
+
+
+# engine/tests/test_attention_flash_decoding.rs:260-651 matrix: GQA ratios, chunk boundaries.
+MATRIX = [
+    (4, 4, 64, 1), (4, 4, 64, 32), (4, 2, 64, 33), (8, 2, 64, 256), (8, 2, 64, 1023),
+    (8, 2, 64, 1024), (8, 2, 64, 1025), (12, 2, 128, 2047), (12, 2, 128, 2500),
+    (8, 2, 128, 4096), (14, 2, 64, 1024), (8, 4, 256, 777), (32, 8, 128, 300), (6, 2, 256, 129),
+    (16, 2, 64, 555), (3, 1, 128, 70), (5, 1, 64, 200),
+]
+
+
+@pytest.mark.parametrize("hq,hkv,d,L", MATRIX)
+@pytest.mark.parametrize("kv", ["f16", "f32"])
+def test_decode_matrix(hq, hkv, d, L, kv):
+    cap = L + 19
+    q = normal((hq, d), 42 + L)
+    k = normal((hkv, cap, d), 137 + L)
+    v = normal((hkv, cap, d), 53 + L)
+    if kv == "f16":
+        k, v = f16(k), f16(v)
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, score_stride=cap)
+    ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, scores_stride=cap)
+    check_attention_out(got, ref, "out")
+    check_scores(sc[:, :L], p[:, :L], "scores")
+    assert np.all(sc[:, L:] == -7.0), "score columns beyond cache_seq_len must stay untouched"
+    assert np.abs(sc[:, :L].sum(axis=1) - 1.0).max() < 1e-3
+    # independent f64 check as well
+    r64, p64 = T.decode_attention(q, k, v, hkv, L)
+    check_attention_out(got, r64, "out vs f64")
+    # no-scores launch (single-split direct path for short L) gives the same output
+    got2 = run_decode(q, k, v, hkv, L, cap)
+    assert np.abs(got2 - got).max() < 1e-5
+
+
+def test_seq_major_layout():
+    hq, hkv, d, L = 8, 2, 128, 700
+    q = normal((hq, d), 1)
+    k = f16(normal((L, hkv, d), 2))
+    v = f16(normal((L, hkv, d), 3))
+    got = run_decode(q, k, v, hkv, L, 0, layout=1)
+    ref = O.attention_gen(q, k, v, hkv, L, 0, head_major=False)
+    check_attention_out(got, ref)
+
+
+def test_closed_form_zero_keys():
+    # engine/src/kv/standard_format.rs:3095-3199: K = 0 => uniform; out = mean(V), scores 0.5/0.5.
+    hq, hkv, d = 2, 1, 64
+    q = normal((hq, d), 5)
+    k = np.zeros((hkv, 4, d), np.float16)
+    v = np.zeros((hkv, 4, d), np.float16)
+    v[0, 0], v[0, 1] = 1.0, 3.0
+    got, sc = run_decode(q, k, v, hkv, 2, 4, scores=True)
+    assert np.allclose(got, 2.0, atol=1e-6) and np.allclose(sc, 0.5, atol=1e-7)
+    assert np.allclose(run_decode(q, k, v, hkv, 1, 4), 1.0, atol=1e-7)
+
+
+@pytest.mark.parametrize("L", [8, 3000])
+def test_nan_guards(L):
+    # engine/src/backend/cpu/common.rs:555-584.
+    hq, hkv, d = 4, 2, 64
+    q = normal((hq, d), 9)
+    k = normal((hkv, L, d), 10)
+    v = normal((hkv, L, d), 11)
+    k[0, 3, 0] = np.nan
+    k[1, L - 1, 5] = np.nan
+    got, sc = run_decode(q, k, v, hkv, L, L, scores=True)
+    ref, p = O.attention_gen(q, k, v, hkv, L, L, scores=True)
+    check_attention_out(got, ref)
+    check_scores(sc, p)
+    assert sc[0, 3] == 0.0 and sc[3, L - 1] == 0.0
+    # every logit NaN for kv head 0 -> uniform weights, out = mean of V rows
+    k[0] = np.nan
+    got, sc = run_decode(q, k, v, hkv, L, L, scores=True)
+    ref, p = O.attention_gen(q, k, v, hkv, L, L, scores=True)
+    check_attention_out(got, ref)
+    check_scores(sc, p)
+    assert np.allclose(sc[0], 1.0 / L)
+    got2 = run_decode(q, k, v, hkv, L, L)
+    check_attention_out(got2, ref)
+
+
+def test_softcap_index_and_window_start():
+    hq, hkv, d, L, cap = 8, 4, 256, 2048, 4096
+    q = normal((hq, d), 21) * 3.0
+    k = f16(normal((hkv, cap, d), 22))
+    v = f16(normal((hkv, cap, d), 23))
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, softcap=5.0)
+    ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, softcap=5.0)
+    check_attention_out(got, ref)
+    check_scores(sc, p)
+    r64, p64 = T.decode_attention(q, k, v, hkv, L, softcap=5.0)
+    check_attention_out(got, r64)
+    # index list == attention over the gathered rows
+    idx = np.sort(np.random.default_rng(3).choice(cap, L, replace=False)).astype(np.int32)
+    got = run_decode(q, k, v, hkv, L, cap, kv_index=dev(idx))
+    ref = O.attention_gen(q, k, v, hkv, L, cap, kv_index=idx)
+    check_attention_out(got, ref)
+    # kv_start: attends slots [kv_start, kv_start + L)
+    got = run_decode(q, k, v, hkv, 1000, cap, kv_start=77)
+    ref = O.attention_gen(q, np.ascontiguousarray(k[:, 77:1077]), np.ascontiguousarray(v[:, 77:1077]), hkv, 1000, 1000)
+    check_attention_out(got, ref)
+
+
+def test_batched_sequences_match_looped_calls():
+    # the reference has no batch dimension (engine/src/backend.rs:277-295): batch == a loop.
+    b, hq, hkv, d, L, cap = 5, 32, 8, 128, 1500, 1536
+    q = normal((b, hq, d), 42)
+    k = f16(normal((b, hkv, cap, d), 137))
+    v = f16(normal((b, hkv, cap, d), 53))
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, batch=b, kv_batch_stride=hkv * cap * d)
+    for i in range(b):
+        ref, p = O.attention_gen(q[i], k[i], v[i], hkv, L, cap, scores=True)
+        check_attention_out(got[i], ref, "seq %d" % i)
+        check_scores(sc[i], p, "seq %d" % i)
+
+
+def test_config1_qwen_shape():
+    # BASELINE config 1: Hq14 Hkv2 d64 L1024, f32 N(0,1) -> F16 KV, scale 1/8.
+    hq, hkv, d, L = 14, 2, 64, 1024
+    q = normal((hq, d), 42)
+    k = f16(normal((hkv, L, d), 137))
+    v = f16(normal((hkv, L, d), 53))
+    got = run_decode(q, k, v, hkv, L, L)
+    check_attention_out(got, O.attention_gen(q, k, v, hkv, L, L))
+    check_attention_out(got, O.attention_gen(q, k, v, hkv, L, L, impl="avx2"))
+    got_cap = run_decode(q, np.concatenate([k, k], 1), np.concatenate([v, v], 1), hkv, L, 2 * L)
+    assert np.array_equal(got, got_cap)
+
+
+@pytest.mark.parametrize("L", [4096, 32768])
+def test_config3_llama8b_shape_single_sequence(L):
+    hq, hkv, d = 32, 8, 128
+    q = normal((hq, d), 42)
+    k = f16(normal((hkv, L, d), 137))
+    v = f16(normal((hkv, L, d), 53))
+    got, sc = run_decode(q, k, v, hkv, L, L, scores=True)
+    ref, p = O.attention_gen(q, k, v, hkv, L, L, scores=True, impl="avx2")
+    check_attention_out(got, ref)
+    check_scores(sc, p)
+
+
+def test_config3_batch16_at_32k_properties_and_sampled_parity():
+    # 2 GiB of KV: generated on the device; parity on two sampled sequences, plus
+    # size-independent properties on all of them.
+    import torch
+    b, hq, hkv, d, L = 16, 32, 8, 128, 32768
+    g = torch.Generator(device="cuda").manual_seed(137)
+    k = torch.randn((b, hkv, L, d), generator=g, device="cuda", dtype=torch.float32).half()
+    v = torch.randn((b, hkv, L, d), generator=g, device="cuda", dtype=torch.float32).half()
+    q = dev(normal((b, hq, d), 42))
+    out = torch.empty((b, hq, d), dtype=torch.float32, device="cuda")
+    sc = torch.empty((b, hq, L), dtype=torch.float32, device="cuda")
+    ctx().attention_gen(q, k, v, out, hkv, L, L, scores=sc, score_stride=L, batch=b,
+                        kv_batch_stride=hkv * L * d)
+    torch.cuda.synchronize()
+    # probabilities: rows sum to 1, out == P @ V (linearity), permutation of tokens is a no-op.
+    assert (sc.sum(-1) - 1).abs().max().item() < 1e-3
+    pv = torch.einsum("bgrl,bgld->bgrd", sc.view(b, hkv, hq // hkv, L), v.float()).reshape(b, hq, d)
+    assert (pv - out).abs().max().item() < 1e-4
+    for i in (0, 11):
+        ref = O.attention_gen(host(q[i]), host(k[i]), host(v[i]), hkv, L, L, impl="avx2")
+        check_attention_out(host(out[i]), ref, "seq %d" % i)
+    perm = torch.randperm(L, device="cuda")
+    out2 = torch.empty_like(out[:1])
+    ctx().attention_gen(q[:1], k[0][:, perm].contiguous(), v[0][:, perm].contiguous(), out2, hkv, L, L)
+    assert (out2[0] - out[0]).abs().max().item() < 1e-5
+
+
+def test_argument_errors_return_negative_codes():
+    import torch
+    import argus_hip as A
+    q = torch.zeros((4, 64), device="cuda")
+    k = torch.zeros((2, 8, 64), device="cuda", dtype=torch.float16)
+    out = torch.zeros((4, 64), device="cuda")
+    c = ctx()
+    assert c.attention_gen(q, k, k, out, 3, 8, 8, check=False) == A.ERR_INVALID          # 4 % 3
+    assert c.attention_gen(q, k, k, out, 2, 0, 8, check=False) == A.ERR_INVALID          # empty
+    assert c.attention_gen(q, k, k, out, 2, 9, 8, check=False) == A.ERR_INVALID          # > capacity
+    q96 = torch.zeros((4, 96), device="cuda")
+    assert c.attention_gen(q96, k, k, q96.clone(), 2, 8, 8, check=False) == A.ERR_UNSUPPORTED
+    sc = torch.zeros((4, 4), device="cuda")
+    assert c.attention_gen(q, k, k, out, 2, 8, 8, scores=sc, score_stride=4, check=False) == A.ERR_INVALID
+    assert "score_stride" in c.last_error()

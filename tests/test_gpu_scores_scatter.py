@@ -1,0 +1,126 @@
+"""GPU parity: score reduce, KV scatter and the post-eviction + H2O flow (BASELINE config 5)."""
+import numpy as np
+import pytest
+
+import oracle as O
+import textbook as T
+from gpu_util import check_attention_out, check_scores, ctx, dev, host, normal
+
+pytestmark = pytest.mark.gpu
+
+
+def f16(x):
+    return O.f32_to_f16_bits(x).view(np.float16)
+
+
+def test_score_reduce_known_answers():
+    # engine/src/bin/test_cuda_gpu_score_device.rs cases 1 and 2.
+    import torch
+    nl, hq, hkv, max_seq, L = 2, 2, 1, 8, 3
+    sc = np.zeros((nl, hq, max_seq), np.float32)
+    sc[0, 0, :3], sc[0, 1, :3] = [0.1, 0.2, 0.7], [0.3, 0.3, 0.4]
+    sc[1, 0, :3], sc[1, 1, :3] = [0.5, 0.4, 0.1], [0.2, 0.2, 0.6]
+    s = dev(sc)
+    imp = torch.zeros(max_seq, device="cuda")
+    himp = torch.zeros(hkv * max_seq, device="cuda")
+    ctx().score_reduce(s, imp, himp, 1.0, nl, hq, hkv, L, max_seq, max_seq)
+    assert np.abs(host(imp)[:3] - [0.7, 0.6, 1.1]).max() < 1e-5
+    assert np.abs(host(himp)[:3] - [0.35, 0.30, 0.55]).max() < 1e-5
+    assert not host(imp)[3:].any()
+    imp.zero_()
+    himp.zero_()
+    for _ in range(2):
+        ctx().score_reduce(s, imp, himp, 0.5, nl, hq, hkv, L, max_seq, max_seq)
+    assert np.abs(host(imp)[:3] - 1.5 * np.array([0.7, 0.6, 1.1])).max() < 1e-5
+    lf = torch.zeros(nl * max_seq, device="cuda")
+    ctx().score_reduce_per_layer(s, lf, 1.0, nl, hq, hkv, L, max_seq, max_seq)
+    assert np.abs(host(lf)[:3] - [0.4, 0.5, 1.1]).max() < 1e-6
+    assert np.abs(host(lf)[8:11] - [0.7, 0.6, 0.7]).max() < 1e-6
+
+
+@pytest.mark.parametrize("nl,hq,hkv,L,stride", [(1, 8, 4, 2048, 4096), (28, 14, 2, 1000, 1024),
+                                                (32, 32, 8, 4097, 8192), (3, 16, 16, 70, 70)])
+def test_score_reduce_vs_oracle(nl, hq, hkv, L, stride):
+    import torch
+    rng = np.random.default_rng(nl * 1000 + L)
+    sc = rng.random((nl, hq, stride), dtype=np.float32)
+    imp0 = rng.random(stride, dtype=np.float32)
+    himp0 = rng.random(hkv * stride, dtype=np.float32)
+    lf0 = rng.random(nl * stride, dtype=np.float32)
+    imp, himp, lf = imp0.copy(), himp0.copy(), lf0.copy()
+    O.score_fused_reduce(sc, imp, himp, 0.9, nl, hq, hkv, L, stride, stride)
+    O.score_reduce_per_layer(sc, lf, 0.9, nl, hq, L, stride, stride)
+    s, di, dh, dl = dev(sc), dev(imp0), dev(himp0), dev(lf0)
+    ctx().score_reduce(s, di, dh, 0.9, nl, hq, hkv, L, stride, stride)
+    ctx().score_reduce_per_layer(s, dl, 0.9, nl, hq, hkv, L, stride, stride)
+    assert np.allclose(host(di), imp, rtol=1e-5, atol=0)
+    assert np.allclose(host(dh), himp, rtol=1e-5, atol=0)
+    assert np.allclose(host(dl), lf, rtol=1e-5, atol=0)
+    # untouched beyond cache_seq_len
+    assert np.array_equal(host(di)[L:], imp0[L:])
+    import argus_hip as A
+    assert ctx().score_reduce(s, di, dh, 0.9, nl, hq, 17, L, stride, stride, check=False) < 0
+
+
+@pytest.mark.parametrize("seq_len,write_pos", [(1, 0), (1, 37), (64, 10), (2048, 0)])
+@pytest.mark.parametrize("to_f16", [True, False])
+def test_kv_scatter(seq_len, write_pos, to_f16):
+    import torch
+    hkv, d, cap = 8, 128, 2100
+    ks = normal((seq_len, hkv, d), 1) * 3
+    vs = normal((seq_len, hkv, d), 2) * 3
+    dt = np.float16 if to_f16 else np.float32
+    kd = np.full((hkv, cap, d), 7, dt)
+    vd = np.full((hkv, cap, d), 7, dt)
+    dk, dv = dev(kd), dev(vd)
+    ctx().kv_scatter(dev(ks), dev(vs), dk, dv, hkv, d, cap, write_pos,
+                     seq_len=None if (seq_len == 1 and to_f16) else seq_len)
+    O.kv_scatter(ks, vs, kd, vd, write_pos)
+    assert np.array_equal(host(dk).view(np.uint16 if to_f16 else np.uint32),
+                          kd.view(np.uint16 if to_f16 else np.uint32))
+    assert np.array_equal(host(dv).view(np.uint16 if to_f16 else np.uint32),
+                          vd.view(np.uint16 if to_f16 else np.uint32))
+    import argus_hip as A
+    assert ctx().kv_scatter(dev(ks), dev(vs), dk, dv, hkv, d, cap, cap, seq_len=seq_len, check=False) == A.ERR_INVALID
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+@pytest.mark.parametrize("softcap", [50.0, 0.0])
+def test_config5_post_eviction_h2o_flow(batch, softcap):
+    # BASELINE config 5 (Gemma-2-2B shape): 8192-token history compacted StreamingLLM-style
+    # (sink 4 + recent 2044 -> kept positions {0..3} U {6148..8191}, 2048 valid slots) into a
+    # capacity-4096 HeadMajor cache; decode with soft-cap 50; per-position probabilities are
+    # emitted and reduced to H2O importance.  soft-cap 0 is the reference-CPU-semantics variant.
+    import torch
+    hq, hkv, d, hist, cap = 8, 4, 256, 8192, 4096
+    keep = O.streaming_keep(4, 2044, hist, 0)
+    L = len(keep)
+    assert L == 2048
+    q = normal((batch, hq, d), 42)
+    kc = np.zeros((batch, hkv, cap, d), np.float16)
+    vc = np.zeros((batch, hkv, cap, d), np.float16)
+    for b in range(batch):
+        kh = f16(normal((hkv, hist, d), 137 + b))
+        vh = f16(normal((hkv, hist, d), 53 + b))
+        kc[b] = O.compact_keep(kh, keep, cap)
+        vc[b] = O.compact_keep(vh, keep, cap)
+    out = torch.empty((batch, hq, d), device="cuda")
+    sc = torch.zeros((batch, hq, cap), device="cuda")
+    ctx().attention_gen(dev(q), dev(kc), dev(vc), out, hkv, L, cap, scores=sc, score_stride=cap,
+                        batch=batch, kv_batch_stride=hkv * cap * d, softcap=softcap)
+    got, gsc = host(out), host(sc)
+    for b in range(batch):
+        ref, p = O.attention_gen(q[b], kc[b], vc[b], hkv, L, cap, scores=True, scores_stride=cap,
+                                 softcap=softcap)
+        check_attention_out(got[b], ref, "seq %d" % b)
+        check_scores(gsc[b, :, :L], p[:, :L], "seq %d" % b)
+        # fused reduce (single layer) on the device score buffer of this sequence
+        imp = torch.zeros(cap, device="cuda")
+        himp = torch.zeros(hkv * cap, device="cuda")
+        ctx().score_reduce(sc[b], imp, himp, 1.0, 1, hq, hkv, L, cap, cap)
+        oi, oh = np.zeros(cap, np.float32), np.zeros(hkv * cap, np.float32)
+        O.score_fused_reduce(p, oi, oh, 1.0, 1, hq, hkv, L, cap, cap)
+        check_scores(host(imp), oi, "importance")
+        check_scores(host(himp), oh, "head importance")
+        flat, head = T.score_reduce(T.decode_attention(q[b], kc[b], vc[b], hkv, L, softcap=softcap)[1][None], hkv)
+        check_scores(host(imp)[:L], flat, "importance vs f64")
