@@ -20,6 +20,7 @@
 #include "argus_hip_internal.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace {
 
@@ -55,9 +56,16 @@ struct KvVec<float> {
   using vec = float4_t;
 };
 
-__device__ __forceinline__ float apply_softcap(float s, float cap) {
-  return cap > 0.0f ? cap * tanhf(s / cap) : s;
+// cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1); the argument is clamped where
+// tanh is 1 to f32 precision so exp cannot overflow.  The caller handles NaN.
+__device__ __forceinline__ float softcap_tanh(float s, float cap, float inv_cap) {
+  float x = s * inv_cap;
+  x = fminf(fmaxf(x, -15.0f), 15.0f);
+  const float e = __expf(2.0f * x);
+  return cap * (1.0f - 2.0f * __frcp_rn(e + 1.0f));
 }
+
+enum DecodeMode { kPlain = 0, kSoftcap = 1, kGeneric = 2 };
 
 // Uniform-weights fallback of common.rs:561-577: out = mean of the attended V rows, every
 // probability 1/len.  Only reached when no logit is finite, so speed is irrelevant.
@@ -81,7 +89,7 @@ __device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
   }
 }
 
-template <int D, int GT, typename KV_T, int U>
+template <int D, int GT, typename KV_T, int U, int MODE>
 __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p) {
   constexpr int E = KvVec<KV_T>::E;
   using vec_t = typename KvVec<KV_T>::vec;
@@ -122,17 +130,23 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
     for (int e = 0; e < E; ++e) acc[g][e] = 0.0f;
   }
 
-  for (int base = t_begin + wave * TILE; base < t_end; base += 4 * TILE) {
+  const bool use_idx = (MODE == kGeneric) && idx != nullptr;
+  const bool use_cap = (MODE == kSoftcap) || (MODE == kGeneric && p.softcap > 0.0f);
+  const float inv_cap = use_cap ? 1.0f / p.softcap : 0.0f;
+
+  // One tile = U load instructions per stream per wave.  FULL tiles need no row masking.
+  auto process_tile = [&](const int base, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
     vec_t kr[U], vr[U];
     bool valid[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = base + u * RPW + grp;
-      valid[u] = t < t_end;
+      valid[u] = FULL || t < t_end;
       const int tc = valid[u] ? t : (t_end - 1);
-      const int64_t slot = idx ? (int64_t)idx[tc] : (int64_t)(p.kv_start + tc);
-      kr[u] = *(const vec_t *)(kb + slot * p.row_stride);
-      vr[u] = *(const vec_t *)(vb + slot * p.row_stride);
+      const int64_t slot = use_idx ? (int64_t)idx[tc] : (int64_t)(p.kv_start + tc);
+      kr[u] = __builtin_nontemporal_load((const vec_t *)(kb + slot * p.row_stride));
+      vr[u] = __builtin_nontemporal_load((const vec_t *)(vb + slot * p.row_stride));
     }
 
     float s[U][GT];
@@ -144,8 +158,13 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
 #pragma unroll
         for (int e = 0; e < E; ++e) part = fmaf(q[g][e], (float)kr[u][e], part);
         float sv = group_allreduce_sum<LPR>(part);
-        sv = apply_softcap(sv, p.softcap);
-        sv = (sv != sv) ? kNegInf : sv;  // NaN logit counts as -inf (common.rs:555-560)
+        // NaN logit counts as -inf (common.rs:555-560)
+        if (use_cap) {
+          const float capped = softcap_tanh(sv, p.softcap, inv_cap);
+          sv = (sv != sv) ? kNegInf : capped;
+        } else {
+          sv = fmaxf(sv, kNegInf);
+        }
         s[u][g] = valid[u] ? sv : kNegInf;
       }
     }
@@ -184,6 +203,12 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
       }
       l[g] = l[g] * alpha + lsum;
     }
+  };
+
+  {
+    int base = t_begin + wave * TILE;
+    for (; base + TILE <= t_end; base += 4 * TILE) process_tile(base, std::true_type{});
+    if (base < t_end) process_tile(base, std::false_type{});
   }
 
   // ---- merge the RPW row groups of this wave --------------------------------------------
@@ -261,20 +286,30 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
 }
 
 // Second pass: log-sum-exp merge of the splits of one (sequence, Q head); optional in-place
-// logits -> probabilities rewrite of the score row.
-template <typename KV_T>
-__global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams p, int D) {
+// logits -> probabilities rewrite of the score row.  The 256 threads are arranged as
+// (split group) x (float4 column) so the loop over splits is short and the loads are wide.
+constexpr int kMaxSplits = 128;
+
+template <typename KV_T, int D>
+__global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams p) {
+  constexpr int CQ = D / 4;      // float4 columns per row
+  constexpr int NSG = 256 / CQ;  // split groups
   const int h = blockIdx.x, b = blockIdx.y;
   const int64_t pbase = ((int64_t)b * p.n_heads_q + h) * p.nsplit;
+  __shared__ float sh_w[kMaxSplits];
   __shared__ float sh_m, sh_l;
+  __shared__ float4_t sh_o[NSG][CQ];
   if (threadIdx.x < 64) {
     float mm = kNegInf;
     for (int s = threadIdx.x; s < p.nsplit; s += 64) mm = fmaxf(mm, p.ws_ml[(pbase + s) * 2]);
     mm = wave_allreduce_max(mm);
     const float m_ref = (mm == kNegInf) ? 0.0f : mm;
     float ll = 0.0f;
-    for (int s = threadIdx.x; s < p.nsplit; s += 64)
-      ll += p.ws_ml[(pbase + s) * 2 + 1] * __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
+    for (int s = threadIdx.x; s < p.nsplit; s += 64) {
+      const float w = __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
+      sh_w[s] = w;
+      ll += p.ws_ml[(pbase + s) * 2 + 1] * w;
+    }
     ll = wave_allreduce_sum(ll);
     if (threadIdx.x == 0) {
       sh_m = mm;
@@ -287,17 +322,21 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     uniform_fallback<KV_T>(p, b, h, D);
     return;
   }
-  const float m_ref = mm;
   const float inv = 1.0f / ll;
-  for (int c = threadIdx.x; c < D; c += 256) {
-    float o = 0.0f;
-    for (int s = 0; s < p.nsplit; ++s)
-      o += p.ws_o[(pbase + s) * D + c] * __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
-    p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = o * inv;
+  const int cq = threadIdx.x % CQ, sg = threadIdx.x / CQ;
+  float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int s = sg; s < p.nsplit; s += NSG)
+    o += *(const float4_t *)(p.ws_o + (pbase + s) * D + 4 * cq) * sh_w[s];
+  sh_o[sg][cq] = o;
+  __syncthreads();
+  if (sg == 0) {
+#pragma unroll
+    for (int g = 1; g < NSG; ++g) o += sh_o[g][cq];
+    *(float4_t *)(p.out + (int64_t)b * p.out_bs + (int64_t)h * D + 4 * cq) = o * inv;
   }
   if (p.scores) {
     float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    for (int t = threadIdx.x; t < p.len; t += 256) srow[t] = __expf(srow[t] - m_ref) * inv;
+    for (int t = threadIdx.x; t < p.len; t += 256) srow[t] = __expf(srow[t] - mm) * inv;
   }
 }
 
@@ -314,9 +353,11 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
   constexpr int tile_rows = 4 * (64 / (D / E)) * U;  // rows one workgroup consumes per iteration
 
   const int pairs = batch * p.n_heads_kv;
-  const int target_wgs = ctx->compute_units * 4;
+  // Many more workgroups than resident slots, so the last partially filled round of the grid
+  // costs little; bounded below by one tile per wave.
+  const int target_wgs = ctx->compute_units * 24;
   const int max_splits = (p.len + tile_rows - 1) / tile_rows;
-  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, 512}));
+  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, kMaxSplits}));
   int chunk = (p.len + nsplit - 1) / nsplit;
   chunk = (chunk + tile_rows - 1) / tile_rows * tile_rows;
   nsplit = (p.len + chunk - 1) / chunk;
@@ -336,11 +377,16 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
   dim3 grid(nsplit, p.n_heads_kv, batch);
   {
     KernelTimer timer(ctx, stream);
-    hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U>), grid, dim3(256), 0, stream, p);
+    if (p.kv_index)
+      hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kGeneric>), grid, dim3(256), 0, stream, p);
+    else if (p.softcap > 0.0f)
+      hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kSoftcap>), grid, dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kPlain>), grid, dim3(256), 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   if (!p.direct) {
-    hipLaunchKernelGGL((decode_combine_kernel<KV_T>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p, D);
+    hipLaunchKernelGGL((decode_combine_kernel<KV_T, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
     ARGUS_HIP_CHECK(ctx, hipGetLastError());
   }
   return ARGUS_HIP_OK;
@@ -417,6 +463,12 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
   p.softcap = a->softcap;
   if (a->batch > 1 && p.kv_bs == 0)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: batch > 1 needs kv_batch_stride");
+  // The kernels move K/V rows and output rows as 16-byte vectors.
+  const int64_t kv_vec = a->kv_dtype == ARGUS_HIP_F16 ? 8 : 4;
+  if (((uintptr_t)a->k_cache | (uintptr_t)a->v_cache | (uintptr_t)a->out) & 15)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: k/v/out must be 16-byte aligned");
+  if ((p.kv_bs % kv_vec) || (p.out_bs % 4))
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: batch strides must keep 16-byte alignment");
 
   hipStream_t stream = (hipStream_t)a->stream;
   const bool want_scores = a->scores_out != nullptr;
