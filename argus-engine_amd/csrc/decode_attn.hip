@@ -17,31 +17,14 @@
 //    combines the splits with a log-sum-exp merge, writes `out`, and -- when post-softmax scores
 //    were requested -- turns the logits the first pass stored in `scores_out` into probabilities
 //    in place (exact global max / sum are only known there).
-#include "argus_hip_internal.hpp"
+#include "decode_common.hpp"
 
 #include <algorithm>
 #include <type_traits>
 
 namespace {
 
-struct DecodeParams {
-  const float *q;
-  const void *k;
-  const void *v;
-  float *out;
-  float *scores;
-  const int32_t *kv_index;
-  float *ws_ml;  // [batch, Hq, nsplit, 2]
-  float *ws_o;   // [batch, Hq, nsplit, D]
-  int32_t n_heads_q, n_heads_kv, group;  // group = Hq / Hkv
-  int32_t len, kv_start, chunk, nsplit;
-  int32_t score_stride;
-  int64_t row_stride;   // elements between consecutive token rows of one KV head
-  int64_t head_stride;  // elements between KV heads
-  int64_t q_bs, out_bs, kv_bs, score_bs, index_bs;
-  float scale, softcap;
-  int32_t direct;  // nsplit == 1 and no scores: first pass writes `out` itself
-};
+using namespace argus_decode;
 
 template <typename KV_T>
 struct KvVec;
@@ -56,38 +39,7 @@ struct KvVec<float> {
   using vec = float4_t;
 };
 
-// cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1); the argument is clamped where
-// tanh is 1 to f32 precision so exp cannot overflow.  The caller handles NaN.
-__device__ __forceinline__ float softcap_tanh(float s, float cap, float inv_cap) {
-  float x = s * inv_cap;
-  x = fminf(fmaxf(x, -15.0f), 15.0f);
-  const float e = __expf(2.0f * x);
-  return cap * (1.0f - 2.0f * __frcp_rn(e + 1.0f));
-}
-
 enum DecodeMode { kPlain = 0, kSoftcap = 1, kGeneric = 2 };
-
-// Uniform-weights fallback of common.rs:561-577: out = mean of the attended V rows, every
-// probability 1/len.  Only reached when no logit is finite, so speed is irrelevant.
-template <typename KV_T>
-__device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
-  const int kvh = h / p.group;
-  const KV_T *vb = (const KV_T *)p.v + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;
-  const int32_t *idx = p.kv_index ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
-  const float u = 1.0f / (float)p.len;
-  for (int c = threadIdx.x; c < D; c += blockDim.x) {
-    float acc = 0.0f;
-    for (int t = 0; t < p.len; ++t) {
-      const int64_t slot = idx ? idx[t] : (p.kv_start + t);
-      acc += u * (float)vb[slot * p.row_stride + c];
-    }
-    p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = acc;
-  }
-  if (p.scores) {
-    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = u;
-  }
-}
 
 template <int D, int GT, typename KV_T, int U, int MODE>
 __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p) {
@@ -285,61 +237,6 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
   }
 }
 
-// Second pass: log-sum-exp merge of the splits of one (sequence, Q head); optional in-place
-// logits -> probabilities rewrite of the score row.  The 256 threads are arranged as
-// (split group) x (float4 column) so the loop over splits is short and the loads are wide.
-constexpr int kMaxSplits = 128;
-
-template <typename KV_T, int D>
-__global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams p) {
-  constexpr int CQ = D / 4;      // float4 columns per row
-  constexpr int NSG = 256 / CQ;  // split groups
-  const int h = blockIdx.x, b = blockIdx.y;
-  const int64_t pbase = ((int64_t)b * p.n_heads_q + h) * p.nsplit;
-  __shared__ float sh_w[kMaxSplits];
-  __shared__ float sh_m, sh_l;
-  __shared__ float4_t sh_o[NSG][CQ];
-  if (threadIdx.x < 64) {
-    float mm = kNegInf;
-    for (int s = threadIdx.x; s < p.nsplit; s += 64) mm = fmaxf(mm, p.ws_ml[(pbase + s) * 2]);
-    mm = wave_allreduce_max(mm);
-    const float m_ref = (mm == kNegInf) ? 0.0f : mm;
-    float ll = 0.0f;
-    for (int s = threadIdx.x; s < p.nsplit; s += 64) {
-      const float w = __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
-      sh_w[s] = w;
-      ll += p.ws_ml[(pbase + s) * 2 + 1] * w;
-    }
-    ll = wave_allreduce_sum(ll);
-    if (threadIdx.x == 0) {
-      sh_m = mm;
-      sh_l = ll;
-    }
-  }
-  __syncthreads();
-  const float mm = sh_m, ll = sh_l;
-  if (!(ll > 0.0f && ll < __builtin_huge_valf())) {
-    uniform_fallback<KV_T>(p, b, h, D);
-    return;
-  }
-  const float inv = 1.0f / ll;
-  const int cq = threadIdx.x % CQ, sg = threadIdx.x / CQ;
-  float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int s = sg; s < p.nsplit; s += NSG)
-    o += *(const float4_t *)(p.ws_o + (pbase + s) * D + 4 * cq) * sh_w[s];
-  sh_o[sg][cq] = o;
-  __syncthreads();
-  if (sg == 0) {
-#pragma unroll
-    for (int g = 1; g < NSG; ++g) o += sh_o[g][cq];
-    *(float4_t *)(p.out + (int64_t)b * p.out_bs + (int64_t)h * D + 4 * cq) = o * inv;
-  }
-  if (p.scores) {
-    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    for (int t = threadIdx.x; t < p.len; t += 256) srow[t] = __expf(srow[t] - mm) * inv;
-  }
-}
-
 template <int D, int GT, typename KV_T>
 constexpr int unroll_for() {
   // Keep q + acc + in-flight K/V rows inside the register file at >= 2 waves per SIMD.
@@ -386,7 +283,7 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   if (!p.direct) {
-    hipLaunchKernelGGL((decode_combine_kernel<KV_T, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<KV_T>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
     ARGUS_HIP_CHECK(ctx, hipGetLastError());
   }
   return ARGUS_HIP_OK;
