@@ -1,0 +1,335 @@
+// Causal GQA flash-attention prefill on the gfx950 matrix cores.
+//
+// Stands in for Backend::flash_attention_prefill (engine/src/backend.rs:1011-1027; CPU semantics
+// engine/src/layers/attention.rs:78-351, CUDA behaviour model
+// engine/src/backend/cuda_pc/kernels.cu:559-816): key c is visible to query row r iff
+// c <= r + q_start_pos (and c + window > r + q_start_pos), q_start_pos = cache_seq_len - seq_len;
+// fully masked rows give zeros.
+//
+// Design:
+//  * v_mfma_f32_32x32x16_f16 throughout, in the transposed formulation
+//        S^T = K . Q^T     (A = K rows from LDS, B = Q rows held in registers)
+//        O^T = V^T . P^T   (A = V^T from LDS, B = P^T taken straight from the S^T accumulators)
+//    so a lane owns one query column: the softmax runs over in-lane registers plus one
+//    cross-half shuffle, the O rescale is a per-lane scalar, and P never goes through LDS.
+//  * One wave = 32 query rows of one Q head.  A workgroup's 4 waves are HPW heads of one GQA group
+//    times 4/HPW consecutive 32-row blocks; they share each K/V tile staged once in LDS (K row
+//    major, V transposed while being written), so GQA multiplies neither HBM nor LDS-fill traffic.
+//  * The next K/V tile is fetched into registers while the current one is being consumed.
+//  * blockIdx is laid out so that consecutive workgroups hit different KV heads (one XCD / L2 per
+//    KV head when there are 8 of them) and long (late) query tiles are issued before short ones,
+//    pairing a long and a short tile on each compute unit.
+#include "argus_hip_internal.hpp"
+
+namespace {
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+struct PrefillParams {
+  const void *q;
+  const void *k;
+  const void *v;
+  void *out;
+  int32_t n_heads_q, n_heads_kv, group;
+  int32_t seq_len, cache_len, q_start, capacity, batch, window;
+  int32_t n_qtiles, group_chunks;  // grid decomposition
+  int32_t q_f16, out_f16;
+  float scale_log2e;
+};
+
+template <typename KV_T>
+__device__ __forceinline__ half8_t load_kv_chunk(const KV_T *p);
+template <>
+__device__ __forceinline__ half8_t load_kv_chunk<_Float16>(const _Float16 *p) {
+  return *(const half8_t *)p;
+}
+template <>
+__device__ __forceinline__ half8_t load_kv_chunk<float>(const float *p) {
+  const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
+  half8_t h;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    h[e] = (_Float16)a[e];
+    h[4 + e] = (_Float16)b[e];
+  }
+  return h;
+}
+
+template <int D, int HPW, typename KV_T>
+__global__ __launch_bounds__(256) void prefill_kernel(const PrefillParams p) {
+  constexpr int BN = (D <= 128) ? 64 : 32;   // keys per tile
+  constexpr int QPW = 4 / HPW;               // 32-row query blocks per workgroup
+  constexpr int KP = D + 8;                  // K tile row pitch (halfs)
+  constexpr int VP = BN + 4;                 // V^T tile row pitch (halfs), keeps 8-byte alignment
+  constexpr int KK = D / 16;                 // MFMA k-steps over head_dim
+  constexpr int KB = BN / 32;                // S^T row blocks (32 keys each)
+  constexpr int RB = D / 32;                 // O^T row blocks (32 channels each)
+  constexpr int CH = BN * D / 8 / 256;       // 16-byte chunks per thread per tile
+
+  __shared__ __attribute__((aligned(16))) _Float16 sK[BN * KP];
+  __shared__ __attribute__((aligned(16))) _Float16 sVt[D * VP];
+
+  // ---- work decomposition ------------------------------------------------------------------
+  const int pairs = p.batch * p.n_heads_kv;
+  const int pair = blockIdx.x % pairs;
+  const int j = blockIdx.x / pairs;
+  const int b = pair / p.n_heads_kv, kvh = pair % p.n_heads_kv;
+  const int gc = j % p.group_chunks;
+  const int jt = j / p.group_chunks;
+  // long tiles first (descending), then the short ones ascending
+  const int half_t = (p.n_qtiles + 1) / 2;
+  const int qt = jt < half_t ? (p.n_qtiles - 1 - jt) : (jt - half_t);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ln = lane & 31, hl = lane >> 5;
+  const int h = kvh * p.group + min(gc * HPW + (wave % HPW), p.group - 1);
+  const bool head_ok = gc * HPW + (wave % HPW) < p.group;
+  const int qb = qt * QPW + wave / HPW;
+  const int r0 = qb * 32;            // first query row of this wave
+  const int row = r0 + ln;           // this lane's query row
+  const bool row_ok = head_ok && row < p.seq_len;
+
+  // ---- Q as the B operand: lane (query ln, half hl) holds Q[row][16kk + 8hl .. +7] ----------
+  half8_t qreg[KK];
+  {
+    const int64_t qoff = (((int64_t)b * p.seq_len + row) * p.n_heads_q + h) * D + 8 * hl;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (row_ok) {
+        if (p.q_f16) x = *(const half8_t *)((const _Float16 *)p.q + qoff + 16 * kk);
+        else x = load_kv_chunk<float>((const float *)p.q + qoff + 16 * kk);
+      }
+      qreg[kk] = x;
+    }
+  }
+
+  float16_t o_acc[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o_acc[r][i] = 0.0f;
+  float m_run = kNegInf, l_run = 0.0f;
+
+  // ---- key range of the workgroup -----------------------------------------------------------
+  const int wg_row_last = min(p.seq_len, (qt + 1) * QPW * 32) - 1;
+  const int kv_end = min(p.cache_len, wg_row_last + p.q_start + 1);
+  int kv_begin = 0;
+  if (p.window > 0) kv_begin = max(0, qt * QPW * 32 + p.q_start - p.window + 1);
+  const int kt_begin = kv_begin / BN, kt_end = (kv_end + BN - 1) / BN;
+
+  const KV_T *kbase = (const KV_T *)p.k + ((int64_t)b * p.n_heads_kv + kvh) * p.capacity * D;
+  const KV_T *vbase = (const KV_T *)p.v + ((int64_t)b * p.n_heads_kv + kvh) * p.capacity * D;
+
+  half8_t kpre[CH], vpre[CH];
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int cid = threadIdx.x + 256 * c;
+      const int key = kt * BN + cid / (D / 8), dc = cid % (D / 8);
+      half8_t kx = {0, 0, 0, 0, 0, 0, 0, 0}, vx = kx;
+      if (key < p.cache_len) {
+        kx = load_kv_chunk<KV_T>(kbase + (int64_t)key * D + 8 * dc);
+        vx = load_kv_chunk<KV_T>(vbase + (int64_t)key * D + 8 * dc);
+      }
+      kpre[c] = kx;
+      vpre[c] = vx;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int cid = threadIdx.x + 256 * c;
+      const int key = cid / (D / 8), dc = cid % (D / 8);
+      *(half8_t *)(sK + key * KP + 8 * dc) = kpre[c];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sVt[(8 * dc + e) * VP + key] = vpre[c][e];
+    }
+  };
+
+  if (kt_begin < kt_end) fetch(kt_begin);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    __syncthreads();  // every wave is done reading the previous tile
+    stage();
+    __syncthreads();
+    if (kt + 1 < kt_end) fetch(kt + 1);
+
+    const int key0 = kt * BN;
+    // Waves whose rows cannot see this tile skip the math (they still take part in the barriers).
+    const int wave_hi = r0 + 31 + p.q_start;  // largest visible key of the wave
+    const int wave_lo = p.window > 0 ? (r0 + p.q_start - p.window + 1) : 0;
+    if (!head_ok || r0 >= p.seq_len || key0 > wave_hi || key0 + BN <= wave_lo) continue;
+
+    // ---- S^T = K . Q^T ------------------------------------------------------------------------
+    float16_t s_acc[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_acc[kb][i] = 0.0f;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
+        s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
+      }
+    }
+
+    // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) ---------
+    const int q_pos = row + p.q_start;
+    const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
+                           (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
+    if (need_mask) {
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + 32 * kb + 8 * (i / 4) + 4 * hl + (i % 4);
+          bool ok = key <= q_pos && key < p.cache_len;
+          if (p.window > 0) ok = ok && (key + p.window > q_pos);
+          if (!ok) s_acc[kb][i] = kNegInf;
+        }
+    }
+
+    // ---- online softmax for this lane's query column ----------------------------------------
+    float mt = kNegInf;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m_run, mt * p.scale_log2e);
+    const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+    m_run = m_new;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        s_acc[kb][i] = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][i], p.scale_log2e, -m_ref));
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
+    }
+
+    // ---- O^T += V^T . P^T --------------------------------------------------------------------
+    // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
+    // rounding cancels in the final normalisation.
+    float lsum = 0.0f;
+#pragma unroll
+    for (int jn = 0; jn < BN / 16; ++jn) {
+      half8_t pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pb[e] = (_Float16)s_acc[jn / 2][8 * (jn % 2) + e];
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const half2_t pr = {pb[e], pb[e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
+        lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
+      }
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const _Float16 *vrow = sVt + (32 * r + ln) * VP + 16 * jn + 4 * hl;
+        const half4_t lo = *(const half4_t *)vrow, hi = *(const half4_t *)(vrow + 8);
+        const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, o_acc[r], 0, 0, 0);
+      }
+    }
+    l_run = l_run * alpha + lsum;
+  }
+
+  // ---- normalise and store: lane = query row, registers = channels ---------------------------
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if (!row_ok) return;
+  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+  const int64_t ooff = (((int64_t)b * p.seq_len + row) * p.n_heads_q + h) * D;
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int d0 = 32 * r + 8 * i4 + 4 * hl;
+      float4_t o = {o_acc[r][4 * i4] * inv, o_acc[r][4 * i4 + 1] * inv, o_acc[r][4 * i4 + 2] * inv,
+                    o_acc[r][4 * i4 + 3] * inv};
+      if (p.out_f16) {
+        half4_t oh = {(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
+        *(half4_t *)((_Float16 *)p.out + ooff + d0) = oh;
+      } else {
+        *(float4_t *)((float *)p.out + ooff + d0) = o;
+      }
+    }
+}
+
+template <int D, int HPW, typename KV_T>
+int launch(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
+  constexpr int QPW = 4 / HPW;
+  p.n_qtiles = (p.seq_len + 32 * QPW - 1) / (32 * QPW);
+  p.group_chunks = (p.group + HPW - 1) / HPW;
+  const int64_t wgs = (int64_t)p.batch * p.n_heads_kv * p.group_chunks * p.n_qtiles;
+  if (wgs > 0x7fffffff) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: grid too large");
+  {
+    KernelTimer timer(ctx, stream);
+    hipLaunchKernelGGL((prefill_kernel<D, HPW, KV_T>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  }
+  ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  return 1;  // dispatched
+}
+
+template <int D, typename KV_T>
+int dispatch_heads(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
+  if (p.group % 4 == 0) return launch<D, 4, KV_T>(ctx, p, stream);
+  if (p.group % 2 == 0) return launch<D, 2, KV_T>(ctx, p, stream);
+  return launch<D, 1, KV_T>(ctx, p, stream);
+}
+
+template <typename KV_T>
+int dispatch_dim(argus_hip_ctx *ctx, PrefillParams &p, int D, hipStream_t stream) {
+  switch (D) {
+    case 64: return dispatch_heads<64, KV_T>(ctx, p, stream);
+    case 128: return dispatch_heads<128, KV_T>(ctx, p, stream);
+    default: return dispatch_heads<256, KV_T>(ctx, p, stream);
+  }
+}
+
+}  // namespace
+
+ARGUS_API int argus_hip_flash_attention_prefill(argus_hip_ctx *ctx, const argus_hip_prefill_args *a) {
+  if (!ctx || !a) return ARGUS_HIP_ERR_INVALID;
+  if (!a->q || !a->k_cache || !a->v_cache || !a->out)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "flash_attention_prefill: null tensor pointer");
+  if (a->n_heads_q <= 0 || a->n_heads_kv <= 0 || a->n_heads_q % a->n_heads_kv)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "flash_attention_prefill: heads %d/%d", a->n_heads_q, a->n_heads_kv);
+  if (a->seq_len <= 0 || a->batch_size <= 0 || a->cache_seq_len < a->seq_len || a->cache_seq_len > a->kv_capacity ||
+      a->window < 0)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "flash_attention_prefill: seq_len %d cache_seq_len %d capacity %d",
+                      a->seq_len, a->cache_seq_len, a->kv_capacity);
+  // Declined cases: the caller runs its CPU path (same set as cuda_pc.rs:851-860).
+  if (!a->is_head_major) return 0;
+  if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256) return 0;
+  if (a->kv_dtype != ARGUS_HIP_F16 && a->kv_dtype != ARGUS_HIP_F32) return 0;
+  if ((a->q_dtype != ARGUS_HIP_F16 && a->q_dtype != ARGUS_HIP_F32) ||
+      (a->out_dtype != ARGUS_HIP_F16 && a->out_dtype != ARGUS_HIP_F32))
+    return 0;
+  if (((uintptr_t)a->q | (uintptr_t)a->k_cache | (uintptr_t)a->v_cache | (uintptr_t)a->out) & 15)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "flash_attention_prefill: tensors must be 16-byte aligned");
+
+  PrefillParams p{};
+  p.q = a->q;
+  p.k = a->k_cache;
+  p.v = a->v_cache;
+  p.out = a->out;
+  p.n_heads_q = a->n_heads_q;
+  p.n_heads_kv = a->n_heads_kv;
+  p.group = a->n_heads_q / a->n_heads_kv;
+  p.seq_len = a->seq_len;
+  p.cache_len = a->cache_seq_len;
+  p.q_start = a->cache_seq_len - a->seq_len;
+  p.capacity = a->kv_capacity;
+  p.batch = a->batch_size;
+  p.window = a->window;
+  p.q_f16 = a->q_dtype == ARGUS_HIP_F16;
+  p.out_f16 = a->out_dtype == ARGUS_HIP_F16;
+  p.scale_log2e = 1.4426950408889634f / sqrtf((float)a->head_dim);
+  hipStream_t stream = (hipStream_t)a->stream;
+  return a->kv_dtype == ARGUS_HIP_F16 ? dispatch_dim<_Float16>(ctx, p, a->head_dim, stream)
+                                      : dispatch_dim<float>(ctx, p, a->head_dim, stream);
+}

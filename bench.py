@@ -86,6 +86,55 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
                 gbps_wall=nbytes / wall / 1e9, gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None)
 
 
+def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res_cap=128, res_f16=False,
+               rotate=8):
+    """BASELINE config 4: q_tokens = 8064 quantised + 128 residual tokens.  Blocks are synthetic
+    (random codes, f16 scale/min headers); `rotate` block sets are cycled."""
+    import torch
+    q_tokens = (n_tokens - 1) // res_cap * res_cap
+    res_tokens = n_tokens - q_tokens
+    bb = 4 + 32 * bits // 8
+    nblk = q_tokens * hkv * d // 32
+    g = torch.Generator(device="cuda").manual_seed(4)
+
+    def blocks():
+        raw = torch.randint(0, 256, (nblk, bb), generator=g, device="cuda", dtype=torch.uint8)
+        hdr = torch.empty((nblk, 2), device="cuda", dtype=torch.float16)
+        hdr[:, 0] = 6.0 / (2 ** bits - 1)
+        hdr[:, 1] = -3.0
+        raw[:, :4] = hdr.view(torch.uint8)
+        return raw.reshape(-1)
+
+    sets = [(blocks(), blocks()) for _ in range(rotate)]
+    rdt = torch.float16 if res_f16 else torch.float32
+    res_k = torch.randn((hkv, res_cap, d), generator=g, device="cuda").to(rdt)
+    res_v = torch.randn((hkv, res_cap, d), generator=g, device="cuda").to(rdt)
+    q = torch.randn((hq, d), generator=g, device="cuda")
+    out = torch.empty((hq, d), device="cuda")
+    state = {"i": 0}
+
+    def step():
+        qk, qv = sets[state["i"] % rotate]
+        state["i"] += 1
+        ctx.attention_gen_quant(q, qk, qv, res_k, res_v, out, hkv, q_tokens, res_tokens, res_cap,
+                                1.0 / d ** 0.5, bits)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ctx.kernel_timing_begin(steps)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    kms = ctx.kernel_timing_end(steps)
+    nbytes = 2 * nblk * bb + 2 * hkv * res_tokens * d * (2 if res_f16 else 4) + hq * d * 4 * 2
+    kernel_ms = sum(kms) / max(len(kms), 1)
+    return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
+                gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9)
+
+
 def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
     """Restated CpuBackendAVX2::attention_gen on one sequence of the primary workload."""
     import numpy as np
@@ -180,6 +229,9 @@ def main():
         add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
             bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=4),
             "scores emitted; kernel time covers the split pass only")
+        add("cfg4_kivi_q4_L8192_res128_f32", bench_kivi(ctx, 4, es, ew), "8 block sets rotated; single launch, 11.4 MB")
+        add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")
+        add("cfg4_kivi_q4_L8192_res128_f16", bench_kivi(ctx, 4, es, ew, res_f16=True), "F16 residual window")
         line["extras"] = ex
 
     if not args.no_cpu:
