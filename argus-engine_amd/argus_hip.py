@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libargus_hip.so")
+# ARGUS_HIP_LIB selects another build of the same library (profiling / A-B runs).
+LIB_PATH = os.environ.get("ARGUS_HIP_LIB") or os.path.join(_HERE, "libargus_hip.so")
 
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_RUNTIME, ERR_NOMEM = 0, -1, -2, -3, -4
 F32, F16 = 0, 1

@@ -56,19 +56,28 @@ __device__ __forceinline__ half8_t load_kv_chunk<float>(const float *p) {
   return h;
 }
 
-template <int D, int HPW, typename KV_T>
-__global__ __launch_bounds__(256) void prefill_kernel(const PrefillParams p) {
-  constexpr int BN = (D <= 128) ? 64 : 32;   // keys per tile
+// Sizes of one staged K/V tile pair, shared by the kernel and the launcher.
+template <int D>
+struct PrefillTile {
+  static constexpr int BN = (D <= 128) ? 64 : 32;  // keys per tile
+  static constexpr int KP = D + 8;                 // K tile row pitch (halfs)
+  static constexpr int VP = BN + 4;                // V^T tile row pitch (halfs), keeps 8-byte alignment
+  static constexpr int HALFS = BN * KP + D * VP;   // halfs per (K, V^T) tile pair
+};
+
+template <int D, int HPW, int NG, typename KV_T>
+__global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p) {
+  using TL = PrefillTile<D>;
+  constexpr int BN = TL::BN, KP = TL::KP, VP = TL::VP;
+  constexpr int NT = 256 * NG;               // threads
   constexpr int QPW = 4 / HPW;               // 32-row query blocks per workgroup
-  constexpr int KP = D + 8;                  // K tile row pitch (halfs)
-  constexpr int VP = BN + 4;                 // V^T tile row pitch (halfs), keeps 8-byte alignment
   constexpr int KK = D / 16;                 // MFMA k-steps over head_dim
   constexpr int KB = BN / 32;                // S^T row blocks (32 keys each)
   constexpr int RB = D / 32;                 // O^T row blocks (32 channels each)
-  constexpr int CH = BN * D / 8 / 256;       // 16-byte chunks per thread per tile
+  constexpr int CH = NG * BN * D / 8 / NT;   // 16-byte chunks per thread per iteration
 
-  __shared__ __attribute__((aligned(16))) _Float16 sK[BN * KP];
-  __shared__ __attribute__((aligned(16))) _Float16 sVt[D * VP];
+  // [2 buffers][NG tiles][K tile | V^T tile]; reused at the end for the cross-group merge.
+  extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
 
   // ---- work decomposition ------------------------------------------------------------------
   const int pairs = p.batch * p.n_heads_kv;
@@ -77,18 +86,21 @@ __global__ __launch_bounds__(256) void prefill_kernel(const PrefillParams p) {
   const int b = pair / p.n_heads_kv, kvh = pair % p.n_heads_kv;
   const int gc = j % p.group_chunks;
   const int jt = j / p.group_chunks;
-  // long tiles first (descending), then the short ones ascending
-  const int half_t = (p.n_qtiles + 1) / 2;
-  const int qt = jt < half_t ? (p.n_qtiles - 1 - jt) : (jt - half_t);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kvg = wave / 4, wq = wave % 4;  // KV group of this wave, query-wave index
   const int ln = lane & 31, hl = lane >> 5;
-  const int h = kvh * p.group + min(gc * HPW + (wave % HPW), p.group - 1);
-  const bool head_ok = gc * HPW + (wave % HPW) < p.group;
-  const int qb = qt * QPW + wave / HPW;
+  const int h = kvh * p.group + gc * HPW + (wq % HPW);
+
+  // Causal work grows linearly with the query tile index, so each workgroup takes the pair
+  // (n_qtiles-1-jt, jt): every workgroup then carries the same number of key tiles.
+  for (int pass = 0; pass < 2; ++pass) {
+  const int qt = pass == 0 ? (p.n_qtiles - 1 - jt) : jt;
+  if (pass == 1 && qt == p.n_qtiles - 1 - jt) break;
+  const int qb = qt * QPW + wq / HPW;
   const int r0 = qb * 32;            // first query row of this wave
   const int row = r0 + ln;           // this lane's query row
-  const bool row_ok = head_ok && row < p.seq_len;
+  const bool row_ok = row < p.seq_len;
 
   // ---- Q as the B operand: lane (query ln, half hl) holds Q[row][16kk + 8hl .. +7] ----------
   half8_t qreg[KK];
@@ -118,18 +130,20 @@ __global__ __launch_bounds__(256) void prefill_kernel(const PrefillParams p) {
   int kv_begin = 0;
   if (p.window > 0) kv_begin = max(0, qt * QPW * 32 + p.q_start - p.window + 1);
   const int kt_begin = kv_begin / BN, kt_end = (kv_end + BN - 1) / BN;
+  const int n_it = (kt_end - kt_begin + NG - 1) / NG;
 
   const KV_T *kbase = (const KV_T *)p.k + ((int64_t)b * p.n_heads_kv + kvh) * p.capacity * D;
   const KV_T *vbase = (const KV_T *)p.v + ((int64_t)b * p.n_heads_kv + kvh) * p.capacity * D;
 
+  // Iteration `it` covers tiles kt_begin + it*NG + g for g < NG (tile g is consumed by KV group g).
   half8_t kpre[CH], vpre[CH];
-  auto fetch = [&](int kt) {
+  auto fetch = [&](int it) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int cid = threadIdx.x + 256 * c;
-      const int key = kt * BN + cid / (D / 8), dc = cid % (D / 8);
+      const int cid = threadIdx.x + NT * c;
+      const int key = (kt_begin + it * NG) * BN + cid / (D / 8), dc = cid % (D / 8);
       half8_t kx = {0, 0, 0, 0, 0, 0, 0, 0}, vx = kx;
-      if (key < p.cache_len) {
+      if (key < kv_end) {
         kx = load_kv_chunk<KV_T>(kbase + (int64_t)key * D + 8 * dc);
         vx = load_kv_chunk<KV_T>(vbase + (int64_t)key * D + 8 * dc);
       }
@@ -137,111 +151,155 @@ __global__ __launch_bounds__(256) void prefill_kernel(const PrefillParams p) {
       vpre[c] = vx;
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](int buf) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int cid = threadIdx.x + 256 * c;
-      const int key = cid / (D / 8), dc = cid % (D / 8);
+      const int cid = threadIdx.x + NT * c;
+      const int trow = cid / (D / 8), dc = cid % (D / 8);
+      const int g = trow / BN, key = trow % BN;
+      _Float16 *sK = smem + (buf * NG + g) * TL::HALFS;
+      _Float16 *sVt = sK + BN * KP;
       *(half8_t *)(sK + key * KP + 8 * dc) = kpre[c];
 #pragma unroll
       for (int e = 0; e < 8; ++e) sVt[(8 * dc + e) * VP + key] = vpre[c][e];
     }
   };
 
-  if (kt_begin < kt_end) fetch(kt_begin);
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    __syncthreads();  // every wave is done reading the previous tile
-    stage();
-    __syncthreads();
-    if (kt + 1 < kt_end) fetch(kt + 1);
+  if (n_it > 0) {
+    fetch(0);
+    stage(0);
+  }
+  __syncthreads();
+  for (int it = 0; it < n_it; ++it) {
+    if (it + 1 < n_it) fetch(it + 1);
 
+    const int kt = kt_begin + it * NG + kvg;
     const int key0 = kt * BN;
-    // Waves whose rows cannot see this tile skip the math (they still take part in the barriers).
+    // Waves whose rows cannot see their tile skip the math (they still take part in the barrier).
     const int wave_hi = r0 + 31 + p.q_start;  // largest visible key of the wave
     const int wave_lo = p.window > 0 ? (r0 + p.q_start - p.window + 1) : 0;
-    if (!head_ok || r0 >= p.seq_len || key0 > wave_hi || key0 + BN <= wave_lo) continue;
+    if (kt < kt_end && r0 < p.seq_len && key0 <= wave_hi && key0 + BN > wave_lo) {
+      const _Float16 *sK = smem + ((it & 1) * NG + kvg) * TL::HALFS;
+      const _Float16 *sVt = sK + BN * KP;
 
-    // ---- S^T = K . Q^T ------------------------------------------------------------------------
-    float16_t s_acc[KB];
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s_acc[kb][i] = 0.0f;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
-        s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
-      }
-    }
-
-    // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) ---------
-    const int q_pos = row + p.q_start;
-    const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
-                           (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
-    if (need_mask) {
+      // ---- S^T = K . Q^T ----------------------------------------------------------------------
+      float16_t s_acc[KB];
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = key0 + 32 * kb + 8 * (i / 4) + 4 * hl + (i % 4);
-          bool ok = key <= q_pos && key < p.cache_len;
-          if (p.window > 0) ok = ok && (key + p.window > q_pos);
-          if (!ok) s_acc[kb][i] = kNegInf;
+        for (int i = 0; i < 16; ++i) s_acc[kb][i] = 0.0f;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
+          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
         }
+
+      // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) -------
+      const int q_pos = row + p.q_start;
+      const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
+                             (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
+      if (need_mask) {
+        const int lo = p.window > 0 ? q_pos - p.window : -1;  // keys <= lo are outside the window
+        const int hi = min(q_pos, p.cache_len - 1);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + 32 * kb + 8 * (i / 4) + 4 * hl + (i % 4);
+            s_acc[kb][i] = (key <= hi && key > lo) ? s_acc[kb][i] : kNegInf;
+          }
+      }
+
+      // ---- online softmax for this lane's query column --------------------------------------
+      float mt = kNegInf;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m_run, mt * p.scale_log2e);
+      const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+      m_run = m_new;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          s_acc[kb][i] = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][i], p.scale_log2e, -m_ref));
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
+      }
+
+      // ---- O^T += V^T . P^T ------------------------------------------------------------------
+      // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
+      // rounding cancels in the final normalisation.
+      float lsum = 0.0f;
+#pragma unroll
+      for (int jn = 0; jn < BN / 16; ++jn) {
+        half8_t pb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pb[e] = (_Float16)s_acc[jn / 2][8 * (jn % 2) + e];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const half2_t pr = {pb[e], pb[e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
+          lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
+        }
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+          const _Float16 *vrow = sVt + (32 * r + ln) * VP + 16 * jn + 4 * hl;
+          const half4_t lo = *(const half4_t *)vrow, hi = *(const half4_t *)(vrow + 8);
+          const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, o_acc[r], 0, 0, 0);
+        }
+      }
+      l_run = l_run * alpha + lsum;
     }
 
-    // ---- online softmax for this lane's query column ----------------------------------------
-    float mt = kNegInf;
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m_run, mt * p.scale_log2e);
-    const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-    m_run = m_new;
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        s_acc[kb][i] = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][i], p.scale_log2e, -m_ref));
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+    if (it + 1 < n_it) stage((it + 1) & 1);
+    __syncthreads();  // next buffer is filled; every wave is done with the current one
+  }
+
+  // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
+  l_run += __shfl_xor(l_run, 32, 64);
+  if constexpr (NG > 1) {
+    float *mrg = (float *)smem;  // [NG-1][4 query waves][RB*16 + 2][64 lanes]
+    constexpr int SLOTS = RB * 16 + 2;
+    if (kvg > 0) {
+      float *dst = mrg + ((kvg - 1) * 4 + wq) * SLOTS * 64 + lane;
 #pragma unroll
       for (int r = 0; r < RB; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
+        for (int i = 0; i < 16; ++i) dst[(r * 16 + i) * 64] = o_acc[r][i];
+      dst[RB * 16 * 64] = m_run;
+      dst[(RB * 16 + 1) * 64] = l_run;
     }
-
-    // ---- O^T += V^T . P^T --------------------------------------------------------------------
-    // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
-    // rounding cancels in the final normalisation.
-    float lsum = 0.0f;
+    __syncthreads();
+    if (kvg == 0) {
 #pragma unroll
-    for (int jn = 0; jn < BN / 16; ++jn) {
-      half8_t pb;
+    for (int g = 1; g < NG; ++g) {
+      const float *src = mrg + ((g - 1) * 4 + wq) * SLOTS * 64 + lane;
+      const float m_o = src[RB * 16 * 64], l_o = src[(RB * 16 + 1) * 64];
+      const float m_new = fmaxf(m_run, m_o);
+      const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+      const float fa = __builtin_amdgcn_exp2f(m_run - m_ref), fb = __builtin_amdgcn_exp2f(m_o - m_ref);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pb[e] = (_Float16)s_acc[jn / 2][8 * (jn % 2) + e];
+      for (int r = 0; r < RB; ++r)
 #pragma unroll
-      for (int e = 0; e < 8; e += 2) {
-        const half2_t pr = {pb[e], pb[e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
-        lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
-      }
-#pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        const _Float16 *vrow = sVt + (32 * r + ln) * VP + 16 * jn + 4 * hl;
-        const half4_t lo = *(const half4_t *)vrow, hi = *(const half4_t *)(vrow + 8);
-        const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, o_acc[r], 0, 0, 0);
-      }
+        for (int i = 0; i < 16; ++i) o_acc[r][i] = o_acc[r][i] * fa + src[(r * 16 + i) * 64] * fb;
+      l_run = l_run * fa + l_o * fb;
+      m_run = m_new;
     }
-    l_run = l_run * alpha + lsum;
+    }
   }
 
   // ---- normalise and store: lane = query row, registers = channels ---------------------------
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  if (!row_ok) return;
-  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+  if (row_ok && kvg == 0) {
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
   const int64_t ooff = (((int64_t)b * p.seq_len + row) * p.n_heads_q + h) * D;
 #pragma unroll
   for (int r = 0; r < RB; ++r)
@@ -257,21 +315,44 @@ __global__ __launch_bounds__(256) void prefill_kernel(const PrefillParams p) {
         *(float4_t *)((float *)p.out + ooff + d0) = o;
       }
     }
+  }
+  __syncthreads();  // the merge area is free again before the next pass stages tiles into it
+  }  // pass
+}
+
+template <int D, int HPW, int NG, typename KV_T>
+int launch_ng(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream, size_t lds_bytes) {
+  constexpr int QPW = 4 / HPW;
+  p.n_qtiles = (p.seq_len + 32 * QPW - 1) / (32 * QPW);
+  p.group_chunks = p.group / HPW;
+  const int64_t wgs = (int64_t)p.batch * p.n_heads_kv * p.group_chunks * ((p.n_qtiles + 1) / 2);
+  if (wgs > 0x7fffffff) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: grid too large");
+  auto kern = prefill_kernel<D, HPW, NG, KV_T>;
+  static bool attr_set = false;  // per instantiation; single inference thread
+  if (!attr_set && lds_bytes > 48 * 1024) {
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    attr_set = true;
+  }
+  {
+    KernelTimer timer(ctx, stream);
+    hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(256 * NG), lds_bytes, stream, p);
+  }
+  ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  return 1;  // dispatched
 }
 
 template <int D, int HPW, typename KV_T>
 int launch(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
-  constexpr int QPW = 4 / HPW;
-  p.n_qtiles = (p.seq_len + 32 * QPW - 1) / (32 * QPW);
-  p.group_chunks = (p.group + HPW - 1) / HPW;
-  const int64_t wgs = (int64_t)p.batch * p.n_heads_kv * p.group_chunks * p.n_qtiles;
-  if (wgs > 0x7fffffff) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: grid too large");
-  {
-    KernelTimer timer(ctx, stream);
-    hipLaunchKernelGGL((prefill_kernel<D, HPW, KV_T>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  // KV groups split the serial chain of key tiles of a query block over 4*NG waves.  Two groups
+  // (8 waves, <= 256 VGPRs each) measured best; four groups need a 128-VGPR cap that spills.
+  const size_t tile_bytes = (size_t)PrefillTile<D>::HALFS * sizeof(_Float16);
+  const size_t lds_limit = ctx->props.sharedMemPerBlock;
+  if constexpr (D <= 128) {
+    if (2 * 2 * tile_bytes <= lds_limit) return launch_ng<D, HPW, 2, KV_T>(ctx, p, stream, 2 * 2 * tile_bytes);
   }
-  ARGUS_HIP_CHECK(ctx, hipGetLastError());
-  return 1;  // dispatched
+  if (2 * tile_bytes > lds_limit)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: %zu bytes of LDS needed, %zu available", 2 * tile_bytes, lds_limit);
+  return launch_ng<D, HPW, 1, KV_T>(ctx, p, stream, 2 * tile_bytes);
 }
 
 template <int D, typename KV_T>

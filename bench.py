@@ -135,6 +135,38 @@ def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res
                 gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9)
 
 
+def bench_prefill(ctx, steps, warmup, hq=32, hkv=8, d=64, s=2048, batch=1, f16_io=True):
+    """BASELINE config 2: causal GQA prefill; FLOPs use the causal count 4*Hq*d*S(S+1)/2."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(42)
+    io = torch.float16 if f16_io else torch.float32
+    q = torch.randn((batch, s, hq, d), generator=g, device="cuda").to(io)
+    k = torch.randn((batch, hkv, s, d), generator=g, device="cuda").half()
+    v = torch.randn((batch, hkv, s, d), generator=g, device="cuda").half()
+    out = torch.empty((batch, s, hq, d), device="cuda", dtype=io)
+
+    def step():
+        rc = ctx.flash_attention_prefill(q, k, v, out, hq, hkv, s, s, d, s, batch_size=batch)
+        assert rc == 1
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ctx.kernel_timing_begin(steps)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    kms = ctx.kernel_timing_end(steps)
+    kernel_ms = sum(kms) / max(len(kms), 1)
+    flops = 4 * hq * d * s * (s + 1) // 2 * batch
+    return dict(us_per_call=round(wall * 1e6, 2), kernel_us=round(kernel_ms * 1e3, 2), causal_flops=flops,
+                tflops_kernel=round(flops / (kernel_ms * 1e-3) / 1e12, 1),
+                mfma_frac_kernel=round(flops / (kernel_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                tflops_wall=round(flops / wall / 1e12, 1))
+
+
 def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
     """Restated CpuBackendAVX2::attention_gen on one sequence of the primary workload."""
     import numpy as np
@@ -168,6 +200,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", default="primary",
+                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5"],
+                    help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (every box has one GPU; the path shards by "
@@ -181,6 +216,22 @@ def main():
         sys.exit(1)
     ctx = argus_hip.Context(0)
     info = ctx.device_info()
+
+    if args.workload != "primary":
+        w = args.workload
+        if w == "decode_b1":
+            res = bench_decode(ctx, 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=4)
+        elif w == "prefill":
+            res = bench_prefill(ctx, args.steps, args.warmup)
+        elif w == "prefill_d128":
+            res = bench_prefill(ctx, args.steps, args.warmup, hq=32, hkv=8, d=128, s=8192)
+        elif w == "cfg5":
+            res = bench_decode(ctx, 8, 4, 256, 2048, 8, args.steps, args.warmup, capacity=4096, scores=True,
+                               softcap=50.0, rotate=4)
+        else:
+            res = bench_kivi(ctx, 4 if w == "kivi_q4" else 8, args.steps, args.warmup)
+        print(json.dumps({"workload": w, "steps": args.steps, "warmup": args.warmup, "result": res}))
+        return
 
     hq, hkv, d, L, batch = 32, 8, 128, 32768, 16
     r = bench_decode(ctx, hq, hkv, d, L, batch, args.steps, args.warmup)
@@ -232,6 +283,9 @@ def main():
         add("cfg4_kivi_q4_L8192_res128_f32", bench_kivi(ctx, 4, es, ew), "8 block sets rotated; single launch, 11.4 MB")
         add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")
         add("cfg4_kivi_q4_L8192_res128_f16", bench_kivi(ctx, 4, es, ew, res_f16=True), "F16 residual window")
+        ex["cfg2_prefill_llama1b_S2048_f16"] = bench_prefill(ctx, es, ew)
+        ex["cfg2_prefill_llama1b_S2048_f32io"] = bench_prefill(ctx, es, ew, f16_io=False)
+        ex["prefill_llama8b_d128_S8192_f16"] = bench_prefill(ctx, max(5, es // 4), 2, hq=32, hkv=8, d=128, s=8192)
         line["extras"] = ex
 
     if not args.no_cpu:
