@@ -82,7 +82,9 @@ class QuantAttnArgs(C.Structure):
 
 class QuantAttnExt(C.Structure):
     _fields_ = [("scores_dev", C.c_uint64), ("score_stride", C.c_size_t),
-                ("res_dtype", C.c_int32), ("softcap", C.c_float)]
+                ("res_dtype", C.c_int32), ("softcap", C.c_float), ("batch", C.c_int32),
+                ("block_batch_stride_bytes", C.c_int64), ("res_batch_stride", C.c_int64),
+                ("score_batch_stride", C.c_int64)]
 
 
 class QuantGatherArgs(C.Structure):
@@ -247,11 +249,12 @@ class Context:
 
     def attention_gen_quant(self, q, qk, qv, res_k, res_v, out, num_heads_kv, q_tokens, res_tokens,
                             res_cap, scale, bits, scores_host=None, scores_dev=None,
-                            score_stride=0, softcap=0.0, check=True):
+                            score_stride=0, softcap=0.0, batch=1, block_batch_stride_bytes=0,
+                            res_batch_stride=0, check=True):
         """scores_host: numpy float32 array (host readback, reference contract);
         scores_dev: torch tensor (device)."""
         import torch
-        hq, d = q.shape
+        hq, d = q.shape[-2], q.shape[-1]
         a = QuantAttnArgs(
             stream=_stream(), q_mem=_ptr(q), qk_mem=_ptr(qk), qv_mem=_ptr(qv),
             res_k_mem=_ptr(res_k), res_v_mem=_ptr(res_v), out_mem=_ptr(out),
@@ -260,10 +263,12 @@ class Context:
             num_heads_kv=num_heads_kv, head_dim=d, q_tokens=q_tokens, res_tokens=res_tokens,
             res_cap=res_cap, scale=scale, bits=bits)
         res_dtype = F16 if res_k.dtype == torch.float16 else F32
-        if scores_dev is None and res_dtype == F32 and softcap == 0.0:
+        if scores_dev is None and res_dtype == F32 and softcap == 0.0 and batch == 1:
             return self._check(lib.argus_hip_attention_gen_quant(self.handle, C.byref(a)), check)
         e = QuantAttnExt(scores_dev=_ptr(scores_dev), score_stride=score_stride,
-                         res_dtype=res_dtype, softcap=softcap)
+                         res_dtype=res_dtype, softcap=softcap, batch=batch,
+                         block_batch_stride_bytes=block_batch_stride_bytes,
+                         res_batch_stride=res_batch_stride, score_batch_stride=0)
         return self._check(lib.argus_hip_attention_gen_quant_ex(self.handle, C.byref(a), C.byref(e)), check)
 
     def gather_update_quant(self, inp, residual, kv_heads, res_cap, head_dim, seq_len, res_pos,

@@ -35,6 +35,8 @@ struct KiviParams {
   int32_t head_dim, q_tokens, res_tokens, res_cap;
   int32_t units_total, units_per_split;
   int32_t res_f16;
+  int64_t qk_bs, qv_bs;  // bytes between consecutive sequences' block streams
+  int64_t res_bs;        // elements between consecutive sequences' residual windows
 };
 
 template <int BITS>
@@ -54,8 +56,11 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
   constexpr int MAXD = 256;
   const DecodeParams &p = kp.d;
   const int D = kp.head_dim;
-  const int split = blockIdx.x, kvh = blockIdx.y;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x;
+  const uint8_t *qk_b = kp.qk + (int64_t)b * kp.qk_bs;
+  const uint8_t *qv_b = kp.qv + (int64_t)b * kp.qv_bs;
+  const int64_t res_off = (int64_t)b * kp.res_bs;
   const int gpf = kp.res_cap / kUnit;   // K groups per flush
   const int bpt = D / kUnit;            // V blocks per token
   const int q_units = kp.q_tokens / kUnit;
@@ -70,7 +75,7 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
   for (int i = tid; i < D * GT; i += 256) {
     const int ch = i / GT, g = i % GT;
     const int h = kvh * p.group + min(g, p.group - 1);
-    sh_q[ch][g] = p.q[(int64_t)h * D + ch] * p.scale;
+    sh_q[ch][g] = p.q[(int64_t)b * p.q_bs + (int64_t)h * D + ch] * p.scale;
   }
   if (tid < GT) {
     sh_m[tid] = kNegInf;
@@ -102,12 +107,12 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
       // K tile: blocks (flush, kvh, gif, ch = 0..D) are contiguous (kivi_attn.cu:256-262).
       const int flush = u / gpf, gif = u % gpf;
       const int64_t kblk = ((int64_t)flush * p.n_heads_kv * gpf + (int64_t)kvh * gpf + gif) * D;
-      const uint32_t *ksrc = (const uint32_t *)(kp.qk + kblk * BB);
+      const uint32_t *ksrc = (const uint32_t *)(qk_b + kblk * BB);
       for (int i = tid; i < D * BB / 4; i += 256) ((uint32_t *)sh_k)[i] = __builtin_nontemporal_load(ksrc + i);
       // V tile: blocks (flush, kvh, tif, b) with tif = 32 consecutive tokens (kivi_attn.cu:357-361).
       const int tif0 = (u * kUnit) % kp.res_cap;
       const int64_t vblk = (((int64_t)flush * p.n_heads_kv + kvh) * kp.res_cap + tif0) * bpt;
-      const uint32_t *vsrc = (const uint32_t *)(kp.qv + vblk * BB);
+      const uint32_t *vsrc = (const uint32_t *)(qv_b + vblk * BB);
       for (int i = tid; i < kUnit * bpt * BB / 4; i += 256) ((uint32_t *)sh_v)[i] = __builtin_nontemporal_load(vsrc + i);
     }
     __syncthreads();
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
         }
       } else if (kt < n_valid) {
         const int rt = (u - q_units) * kUnit + kt;
-        const int64_t rbase = ((int64_t)kvh * kp.res_cap + rt) * D + kcp * kch;
+        const int64_t rbase = res_off + ((int64_t)kvh * kp.res_cap + rt) * D + kcp * kch;
         for (int c = 0; c < kch; ++c) {
           const float x = load_res(kp.res_k, rbase + c, kp.res_f16);
 #pragma unroll
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
       }
       if (t >= n_valid) sv = kNegInf;
       if (p.scores && g < p.group && t < n_valid)
-        p.scores[(int64_t)(kvh * p.group + g) * p.score_stride + tok0 + t] = sv;
+        p.scores[(int64_t)b * p.score_bs + (int64_t)(kvh * p.group + g) * p.score_stride + tok0 + t] = sv;
       const float m_old = sh_m[g];
       const float m_new = fmaxf(m_old, group_allreduce_max<32>(sv));
       const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
         const int t = vtp * vtok + tt;
         if (t < n_valid) {
           const int rt = (u - q_units) * kUnit + t;
-          const float x = load_res(kp.res_v, ((int64_t)kvh * kp.res_cap + rt) * D + vc, kp.res_f16);
+          const float x = load_res(kp.res_v, res_off + ((int64_t)kvh * kp.res_cap + rt) * D + vc, kp.res_f16);
 #pragma unroll
           for (int g = 0; g < GT; ++g) acc[g] = fmaf(sh_p[t][g], x, acc[g]);
         }
@@ -211,7 +216,7 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
       float o = acc[g];
       for (int tp = 1; tp < vparts; ++tp) o += red[(tp * GT + g) * D + vc];
       const int h = kvh * p.group + g;
-      const int64_t pidx = (int64_t)h * p.nsplit + split;
+      const int64_t pidx = ((int64_t)b * p.n_heads_q + h) * p.nsplit + split;
       p.ws_o[pidx * D + vc] = o;
       if (vc == 0) {
         p.ws_ml[pidx * 2 + 0] = sh_m[g];
@@ -314,23 +319,24 @@ __global__ __launch_bounds__(128) void kivi_flush_v_kernel(const float *__restri
 }
 
 template <int BITS>
-int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, hipStream_t stream) {
+int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   DecodeParams &p = kp.d;
   const int D = kp.head_dim;
   const int target_wgs = ctx->compute_units * 4;
-  int nsplit = std::max(1, std::min({(target_wgs + p.n_heads_kv - 1) / p.n_heads_kv, kp.units_total, kMaxSplits}));
+  const int pairs = p.n_heads_kv * batch;
+  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, kp.units_total, kMaxSplits}));
   kp.units_per_split = (kp.units_total + nsplit - 1) / nsplit;
   nsplit = (kp.units_total + kp.units_per_split - 1) / kp.units_per_split;
   p.nsplit = nsplit;
   p.direct = 0;
-  const size_t n_part = (size_t)p.n_heads_q * nsplit;
+  const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
   const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
   int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
   if (rc != ARGUS_HIP_OK) return rc;
   p.ws_ml = ctx->ws;
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
 
-  dim3 grid(nsplit, p.n_heads_kv);
+  dim3 grid(nsplit, p.n_heads_kv, batch);
   {
     KernelTimer timer(ctx, stream);
     if (p.group <= 1) hipLaunchKernelGGL((kivi_split_kernel<BITS, 1>), grid, dim3(256), 0, stream, kp);
@@ -340,9 +346,9 @@ int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, hipStream_t stream) {
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   switch (D) {
-    case 64: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 64>), dim3(p.n_heads_q, 1), dim3(256), 0, stream, p); break;
-    case 128: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 128>), dim3(p.n_heads_q, 1), dim3(256), 0, stream, p); break;
-    default: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 256>), dim3(p.n_heads_q, 1), dim3(256), 0, stream, p); break;
+    case 64: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 64>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p); break;
+    case 128: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 128>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 256>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p); break;
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
@@ -423,12 +429,23 @@ ARGUS_API int argus_hip_attention_gen_quant_ex(argus_hip_ctx *ctx, const argus_h
   kp.res_cap = (int32_t)a->res_cap;
   kp.res_f16 = (ext && ext->res_dtype == ARGUS_HIP_F16) ? 1 : 0;
   kp.units_total = (int32_t)(a->q_tokens / kUnit + (a->res_tokens + kUnit - 1) / kUnit);
+  const int batch = (ext && ext->batch > 1) ? ext->batch : 1;
+  if (batch > 1) {
+    if (want_host) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_quant: host score read-back is single-sequence");
+    if (batch > 65535) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_quant: batch beyond grid limits");
+    if ((ext->block_batch_stride_bytes & 3) || (a->q_tokens && ext->block_batch_stride_bytes == 0) ||
+        (a->res_tokens && ext->res_batch_stride == 0))
+      return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen_quant: batch strides");
+    kp.qk_bs = kp.qv_bs = ext->block_batch_stride_bytes;
+    kp.res_bs = ext->res_batch_stride;
+    p.score_bs = ext->score_batch_stride ? ext->score_batch_stride : (int64_t)a->num_heads_q * stride;
+  }
 
   int rc;
   switch (a->bits) {
-    case 2: rc = launch_kivi<2>(ctx, kp, stream); break;
-    case 4: rc = launch_kivi<4>(ctx, kp, stream); break;
-    default: rc = launch_kivi<8>(ctx, kp, stream); break;
+    case 2: rc = launch_kivi<2>(ctx, kp, batch, stream); break;
+    case 4: rc = launch_kivi<4>(ctx, kp, batch, stream); break;
+    default: rc = launch_kivi<8>(ctx, kp, batch, stream); break;
   }
   if (rc == ARGUS_HIP_OK && want_host) {
     // Blocking read-back into the host slice (gpu_kivi_cuda.rs:204-212).

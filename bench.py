@@ -87,14 +87,16 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
 
 
 def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res_cap=128, res_f16=False,
-               rotate=8):
+               rotate=8, batch=1):
     """BASELINE config 4: q_tokens = 8064 quantised + 128 residual tokens.  Blocks are synthetic
-    (random codes, f16 scale/min headers); `rotate` block sets are cycled."""
+    (random codes, f16 scale/min headers); `rotate` block sets are cycled.  batch > 1 runs that many
+    caches (e.g. the layers of a model) in one launch so the rate is not launch-latency bound."""
     import torch
     q_tokens = (n_tokens - 1) // res_cap * res_cap
     res_tokens = n_tokens - q_tokens
     bb = 4 + 32 * bits // 8
-    nblk = q_tokens * hkv * d // 32
+    nblk1 = q_tokens * hkv * d // 32
+    nblk = nblk1 * batch
     g = torch.Generator(device="cuda").manual_seed(4)
 
     def blocks():
@@ -107,17 +109,18 @@ def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res
 
     sets = [(blocks(), blocks()) for _ in range(rotate)]
     rdt = torch.float16 if res_f16 else torch.float32
-    res_k = torch.randn((hkv, res_cap, d), generator=g, device="cuda").to(rdt)
-    res_v = torch.randn((hkv, res_cap, d), generator=g, device="cuda").to(rdt)
-    q = torch.randn((hq, d), generator=g, device="cuda")
-    out = torch.empty((hq, d), device="cuda")
+    res_k = torch.randn((batch, hkv, res_cap, d), generator=g, device="cuda").to(rdt)
+    res_v = torch.randn((batch, hkv, res_cap, d), generator=g, device="cuda").to(rdt)
+    q = torch.randn((batch, hq, d), generator=g, device="cuda")
+    out = torch.empty((batch, hq, d), device="cuda")
     state = {"i": 0}
 
     def step():
         qk, qv = sets[state["i"] % rotate]
         state["i"] += 1
         ctx.attention_gen_quant(q, qk, qv, res_k, res_v, out, hkv, q_tokens, res_tokens, res_cap,
-                                1.0 / d ** 0.5, bits)
+                                1.0 / d ** 0.5, bits, batch=batch, block_batch_stride_bytes=nblk1 * bb,
+                                res_batch_stride=hkv * res_cap * d)
 
     for _ in range(warmup):
         step()
@@ -129,7 +132,7 @@ def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     kms = ctx.kernel_timing_end(steps)
-    nbytes = 2 * nblk * bb + 2 * hkv * res_tokens * d * (2 if res_f16 else 4) + hq * d * 4 * 2
+    nbytes = 2 * nblk * bb + batch * (2 * hkv * res_tokens * d * (2 if res_f16 else 4) + hq * d * 4 * 2)
     kernel_ms = sum(kms) / max(len(kms), 1)
     return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
                 gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9)
@@ -229,7 +232,7 @@ def main():
             res = bench_decode(ctx, 8, 4, 256, 2048, 8, args.steps, args.warmup, capacity=4096, scores=True,
                                softcap=50.0, rotate=4)
         else:
-            res = bench_kivi(ctx, 4 if w == "kivi_q4" else 8, args.steps, args.warmup)
+            res = bench_kivi(ctx, 4 if w == "kivi_q4" else 8, args.steps, args.warmup, batch=32, rotate=2)
         print(json.dumps({"workload": w, "steps": args.steps, "warmup": args.warmup, "result": res}))
         return
 
@@ -283,6 +286,10 @@ def main():
         add("cfg4_kivi_q4_L8192_res128_f32", bench_kivi(ctx, 4, es, ew), "8 block sets rotated; single launch, 11.4 MB")
         add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")
         add("cfg4_kivi_q4_L8192_res128_f16", bench_kivi(ctx, 4, es, ew, res_f16=True), "F16 residual window")
+        add("cfg4_kivi_q4_x32_caches", bench_kivi(ctx, 4, es, ew, batch=32, rotate=2),
+            "32 caches (layers) per launch, 365 MB: amortised rate")
+        add("cfg4_kivi_q8_x32_caches", bench_kivi(ctx, 8, es, ew, batch=32, rotate=2),
+            "32 caches (layers) per launch, 629 MB: amortised rate")
         ex["cfg2_prefill_llama1b_S2048_f16"] = bench_prefill(ctx, es, ew)
         ex["cfg2_prefill_llama1b_S2048_f32io"] = bench_prefill(ctx, es, ew, f16_io=False)
         ex["prefill_llama8b_d128_S8192_f16"] = bench_prefill(ctx, max(5, es // 4), 2, hq=32, hkv=8, d=128, s=8192)

@@ -191,6 +191,13 @@ typedef struct argus_hip_quant_attn_ext {
   size_t score_stride;
   int32_t res_dtype;     /* ARGUS_HIP_F32 (reference, engine/src/kv/quant_window_cache.rs:171-177) or ARGUS_HIP_F16 */
   float softcap;
+  /* `batch` > 1: that many independent caches (sequences or layers) of identical geometry in one
+   * launch; Q / out are [batch, num_heads_q, head_dim], block streams and residual windows sit at
+   * the strides below.  The reference issues one call per cache. */
+  int32_t batch;
+  int64_t block_batch_stride_bytes; /* between consecutive qk (and qv) block streams */
+  int64_t res_batch_stride;         /* elements between consecutive residual windows */
+  int64_t score_batch_stride;       /* elements; 0 = num_heads_q * score_stride */
 } argus_hip_quant_attn_ext;
 
 /* CudaQuantAttnBackend::{has_quant_attn_kernel, attention_gen_quant, gather_update_quant},

@@ -135,6 +135,31 @@ def test_config4_llama8b_kivi(bits):
     check_attention_out(out16, ref16)
 
 
+def test_batched_caches_match_single_calls():
+    # several caches (sequences / layers) of one geometry in a single launch == one call each
+    import torch
+    nb, hq, hkv, d, R, n, bits = 3, 8, 2, 128, 64, 64 * 3 + 9, 4
+    rng = np.random.default_rng(77)
+    caches = [O.kivi_build(rng.standard_normal((n, hkv, d)).astype(np.float32),
+                           rng.standard_normal((n, hkv, d)).astype(np.float32), R, bits) for _ in range(nb)]
+    q = rng.standard_normal((nb, hq, d)).astype(np.float32)
+    nbytes = caches[0]["qk"].size
+    qk = dev(np.stack([c["qk"] for c in caches]))
+    qv = dev(np.stack([c["qv"] for c in caches]))
+    rk = dev(np.stack([c["res_k"] for c in caches]))
+    rv = dev(np.stack([c["res_v"] for c in caches]))
+    out = torch.empty((nb, hq, d), device="cuda")
+    total = caches[0]["q_tokens"] + caches[0]["res_tokens"]
+    sc = torch.zeros((nb, hq, total), device="cuda")
+    ctx().attention_gen_quant(dev(q), qk, qv, rk, rv, out, hkv, caches[0]["q_tokens"], caches[0]["res_tokens"], R,
+                              1.0 / np.sqrt(d), bits, scores_dev=sc, score_stride=total, batch=nb,
+                              block_batch_stride_bytes=nbytes, res_batch_stride=hkv * R * d)
+    for i, c in enumerate(caches):
+        ref, p = O.kivi_attention(q[i], c, 1.0 / np.sqrt(d), scores=True)
+        check_attention_out(host(out)[i], ref, "cache %d" % i)
+        check_scores(host(sc)[i], p, "cache %d" % i)
+
+
 def test_gather_update_and_flush_bit_exact():
     # Drive the container on the device: append tokens through gather_update_quant, quantise a
     # full residual with quant_flush, and compare blocks bit for bit with the CPU container
