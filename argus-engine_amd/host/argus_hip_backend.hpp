@@ -1,0 +1,351 @@
+// Host-side mirror of the engine interfaces the attention path goes through, written above the
+// C ABI of include/argus_hip.h.  Same method names, argument meaning and error behaviour as the
+// reference traits, so a test written against the reference reads the same here:
+//   HipBackend             ~ `trait Backend`            engine/src/backend.rs:127-1360 (hot-path subset)
+//   HipQuantAttnBackend    ~ `CudaQuantAttnBackend`     crates/argus-extension-api/src/lib.rs:3087-3104
+//   HipScoreReduceBackend  ~ `CudaScoreReduceBackend`   crates/argus-extension-api/src/lib.rs:2938-2948
+//   HipGpuScoreAccumulator ~ `CudaGpuScoreAccumulator`  engine/src/backend/cuda_pc/gpu_score.rs:72-403
+// `Result<T>` stands in for anyhow::Result<T>: ok() / value() / error().
+// Everything runs on the single inference thread and the single in-order stream (null = default),
+// like the reference backends.  Header-only; links against libargus_hip.so.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <memory>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/argus_hip.h"
+
+namespace argus {
+
+template <typename T>
+class Result {
+ public:
+  static Result Ok(T v) { Result r; r.ok_ = true; r.value_ = std::move(v); return r; }
+  static Result Err(std::string msg) { Result r; r.ok_ = false; r.error_ = std::move(msg); return r; }
+  bool ok() const { return ok_; }
+  const T &value() const { return value_; }
+  T &value() { return value_; }
+  const std::string &error() const { return error_; }
+
+ private:
+  bool ok_ = false;
+  T value_{};
+  std::string error_;
+};
+struct Unit {};
+using Status = Result<Unit>;
+inline Status OkStatus() { return Status::Ok(Unit{}); }
+
+// DType subset of engine/src/buffer.rs:25-47.
+enum class DType { F32 = ARGUS_HIP_F32, F16 = ARGUS_HIP_F16, Q4_0 = 100 };
+
+// A tensor is a shape over a lent buffer (engine/src/tensor.rs:8-58); `device` tells whether the
+// pointer is a device pointer of this backend (a `Buffer` of another backend has none).
+struct Tensor {
+  void *ptr = nullptr;
+  DType dtype = DType::F32;
+  std::vector<size_t> dims;
+  bool device = true;
+};
+
+class HipGpuScoreAccumulator;
+
+class HipBackend {
+ public:
+  // Counterpart of the "hip" arm of engine/src/session/init.rs:203-468.
+  static Result<std::shared_ptr<HipBackend>> create(int device = 0) {
+    argus_hip_ctx *ctx = nullptr;
+    const int rc = argus_hip_create(device, &ctx);
+    if (rc != ARGUS_HIP_OK) return Result<std::shared_ptr<HipBackend>>::Err("argus_hip_create failed: code " + std::to_string(rc));
+    return Result<std::shared_ptr<HipBackend>>::Ok(std::shared_ptr<HipBackend>(new HipBackend(ctx)));
+  }
+  ~HipBackend();
+  HipBackend(const HipBackend &) = delete;
+  HipBackend &operator=(const HipBackend &) = delete;
+
+  const char *name() const { return "HIP"; }
+  bool is_gpu() const { return true; }
+  bool is_discrete_gpu() const { return true; }
+  bool is_nosub_device() const { return true; }
+  bool supports_kv_scatter_batch() const { return true; }
+  argus_hip_ctx *ctx() const { return ctx_; }
+
+  // ---- memory (Backend::{read_buffer, write_buffer, copy_slice, synchronize}) ---------------
+  Result<void *> alloc(size_t bytes) {
+    void *p = nullptr;
+    if (argus_hip_malloc(ctx_, bytes, &p) != ARGUS_HIP_OK) return Result<void *>::Err(last_error());
+    return Result<void *>::Ok(p);
+  }
+  Status free(void *p) { return wrap(argus_hip_free(ctx_, p)); }
+  Status write_buffer(void *dst_dev, const void *src_host, size_t bytes) { return wrap(argus_hip_write_buffer(ctx_, nullptr, dst_dev, src_host, bytes)); }
+  Status read_buffer(void *dst_host, const void *src_dev, size_t bytes) { return wrap(argus_hip_read_buffer(ctx_, nullptr, dst_host, src_dev, bytes)); }
+  Status copy_slice(void *dst_dev, const void *src_dev, size_t bytes) { return wrap(argus_hip_copy_slice(ctx_, nullptr, dst_dev, src_dev, bytes)); }
+  Status synchronize() { return wrap(argus_hip_synchronize(ctx_, nullptr)); }
+
+  // ---- Backend::attention_gen (engine/src/backend.rs:284-295) ---------------------------------
+  // `scores_out` is a HOST slice of `scores_len` floats or null; stride = scores_len / num_heads_q;
+  // on return the slice is valid (explicit synchronize + copy-back, cuda_pc.rs:1861-1880).  When the
+  // GPU score accumulator is active its per-layer device slice takes precedence and nothing is
+  // copied back (cuda_pc.rs:1750-1766).  A malformed slice (stride < cache_seq_len) disables the
+  // export instead of failing (cuda_pc.rs:1776-1779).
+  Status attention_gen(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,
+                       size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
+                       float *scores_out, size_t scores_len);
+
+  // ---- Backend::flash_attention_prefill (engine/src/backend.rs:1011-1027) --------------------
+  // Ok(true) = dispatched, Ok(false) = not handled, caller uses its CPU path.
+  Result<bool> flash_attention_prefill(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,
+                                       size_t n_heads_q, size_t n_heads_kv, size_t seq_len, size_t cache_seq_len,
+                                       size_t head_dim, size_t kv_capacity, size_t batch_size, bool is_head_major) {
+    if (!q.device || !k_cache.device || !v_cache.device || !out.device) return Result<bool>::Ok(false);
+    if (k_cache.dtype == DType::Q4_0) return Result<bool>::Ok(false);
+    argus_hip_prefill_args a{};
+    a.q = q.ptr; a.k_cache = k_cache.ptr; a.v_cache = v_cache.ptr; a.out = out.ptr;
+    a.n_heads_q = (int32_t)n_heads_q; a.n_heads_kv = (int32_t)n_heads_kv; a.seq_len = (int32_t)seq_len;
+    a.cache_seq_len = (int32_t)cache_seq_len; a.head_dim = (int32_t)head_dim; a.kv_capacity = (int32_t)kv_capacity;
+    a.batch_size = (int32_t)batch_size; a.is_head_major = is_head_major ? 1 : 0;
+    a.q_dtype = (int32_t)q.dtype; a.kv_dtype = (int32_t)k_cache.dtype; a.out_dtype = (int32_t)out.dtype;
+    const int rc = argus_hip_flash_attention_prefill(ctx_, &a);
+    if (rc < 0) return Result<bool>::Err("flash_attn_prefill launch failed: " + last_error());
+    return Result<bool>::Ok(rc == 1);
+  }
+
+  // ---- Backend::kv_scatter_f32_to_f16 / _batch (engine/src/backend.rs:425-545) ----------------
+  Status kv_scatter_f32_to_f16(const Tensor &k_src, const Tensor &v_src, Tensor &k_dst, Tensor &v_dst,
+                               size_t head_dim, size_t capacity, size_t write_pos) {
+    const size_t kv_heads = k_dst.dims.size() >= 3 ? k_dst.dims[k_dst.dims.size() - 3] : 0;
+    return wrap(argus_hip_kv_scatter_f32_to_f16(ctx_, nullptr, (const float *)k_src.ptr, (const float *)v_src.ptr, k_dst.ptr,
+                                                v_dst.ptr, (int32_t)kv_heads, (int32_t)head_dim, (int32_t)capacity, (int32_t)write_pos));
+  }
+  Status kv_scatter_f32_to_f16_batch(const Tensor &k_src, const Tensor &v_src, Tensor &k_dst, Tensor &v_dst,
+                                     size_t kv_heads, size_t head_dim, size_t capacity, size_t write_pos_start, size_t seq_len) {
+    if (k_dst.dtype == DType::F32)
+      return wrap(argus_hip_kv_scatter_f32_batch(ctx_, nullptr, (const float *)k_src.ptr, (const float *)v_src.ptr, (float *)k_dst.ptr,
+                                                 (float *)v_dst.ptr, (int32_t)kv_heads, (int32_t)head_dim, (int32_t)capacity,
+                                                 (int32_t)write_pos_start, (int32_t)seq_len));
+    return wrap(argus_hip_kv_scatter_f32_to_f16_batch(ctx_, nullptr, (const float *)k_src.ptr, (const float *)v_src.ptr, k_dst.ptr,
+                                                      v_dst.ptr, (int32_t)kv_heads, (int32_t)head_dim, (int32_t)capacity,
+                                                      (int32_t)write_pos_start, (int32_t)seq_len));
+  }
+
+  // ---- GPU score accumulator (Backend::gpu_score_acc[_mut], engine/src/backend.rs:1312-1322) --
+  Status init_gpu_score_acc(size_t n_layers, size_t n_heads_q, size_t n_kv_heads, size_t max_seq_len, float decay);
+  HipGpuScoreAccumulator *gpu_score_acc() { return acc_.get(); }
+
+  std::string last_error() const { return argus_hip_last_error(ctx_); }
+  Status wrap(int rc) const { return rc == ARGUS_HIP_OK ? OkStatus() : Status::Err(last_error() + " (code " + std::to_string(rc) + ")"); }
+
+ private:
+  explicit HipBackend(argus_hip_ctx *ctx) : ctx_(ctx) {}
+  argus_hip_ctx *ctx_;
+  void *score_tmp_ = nullptr;  // reusable device score scratch (cuda_pc.rs `score_tmp_buf`)
+  size_t score_tmp_bytes_ = 0;
+  std::unique_ptr<HipGpuScoreAccumulator> acc_;
+};
+
+// CudaScoreReduceBackend twin: the args struct is the reference POD field for field.
+class HipScoreReduceBackend {
+ public:
+  explicit HipScoreReduceBackend(argus_hip_ctx *ctx) : ctx_(ctx) {}
+  const char *name() const { return "attn_score"; }
+  int reduce(const argus_hip_score_reduce_args &a) const { return ctx_ ? argus_hip_score_reduce(ctx_, &a) : -1; }
+  int reduce_per_layer(const argus_hip_score_reduce_args &a) const { return ctx_ ? argus_hip_score_reduce_per_layer(ctx_, &a) : -1; }
+
+ private:
+  argus_hip_ctx *ctx_;
+};
+
+// CudaQuantAttnBackend twin.  A handle built without a context is *degraded*: every op returns -1
+// without crashing (engine/tests/gate_c_kivi_backend_cap.rs:90-146).
+class HipQuantAttnBackend {
+ public:
+  explicit HipQuantAttnBackend(argus_hip_ctx *ctx) : ctx_(ctx) {}
+  bool has_quant_attn_kernel(uint8_t bits) const { return ctx_ && argus_hip_has_quant_attn_kernel(ctx_, bits) == 1; }
+  bool is_nosub_device() const { return true; }
+  int attention_gen_quant(const argus_hip_quant_attn_args &a) const { return ctx_ ? argus_hip_attention_gen_quant(ctx_, &a) : -1; }
+  int gather_update_quant(const argus_hip_quant_gather_args &a) const { return ctx_ ? argus_hip_gather_update_quant(ctx_, &a) : -1; }
+  // Q2 F16-view helpers are not built: the trait defaults return -1 (lib.rs:3096-3103).
+  int dequant_flush() const { return -1; }
+  int scatter_residual() const { return -1; }
+
+ private:
+  argus_hip_ctx *ctx_;
+};
+
+// CudaGpuScoreAccumulator twin (engine/src/backend/cuda_pc/gpu_score.rs:72-403): persistent device
+// buffers [n_layers, n_heads_q, max_seq_len] scores + cumulative flat / per-head importance; the
+// attention kernel writes each layer's slice, end_step() folds them with the fused reducer.
+class HipGpuScoreAccumulator {
+ public:
+  static Result<std::unique_ptr<HipGpuScoreAccumulator>> create(HipBackend *be, size_t n_layers, size_t n_heads_q,
+                                                                size_t n_kv_heads, size_t max_seq_len, float decay) {
+    using R = Result<std::unique_ptr<HipGpuScoreAccumulator>>;
+    if (n_kv_heads > 16) return R::Err("n_kv_heads exceeds the fused kernel limit of 16");
+    std::unique_ptr<HipGpuScoreAccumulator> a(new HipGpuScoreAccumulator(be));
+    a->n_layers_ = n_layers; a->n_heads_q_ = n_heads_q; a->n_kv_heads_ = n_kv_heads;
+    a->max_seq_len_ = max_seq_len; a->score_stride_ = max_seq_len;
+    const float f = 1.0f - decay;
+    a->decay_factor_ = f < 0.0f ? 0.0f : (f > 1.0f ? 1.0f : f);
+    auto alloc_zeroed = [&](size_t elems, void **out) -> bool {
+      auto r = be->alloc(elems * sizeof(float));
+      if (!r.ok()) return false;
+      *out = r.value();
+      std::vector<float> z(elems, 0.0f);
+      return be->write_buffer(*out, z.data(), elems * sizeof(float)).ok();
+    };
+    if (!alloc_zeroed(n_layers * n_heads_q * max_seq_len, &a->score_buf_) || !alloc_zeroed(max_seq_len, &a->importance_) ||
+        !alloc_zeroed(n_kv_heads * max_seq_len, &a->head_importance_) || !alloc_zeroed(n_layers * max_seq_len, &a->layer_flat_))
+      return R::Err("score buffer allocation failed: " + be->last_error());
+    return R::Ok(std::move(a));
+  }
+  ~HipGpuScoreAccumulator() {
+    for (void *p : {score_buf_, importance_, head_importance_, layer_flat_})
+      if (p) be_->free(p);
+  }
+
+  uint64_t score_buf_device_ptr() const { return (uint64_t)score_buf_; }
+  size_t score_stride() const { return score_stride_; }
+  size_t layer_offset_elems(size_t layer_idx) const { return layer_idx * n_heads_q_ * score_stride_; }
+  size_t current_layer_idx() const { return current_layer_idx_; }
+  void set_current_layer_idx(size_t i) { current_layer_idx_ = i; }
+  bool is_active() const { return active_; }
+  void set_active(bool a) { active_ = a; }
+  void enable_per_layer_flat() { per_layer_flat_ = true; }
+  size_t steps_accumulated() const { return steps_; }
+
+  Status end_step(void *stream, size_t cache_seq_len) {
+    if (!active_ || cache_seq_len == 0) return OkStatus();
+    argus_hip_score_reduce_args a{};
+    a.stream = stream;
+    a.score_buf = (uint64_t)score_buf_; a.importance = (uint64_t)importance_; a.head_importance = (uint64_t)head_importance_;
+    a.decay_factor = decay_factor_; a.n_layers = n_layers_; a.n_heads_q = n_heads_q_; a.n_kv_heads = n_kv_heads_;
+    a.cache_seq_len = cache_seq_len; a.score_stride = score_stride_; a.max_seq_len = max_seq_len_;
+    a.layer_flat_importance = (uint64_t)layer_flat_;
+    HipScoreReduceBackend reducer(be_->ctx());
+    int ret = reducer.reduce(a);
+    if (ret != 0) return Status::Err("attn_score HIP reduce failed: code " + std::to_string(ret));
+    if (per_layer_flat_) {
+      ret = reducer.reduce_per_layer(a);
+      if (ret != 0) return Status::Err("attn_score HIP per-layer reduce failed: code " + std::to_string(ret));
+    }
+    steps_ += 1;
+    current_layer_idx_ = 0;
+    return OkStatus();
+  }
+
+  Result<std::pair<std::vector<float>, std::vector<float>>> sync_to_cpu() const {
+    using R = Result<std::pair<std::vector<float>, std::vector<float>>>;
+    std::vector<float> flat(max_seq_len_), head(n_kv_heads_ * max_seq_len_);
+    if (!be_->read_buffer(flat.data(), importance_, flat.size() * 4).ok() ||
+        !be_->read_buffer(head.data(), head_importance_, head.size() * 4).ok())
+      return R::Err(be_->last_error());
+    return R::Ok({std::move(flat), std::move(head)});
+  }
+  Result<std::vector<float>> sync_layer_flat_to_cpu() const {
+    std::vector<float> lf(n_layers_ * max_seq_len_);
+    if (!be_->read_buffer(lf.data(), layer_flat_, lf.size() * 4).ok()) return Result<std::vector<float>>::Err(be_->last_error());
+    return Result<std::vector<float>>::Ok(std::move(lf));
+  }
+  Status seed_cumulative(const std::vector<float> &flat, const std::vector<float> &head) {
+    if (flat.size() != max_seq_len_) return Status::Err("seed_cumulative: flat.len() != max_seq_len");
+    if (head.size() != n_kv_heads_ * max_seq_len_) return Status::Err("seed_cumulative: head.len() != n_kv_heads*max_seq_len");
+    Status s = be_->write_buffer(importance_, flat.data(), flat.size() * 4);
+    if (!s.ok()) return s;
+    return be_->write_buffer(head_importance_, head.data(), head.size() * 4);
+  }
+  Status reset() {
+    std::vector<float> z(n_layers_ * max_seq_len_ > n_kv_heads_ * max_seq_len_ ? n_layers_ * max_seq_len_ : n_kv_heads_ * max_seq_len_, 0.0f);
+    Status s = be_->write_buffer(importance_, z.data(), max_seq_len_ * 4);
+    if (s.ok()) s = be_->write_buffer(head_importance_, z.data(), n_kv_heads_ * max_seq_len_ * 4);
+    if (s.ok()) s = be_->write_buffer(layer_flat_, z.data(), n_layers_ * max_seq_len_ * 4);
+    steps_ = 0;
+    current_layer_idx_ = 0;
+    return s;
+  }
+  // Test-only, like the reference's debug_fill_score_buf.
+  Status debug_fill_score_buf(const std::vector<float> &scores) {
+    if (scores.size() != n_layers_ * n_heads_q_ * score_stride_) return Status::Err("debug_fill_score_buf: wrong length");
+    return be_->write_buffer(score_buf_, scores.data(), scores.size() * 4);
+  }
+
+ private:
+  explicit HipGpuScoreAccumulator(HipBackend *be) : be_(be) {}
+  HipBackend *be_;
+  void *score_buf_ = nullptr, *importance_ = nullptr, *head_importance_ = nullptr, *layer_flat_ = nullptr;
+  size_t n_layers_ = 0, n_heads_q_ = 0, n_kv_heads_ = 0, max_seq_len_ = 0, score_stride_ = 0;
+  float decay_factor_ = 1.0f;
+  bool active_ = false, per_layer_flat_ = false;
+  size_t steps_ = 0, current_layer_idx_ = 0;
+};
+
+inline HipBackend::~HipBackend() {
+  acc_.reset();
+  if (score_tmp_) argus_hip_free(ctx_, score_tmp_);
+  argus_hip_destroy(ctx_);
+}
+
+inline Status HipBackend::init_gpu_score_acc(size_t n_layers, size_t n_heads_q, size_t n_kv_heads, size_t max_seq_len, float decay) {
+  auto r = HipGpuScoreAccumulator::create(this, n_layers, n_heads_q, n_kv_heads, max_seq_len, decay);
+  if (!r.ok()) return Status::Err(r.error());
+  acc_ = std::move(r.value());
+  return OkStatus();
+}
+
+inline Status HipBackend::attention_gen(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,
+                                        size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
+                                        float *scores_out, size_t scores_len) {
+  // The reference falls back to its CPU companion for non-device buffers and Q4_0 KV
+  // (cuda_pc.rs:1716-1729); this mirror has no CPU companion, so it reports the case.
+  if (!q.device || !k_cache.device || !v_cache.device || !out.device || k_cache.dtype == DType::Q4_0)
+    return Status::Err("attention_gen: not a device F32/F16 call; route to the CPU companion");
+  const std::vector<size_t> &kd = k_cache.dims;
+  // Layout rule of x86.rs:195-198.
+  const bool head_major = kd.size() >= 3 && kd[1] == num_heads_kv && kd[1] != kd[2];
+  argus_hip_attention_gen_args a{};
+  a.q = (const float *)q.ptr; a.k_cache = k_cache.ptr; a.v_cache = v_cache.ptr; a.out = (float *)out.ptr;
+  a.num_heads_q = (int32_t)num_heads_q; a.num_heads_kv = (int32_t)num_heads_kv; a.head_dim = (int32_t)head_dim;
+  a.cache_seq_len = (int32_t)cache_seq_len;
+  a.capacity = head_major ? (int32_t)kd[2] : 0;
+  a.layout = head_major ? ARGUS_HIP_HEAD_MAJOR : ARGUS_HIP_SEQ_MAJOR;
+  a.kv_dtype = (int32_t)k_cache.dtype;
+  a.batch = 1;
+
+  size_t stride = 0;
+  bool copy_back = false;
+  if (acc_ && acc_->is_active()) {
+    a.scores_out = (float *)acc_->score_buf_device_ptr() + acc_->layer_offset_elems(acc_->current_layer_idx());
+    a.score_stride = (int32_t)acc_->score_stride();
+  } else if (scores_out && num_heads_q > 0) {
+    stride = scores_len / num_heads_q;
+    if (stride != 0 && stride >= cache_seq_len) {
+      const size_t need = num_heads_q * stride * sizeof(float);
+      if (need > score_tmp_bytes_) {
+        if (score_tmp_) argus_hip_free(ctx_, score_tmp_);
+        score_tmp_ = nullptr;
+        score_tmp_bytes_ = 0;
+        if (argus_hip_malloc(ctx_, need, &score_tmp_) != ARGUS_HIP_OK) return Status::Err("score buffer: " + last_error());
+        score_tmp_bytes_ = need;
+      }
+      a.scores_out = (float *)score_tmp_;
+      a.score_stride = (int32_t)stride;
+      copy_back = true;
+    }
+  }
+  const int rc = argus_hip_attention_gen(ctx_, &a);
+  if (rc != ARGUS_HIP_OK) return Status::Err("attention_gen kernel launch failed: " + last_error());
+  if (copy_back) {
+    // The caller expects the slice to be valid on return: synchronising read-back of the rows.
+    const size_t total = num_heads_q * stride;
+    const size_t n = scores_len < total ? scores_len : total;
+    Status s = read_buffer(scores_out, score_tmp_, n * sizeof(float));
+    if (!s.ok()) return s;
+  }
+  return OkStatus();
+}
+
+}  // namespace argus

@@ -1,0 +1,303 @@
+// Device tests of the C++ host mirror (argus-engine_amd/host/argus_hip_backend.hpp), written the way
+// the reference's own device tests are: drive the backend through its trait-shaped methods and
+// compare with a host computation.
+//   * score accumulator flow      engine/src/bin/test_cuda_gpu_score_device.rs (cases 1-3)
+//   * attention_gen unit shape    engine/src/backend/cpu/x86.rs:1811-1973 (LCG seeds 42/137/53)
+//   * KIVI residual-only pattern  engine/src/bin/test_cuda_quant_attn_device.rs:108-178 (Test A)
+//   * degraded capability handle  engine/tests/gate_c_kivi_backend_cap.rs:90-146
+// The CPU oracle (test infrastructure) supplies the expected values.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "../../argus-engine_amd/host/argus_hip_backend.hpp"
+
+extern "C" {
+void oracle_gen_data(float *dst, int64_t n, uint32_t seed);
+void oracle_f32_to_f16(const float *src, uint16_t *dst, int64_t n);
+int oracle_attention_gen_scalar(const float *q, const void *k, const void *v, float *out, int hq, int hkv, int d, int len,
+                                int capacity, int head_major, int kv_dtype, float *scores, int64_t stride, float softcap,
+                                const int32_t *kv_index);
+int oracle_prefill_attention(const float *q, const void *k, const void *v, float *out, int hq, int hkv, int seq_len,
+                             int cache_len, int d, int capacity, int batch, int kv_dtype, int window, int n_threads);
+int oracle_score_fused_reduce(const float *scores, float *imp, float *himp, float decay_factor, int n_layers, int hq,
+                              int hkv, int len, int64_t stride, int max_seq);
+void oracle_kv_scatter(const float *k_src, const float *v_src, void *k_dst, void *v_dst, int kv_heads, int head_dim,
+                       int capacity, int write_pos_start, int seq_len, int dst_f16);
+}
+
+using namespace argus;
+
+static int g_fail = 0;
+#define CHECK(cond, ...)                                       \
+  do {                                                         \
+    if (!(cond)) {                                             \
+      printf("FAIL %s:%d: ", __FILE__, __LINE__);              \
+      printf(__VA_ARGS__);                                     \
+      printf("\n");                                            \
+      ++g_fail;                                                \
+    }                                                          \
+  } while (0)
+
+static float max_abs_diff(const std::vector<float> &a, const std::vector<float> &b) {
+  float m = 0;
+  for (size_t i = 0; i < a.size(); ++i) m = fmaxf(m, fabsf(a[i] - b[i]));
+  return m;
+}
+
+struct DevBuf {
+  HipBackend *be;
+  void *p = nullptr;
+  DevBuf(HipBackend *b, size_t bytes, const void *host = nullptr) : be(b) {
+    p = be->alloc(bytes).value();
+    if (host) be->write_buffer(p, host, bytes);
+  }
+  ~DevBuf() { be->free(p); }
+};
+
+static void test_score_accumulator(HipBackend &be) {
+  const size_t n_layers = 2, hq = 2, hkv = 1, max_seq = 8, len = 3;
+  CHECK(be.init_gpu_score_acc(n_layers, hq, hkv, max_seq, 0.0f).ok(), "init");
+  be.gpu_score_acc()->set_active(true);
+  std::vector<float> scores(n_layers * hq * max_seq, 0.0f);
+  auto set = [&](size_t l, size_t h, float a, float b, float c) {
+    float *p = &scores[l * hq * max_seq + h * max_seq];
+    p[0] = a; p[1] = b; p[2] = c;
+  };
+  set(0, 0, 0.1f, 0.2f, 0.7f); set(0, 1, 0.3f, 0.3f, 0.4f); set(1, 0, 0.5f, 0.4f, 0.1f); set(1, 1, 0.2f, 0.2f, 0.6f);
+  CHECK(be.gpu_score_acc()->debug_fill_score_buf(scores).ok(), "fill");
+  CHECK(be.gpu_score_acc()->end_step(nullptr, len).ok(), "end_step");
+  CHECK(be.synchronize().ok(), "sync");
+  auto r = be.gpu_score_acc()->sync_to_cpu();
+  CHECK(r.ok(), "sync_to_cpu");
+  const float exp_flat[3] = {0.7f, 0.6f, 1.1f}, exp_head[3] = {0.35f, 0.30f, 0.55f};
+  for (size_t t = 0; t < len; ++t) {
+    CHECK(fabsf(r.value().first[t] - exp_flat[t]) < 1e-5f, "case1 flat[%zu]=%g", t, r.value().first[t]);
+    CHECK(fabsf(r.value().second[t] - exp_head[t]) < 1e-5f, "case1 head[%zu]=%g", t, r.value().second[t]);
+  }
+  CHECK(be.gpu_score_acc()->steps_accumulated() == 1, "steps");
+  // case 2: decay 0.5, two identical steps -> 1.5 x
+  CHECK(be.init_gpu_score_acc(n_layers, hq, hkv, max_seq, 0.5f).ok(), "init2");
+  be.gpu_score_acc()->set_active(true);
+  be.gpu_score_acc()->debug_fill_score_buf(scores);
+  be.gpu_score_acc()->end_step(nullptr, len);
+  be.gpu_score_acc()->end_step(nullptr, len);
+  be.synchronize();
+  auto r2 = be.gpu_score_acc()->sync_to_cpu();
+  for (size_t t = 0; t < len; ++t) CHECK(fabsf(r2.value().first[t] - 1.5f * exp_flat[t]) < 1e-5f, "case2 flat[%zu]", t);
+  // case 3: seed round trip, then reset
+  CHECK(be.init_gpu_score_acc(n_layers, hq, hkv, max_seq, 0.0f).ok(), "init3");
+  std::vector<float> sf(max_seq), sh(hkv * max_seq);
+  for (size_t i = 0; i < max_seq; ++i) sf[i] = (float)i + 1.0f;
+  for (size_t i = 0; i < sh.size(); ++i) sh[i] = 0.25f * (float)i;
+  CHECK(be.gpu_score_acc()->seed_cumulative(sf, sh).ok(), "seed");
+  auto r3 = be.gpu_score_acc()->sync_to_cpu();
+  CHECK(r3.value().first == sf && r3.value().second == sh, "case3 seed round trip");
+  CHECK(!be.gpu_score_acc()->seed_cumulative(std::vector<float>(3), sh).ok(), "seed length check");
+  CHECK(be.gpu_score_acc()->reset().ok(), "reset");
+  auto r4 = be.gpu_score_acc()->sync_to_cpu();
+  for (float x : r4.value().first) CHECK(x == 0.0f, "reset clears");
+  printf("[score] accumulator cases 1-3 ok\n");
+}
+
+static void test_attention_gen(HipBackend &be) {
+  const int hq = 4, hkv = 2, d = 64, len = 16, cap = 32;
+  std::vector<float> q(hq * d), kf(hkv * cap * d), vf(hkv * cap * d);
+  oracle_gen_data(q.data(), q.size(), 42); oracle_gen_data(kf.data(), kf.size(), 137); oracle_gen_data(vf.data(), vf.size(), 53);
+  std::vector<uint16_t> kh(kf.size()), vh(vf.size());
+  oracle_f32_to_f16(kf.data(), kh.data(), kf.size()); oracle_f32_to_f16(vf.data(), vh.data(), vf.size());
+  for (int f16 = 0; f16 < 2; ++f16) {
+    const void *kp = f16 ? (const void *)kh.data() : (const void *)kf.data();
+    const void *vp = f16 ? (const void *)vh.data() : (const void *)vf.data();
+    const size_t kvb = kf.size() * (f16 ? 2 : 4);
+    DevBuf dq(&be, q.size() * 4, q.data()), dk(&be, kvb, kp), dv(&be, kvb, vp), dout(&be, q.size() * 4);
+    Tensor tq{dq.p, DType::F32, {(size_t)hq, (size_t)d}}, tout{dout.p, DType::F32, {(size_t)hq, (size_t)d}};
+    Tensor tk{dk.p, f16 ? DType::F16 : DType::F32, {1, (size_t)hkv, (size_t)cap, (size_t)d}}, tv = tk;
+    tv.ptr = dv.p;
+    // scores at stride `cap` (> cache_seq_len): rows beyond len keep their sentinel
+    std::vector<float> sc(hq * cap, -7.0f), ref(hq * d), ref_sc(hq * cap, -7.0f), got(hq * d);
+    CHECK(be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, sc.data(), sc.size()).ok(), "attention_gen");
+    be.read_buffer(got.data(), dout.p, got.size() * 4);
+    oracle_attention_gen_scalar(q.data(), kp, vp, ref.data(), hq, hkv, d, len, cap, 1, f16, ref_sc.data(), cap, 0.0f, nullptr);
+    CHECK(max_abs_diff(got, ref) < (f16 ? 1e-3f : 1e-4f), "attention_gen out diff %g", max_abs_diff(got, ref));
+    float worst = 0;
+    for (int h = 0; h < hq; ++h)
+      for (int t = 0; t < len; ++t) worst = fmaxf(worst, fabsf(sc[h * cap + t] - ref_sc[h * cap + t]) / ref_sc[h * cap + t]);
+    CHECK(worst < 1e-4f, "scores rel diff %g", worst);
+    // a malformed score slice (stride < cache_seq_len) disables the export, the call still succeeds
+    std::vector<float> small(hq * 4, -7.0f);
+    CHECK(be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, small.data(), small.size()).ok(), "malformed slice");
+    for (float x : small) CHECK(x == -7.0f, "malformed slice untouched");
+    // SeqMajor-shaped tensor ([len, hkv, d]) is detected from the shape
+    Tensor host_q = tq;
+    host_q.device = false;
+    CHECK(!be.attention_gen(host_q, tk, tv, tout, hq, hkv, d, len, nullptr, 0).ok(), "host tensor is refused");
+  }
+  printf("[attention_gen] unit shape f32/f16 + host score slice ok\n");
+}
+
+static void test_accumulator_binding(HipBackend &be) {
+  // With the accumulator active the kernel writes the layer's slice of the persistent score buffer
+  // and the host slice is left alone (cuda_pc.rs:1750-1766); end_step then reduces on the device.
+  const int n_layers = 3, hq = 8, hkv = 4, d = 128, len = 300, max_seq = 512;
+  CHECK(be.init_gpu_score_acc(n_layers, hq, hkv, max_seq, 0.0f).ok(), "init");
+  be.gpu_score_acc()->set_active(true);
+  std::vector<float> all_scores((size_t)n_layers * hq * max_seq, 0.0f);
+  for (int l = 0; l < n_layers; ++l) {
+    std::vector<float> q(hq * d), kf(hkv * max_seq * d), vf(kf.size());
+    oracle_gen_data(q.data(), q.size(), 100 + l); oracle_gen_data(kf.data(), kf.size(), 200 + l); oracle_gen_data(vf.data(), vf.size(), 300 + l);
+    for (auto &x : q) x *= 4.0f;
+    std::vector<uint16_t> kh(kf.size()), vh(vf.size());
+    oracle_f32_to_f16(kf.data(), kh.data(), kf.size()); oracle_f32_to_f16(vf.data(), vh.data(), vf.size());
+    DevBuf dq(&be, q.size() * 4, q.data()), dk(&be, kh.size() * 2, kh.data()), dv(&be, vh.size() * 2, vh.data()), dout(&be, q.size() * 4);
+    Tensor tq{dq.p, DType::F32, {(size_t)hq, (size_t)d}}, tout = tq, tk{dk.p, DType::F16, {1, (size_t)hkv, (size_t)max_seq, (size_t)d}}, tv = tk;
+    tout.ptr = dout.p; tv.ptr = dv.p;
+    be.gpu_score_acc()->set_current_layer_idx(l);
+    std::vector<float> host_sc(hq * len, -7.0f);
+    CHECK(be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, host_sc.data(), host_sc.size()).ok(), "attention_gen layer %d", l);
+    for (float x : host_sc) CHECK(x == -7.0f, "host slice untouched while the accumulator is armed");
+    std::vector<float> ref(hq * d);
+    oracle_attention_gen_scalar(q.data(), kh.data(), vh.data(), ref.data(), hq, hkv, d, len, max_seq, 1, 1,
+                                &all_scores[(size_t)l * hq * max_seq], max_seq, 0.0f, nullptr);
+  }
+  CHECK(be.gpu_score_acc()->end_step(nullptr, len).ok(), "end_step");
+  be.synchronize();
+  auto r = be.gpu_score_acc()->sync_to_cpu();
+  std::vector<float> imp(max_seq, 0.0f), himp(hkv * max_seq, 0.0f);
+  oracle_score_fused_reduce(all_scores.data(), imp.data(), himp.data(), 1.0f, n_layers, hq, hkv, len, max_seq, max_seq);
+  float worst = 0;
+  for (int t = 0; t < len; ++t) worst = fmaxf(worst, fabsf(r.value().first[t] - imp[t]) / imp[t]);
+  for (size_t i = 0; i < himp.size(); ++i)
+    if (himp[i] > 0) worst = fmaxf(worst, fabsf(r.value().second[i] - himp[i]) / himp[i]);
+  CHECK(worst < 1e-4f, "importance rel diff %g", worst);
+  be.gpu_score_acc()->set_active(false);
+  printf("[score] attention -> accumulator slice -> fused reduce ok (rel %.2e)\n", worst);
+}
+
+static void test_prefill_and_scatter(HipBackend &be) {
+  const int hq = 8, hkv = 2, d = 64, s = 100, cap = 128;
+  std::vector<float> q((size_t)s * hq * d), ksrc((size_t)s * hkv * d), vsrc(ksrc.size());
+  oracle_gen_data(q.data(), q.size(), 1); oracle_gen_data(ksrc.data(), ksrc.size(), 2); oracle_gen_data(vsrc.data(), vsrc.size(), 3);
+  // write path: scatter the prompt's K/V rows into the HeadMajor F16 cache (supports_kv_scatter_batch)
+  DevBuf dq(&be, q.size() * 4, q.data()), dks(&be, ksrc.size() * 4, ksrc.data()), dvs(&be, vsrc.size() * 4, vsrc.data());
+  std::vector<uint16_t> zero((size_t)hkv * cap * d, 0), kc = zero, vc = zero;
+  DevBuf dk(&be, zero.size() * 2, zero.data()), dv(&be, zero.size() * 2, zero.data()), dout(&be, q.size() * 4);
+  Tensor tks{dks.p, DType::F32, {(size_t)s, (size_t)hkv, (size_t)d}}, tvs = tks;
+  tvs.ptr = dvs.p;
+  Tensor tk{dk.p, DType::F16, {1, (size_t)hkv, (size_t)cap, (size_t)d}}, tv = tk;
+  tv.ptr = dv.p;
+  CHECK(be.supports_kv_scatter_batch(), "scatter batch");
+  CHECK(be.kv_scatter_f32_to_f16_batch(tks, tvs, tk, tv, hkv, d, cap, 0, s).ok(), "kv_scatter batch");
+  oracle_kv_scatter(ksrc.data(), vsrc.data(), kc.data(), vc.data(), hkv, d, cap, 0, s, 1);
+  std::vector<uint16_t> got_k(zero.size());
+  be.read_buffer(got_k.data(), dk.p, got_k.size() * 2);
+  CHECK(memcmp(got_k.data(), kc.data(), kc.size() * 2) == 0, "scattered K cache bit-exact");
+  CHECK(!be.kv_scatter_f32_to_f16_batch(tks, tvs, tk, tv, hkv, d, cap, cap - 1, s).ok(), "scatter beyond capacity fails");
+  // prefill over the scattered cache
+  Tensor tq{dq.p, DType::F32, {1, (size_t)s, (size_t)hq, (size_t)d}}, tout = tq;
+  tout.ptr = dout.p;
+  auto r = be.flash_attention_prefill(tq, tk, tv, tout, hq, hkv, s, s, d, cap, 1, true);
+  CHECK(r.ok() && r.value(), "prefill dispatched");
+  std::vector<float> got(q.size()), ref(q.size());
+  be.read_buffer(got.data(), dout.p, got.size() * 4);
+  oracle_prefill_attention(q.data(), kc.data(), vc.data(), ref.data(), hq, hkv, s, s, d, cap, 1, 1, 0, 0);
+  CHECK(max_abs_diff(got, ref) < 2e-3f, "prefill diff %g", max_abs_diff(got, ref));
+  // Ok(false): SeqMajor and unsupported head_dim are declined, the caller keeps its CPU path
+  auto r2 = be.flash_attention_prefill(tq, tk, tv, tout, hq, hkv, s, s, d, cap, 1, false);
+  CHECK(r2.ok() && !r2.value(), "SeqMajor declined");
+  auto r3 = be.flash_attention_prefill(tq, tk, tv, tout, hq, hkv, s, s, 96, cap, 1, true);
+  CHECK(r3.ok() && !r3.value(), "head_dim 96 declined");
+  auto r4 = be.flash_attention_prefill(tq, tk, tv, tout, hq, 3, s, s, d, cap, 1, true);
+  CHECK(!r4.ok(), "bad head counts are an error");
+  printf("[prefill] kv_scatter -> flash_attention_prefill ok, declines reported as Ok(false)\n");
+}
+
+static void test_quant_attn(HipBackend &be) {
+  HipQuantAttnBackend degraded(nullptr);
+  argus_hip_quant_attn_args za{};
+  argus_hip_quant_gather_args zg{};
+  CHECK(!degraded.has_quant_attn_kernel(2) && degraded.attention_gen_quant(za) == -1 && degraded.gather_update_quant(zg) == -1 &&
+            degraded.dequant_flush() == -1 && degraded.scatter_residual() == -1,
+        "degraded handle returns -1 everywhere");
+  HipQuantAttnBackend cap(be.ctx());
+  CHECK(cap.has_quant_attn_kernel(2) && cap.has_quant_attn_kernel(4) && cap.has_quant_attn_kernel(8) && !cap.has_quant_attn_kernel(3), "kernels present");
+  // Test A of the reference device test at head_dim 64: residual-only attention with host score read-back.
+  const size_t nhq = 2, nhkv = 1, hd = 64, res_cap = 32, r = 20;
+  const float scale = 1.0f / sqrtf((float)hd);
+  std::vector<float> q(nhq * hd), rk(nhkv * res_cap * hd, 0.0f), rv(rk.size(), 0.0f);
+  for (size_t h = 0; h < nhq; ++h)
+    for (size_t d = 0; d < hd; ++d) q[h * hd + d] = 0.1f * (float)((h * 7 + d) % 5) - 0.2f;
+  for (size_t t = 0; t < r; ++t)
+    for (size_t d = 0; d < hd; ++d) {
+      rk[t * hd + d] = 0.05f * (float)((t * 3 + d) % 7) - 0.15f;
+      rv[t * hd + d] = 0.03f * (float)((t + d * 2) % 9);
+    }
+  DevBuf dq(&be, q.size() * 4, q.data()), drk(&be, rk.size() * 4, rk.data()), drv(&be, rv.size() * 4, rv.data()), dummy(&be, 16), dout(&be, q.size() * 4);
+  // gather_update_quant appends a token row to the residual ring
+  std::vector<float> tok(nhkv * hd, 0.5f);
+  DevBuf dtok(&be, tok.size() * 4, tok.data());
+  argus_hip_quant_gather_args g{nullptr, (uint64_t)dtok.p, (uint64_t)drk.p, nhkv, res_cap, hd, 1, r};
+  CHECK(cap.gather_update_quant(g) == 0, "gather_update_quant");
+  std::vector<float> rk_back(rk.size());
+  be.read_buffer(rk_back.data(), drk.p, rk_back.size() * 4);
+  CHECK(rk_back[r * hd + 3] == 0.5f && rk_back[(r - 1) * hd + 3] == rk[(r - 1) * hd + 3], "residual row appended at res_pos");
+  std::vector<float> scores_host(nhq * r, 0.0f);
+  argus_hip_quant_attn_args a{};
+  a.q_mem = (uint64_t)dq.p; a.qk_mem = (uint64_t)dummy.p; a.qv_mem = (uint64_t)dummy.p;
+  a.res_k_mem = (uint64_t)drk.p; a.res_v_mem = (uint64_t)drv.p; a.out_mem = (uint64_t)dout.p;
+  a.scores_out = scores_host.data(); a.scores_len = scores_host.size();
+  a.num_heads_q = nhq; a.num_heads_kv = nhkv; a.head_dim = hd; a.q_tokens = 0; a.res_tokens = r; a.res_cap = res_cap;
+  a.scale = scale; a.bits = 2;
+  CHECK(cap.attention_gen_quant(a) == 0, "attention_gen_quant residual rc");
+  std::vector<float> o(nhq * hd);
+  be.read_buffer(o.data(), dout.p, o.size() * 4);
+  for (size_t h = 0; h < nhq; ++h) {
+    // host f64 textbook attention, as in the reference test
+    std::vector<double> s(r);
+    double mx = -1e300, sum = 0;
+    for (size_t t = 0; t < r; ++t) {
+      double acc = 0;
+      for (size_t d = 0; d < hd; ++d) acc += (double)q[h * hd + d] * (double)rk[t * hd + d];
+      s[t] = acc * (double)scale;
+      mx = fmax(mx, s[t]);
+    }
+    for (size_t t = 0; t < r; ++t) { s[t] = exp(s[t] - mx); sum += s[t]; }
+    double wsum = 0;
+    for (size_t t = 0; t < r; ++t) {
+      CHECK(fabs(scores_host[h * r + t] - s[t] / sum) < 1e-4, "A: weight[h%zu,t%zu]", h, t);
+      wsum += scores_host[h * r + t];
+    }
+    CHECK(fabs(wsum - 1.0) < 1e-4, "A: weights sum %g", wsum);
+    for (size_t d = 0; d < hd; ++d) {
+      double od = 0;
+      for (size_t t = 0; t < r; ++t) od += s[t] / sum * (double)rv[t * hd + d];
+      CHECK(fabs(o[h * hd + d] - od) < 1e-4, "A: O[h%zu,d%zu]", h, d);
+    }
+  }
+  a.bits = 3;
+  CHECK(cap.attention_gen_quant(a) < 0, "unsupported bits return a negative code");
+  printf("[kivi] degraded handle, gather_update, residual-only attention + host score read-back ok\n");
+}
+
+int main() {
+  auto r = HipBackend::create(0);
+  if (!r.ok()) {
+    printf("no HIP device: %s\n", r.error().c_str());
+    return 77;
+  }
+  HipBackend &be = *r.value();
+  CHECK(std::string(be.name()) == "HIP" && be.is_gpu() && be.is_discrete_gpu() && be.is_nosub_device(), "identity");
+  test_score_accumulator(be);
+  test_attention_gen(be);
+  test_accumulator_binding(be);
+  test_prefill_and_scatter(be);
+  test_quant_attn(be);
+  if (g_fail) {
+    printf("%d check(s) FAILED\n", g_fail);
+    return 1;
+  }
+  printf("ALL PASS: host mirror verified on-device\n");
+  return 0;
+}
