@@ -20,6 +20,8 @@
 #include "decode_common.hpp"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 namespace {
@@ -369,6 +371,12 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
 
   hipStream_t stream = (hipStream_t)a->stream;
   const bool want_scores = a->scores_out != nullptr;
+  // ARGUS_HIP_DECODE=valu keeps the vector-ALU kernel for A/B measurements.
+  static const bool force_valu = [] {
+    const char *e = getenv("ARGUS_HIP_DECODE");
+    return e && strcmp(e, "valu") == 0;
+  }();
+  if (!force_valu && decode_mfma_supported(p, D, a->kv_dtype)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
   switch (a->kv_dtype) {
     case ARGUS_HIP_F16: return dispatch_dim<_Float16>(ctx, p, D, a->batch, want_scores, stream);
     case ARGUS_HIP_F32: return dispatch_dim<float>(ctx, p, D, a->batch, want_scores, stream);

@@ -124,4 +124,8 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   }
 }
 
+// Matrix-core variant (decode_mfma.hip): F16 cache, contiguous slots, no soft-cap.
+bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype);
+int launch_decode_mfma(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hipStream_t stream);
+
 }  // namespace argus_decode

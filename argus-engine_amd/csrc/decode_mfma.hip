@@ -1,0 +1,273 @@
+// Split-KV flash-decode on the matrix cores: the F16-cache, no-soft-cap, contiguous-slot case of
+// Backend::attention_gen (engine/src/backend.rs:284-295).
+//
+// The vector-ALU decode kernel spends ~8 FMAs per K/V element pair per query head; at 5.6 TB/s
+// that keeps the VALUs ~60 % busy and is what limits it.  Here both products run as MFMAs whose
+// operands are exactly what a 16-byte row load puts in a lane, so nothing goes through LDS and the
+// VALUs only do the softmax:
+//
+//   S^T[token][head] = K . Q^T     v_mfma_f32_16x16x32_f16
+//       A (m = token = lane%16, k-group = lane/16): 8 channels = one 16-byte chunk of the token's
+//       K row.  Lane (j, r) loads chunk 4*kk + j of row r, so a wave's load covers 16 rows x 64 B.
+//       B (n = head = lane%16): the same chunk of Q, pre-scaled, split into f16 hi + lo parts (two
+//       MFMAs) so the logits keep f32-level accuracy.
+//       D: lane (j, h) holds the logits of tokens 4j..4j+3 for head h.
+//   O[head][channel] = P . V       v_mfma_f32_16x16x16_f16
+//       A (m = head, k = 4j + e): P for tokens 4j..4j+3 -- the lane's own softmax results.
+//       B (n = channel slot, k = 4j + e): lane group j loads rows 4j..4j+3 (one 16-byte piece
+//       each); a 4x8 in-register transpose (v_pack/v_perm) turns them into one operand per channel.
+//
+// Up to 16 query heads per KV head share the pass.  Split partials and the combine pass are the
+// ones of the vector-ALU kernel (decode_common.hpp).
+#include "decode_common.hpp"
+
+#include <algorithm>
+
+namespace argus_decode {
+
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+template <int D>
+struct MfmaShape {
+  static constexpr int KK = D / 32;                 // QK k-steps (32 channels each)
+  static constexpr int VC = (D >= 128) ? 8 : 4;     // halfs a lane loads per V row piece
+  static constexpr int VSEG = D / (16 * VC);        // pieces per row per lane
+  static constexpr int NACC = VC * VSEG;            // O accumulators (float4 each)
+  static constexpr int MAXH = (D == 256) ? 8 : 16;  // query heads per KV head (bounds the merge LDS)
+};
+
+template <int VC>
+struct VPiece;
+template <>
+struct VPiece<8> { using type = half8_t; };
+template <>
+struct VPiece<4> { using type = half4_t; };
+
+template <int D, int TW>
+__global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) {
+  using SH = MfmaShape<D>;
+  constexpr int KK = SH::KK, VC = SH::VC, VSEG = SH::VSEG, NACC = SH::NACC;
+  using vpiece_t = typename VPiece<VC>::type;
+  constexpr int TILE = 16 * TW;  // tokens per wave iteration
+  constexpr float kLn2 = 0.6931471805599453f;
+
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane >> 4, r = lane & 15;
+  const int G = p.group;
+
+  const int t_begin = split * p.chunk;
+  const int t_end = min(p.len, t_begin + p.chunk);
+
+  const _Float16 *kb = (const _Float16 *)p.k + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;
+  const _Float16 *vb = (const _Float16 *)p.v + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;
+
+  // ---- Q operand: lane (j, h = r) holds chunk 4kk + j of head h, scaled to the log2 domain ------
+  half8_t qh[KK], ql[KK];
+  {
+    const float c = p.scale * 1.4426950408889634f;
+    const int h = kvh * G + min(r, G - 1);
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)h * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = (r < G) ? qp[(4 * kk + j) * 8 + e] * c : 0.0f;
+        const _Float16 hi = (_Float16)x;
+        qh[kk][e] = hi;
+        ql[kk][e] = (_Float16)(x - (float)hi);
+      }
+    }
+  }
+
+  float4_t o_acc[NACC];
+#pragma unroll
+  for (int a = 0; a < NACC; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
+
+  const int64_t rs = p.row_stride;
+  for (int base = t_begin + wave * TILE; base < t_end; base += 4 * TILE) {
+    // ---- loads: TW tiles of 16 tokens -----------------------------------------------------------
+    half8_t kr[TW][KK];
+    vpiece_t vr[TW][VSEG][4];
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+      const int t0 = base + 16 * tw;
+      const int krow = min(t0 + r, t_end - 1) + p.kv_start;
+      const _Float16 *kp = kb + (int64_t)krow * rs + 8 * j;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) kr[tw][kk] = __builtin_nontemporal_load((const half8_t *)(kp + 32 * kk));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int vrow = min(t0 + 4 * j + e, t_end - 1) + p.kv_start;
+        const _Float16 *vp = vb + (int64_t)vrow * rs + VC * r;
+#pragma unroll
+        for (int sg = 0; sg < VSEG; ++sg)
+          vr[tw][sg][e] = __builtin_nontemporal_load((const vpiece_t *)(vp + 16 * VC * sg));
+      }
+    }
+
+    // ---- logits ---------------------------------------------------------------------------------
+    float4_t s[TW];
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+      s[tw] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        s[tw] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kr[tw][kk], qh[kk], s[tw], 0, 0, 0);
+        s[tw] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kr[tw][kk], ql[kk], s[tw], 0, 0, 0);
+      }
+    }
+    const bool full = base + TILE <= t_end;
+    float mt = kNegInf;
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float sv = fmaxf(s[tw][i], kNegInf);  // NaN logit counts as -inf (common.rs:555-560)
+        if (!full && base + 16 * tw + 4 * j + i >= t_end) sv = kNegInf;
+        s[tw][i] = sv;
+        mt = fmaxf(mt, sv);
+      }
+    if (p.scores && r < G) {
+      // Logits in natural units; the combine pass rewrites them as probabilities.
+      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + r) * p.score_stride;
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = base + 16 * tw + 4 * j + i;
+          if (t < t_end) srow[t] = s[tw][i] * kLn2;
+        }
+    }
+
+    // ---- online softmax: the running max of a head is shared by the four lane groups -----------
+    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+    m_run = m_new;
+    half4_t pa[TW];
+    float lsum = 0.0f;
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pa[tw][i] = (_Float16)__builtin_amdgcn_exp2f(s[tw][i] - m_ref);
+      // row sum over the f16-rounded weights the matrix cores consume
+      const half2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+      lsum = __builtin_amdgcn_fdot2(half2_t{pa[tw][0], pa[tw][1]}, one, lsum, false);
+      lsum = __builtin_amdgcn_fdot2(half2_t{pa[tw][2], pa[tw][3]}, one, lsum, false);
+    }
+    l_run = l_run * alpha + lsum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+      // O accumulator register i of lane group j belongs to head 4j + i: fetch that head's factor.
+      float al[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 4 * j + i, 64);
+#pragma unroll
+      for (int a = 0; a < NACC; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o_acc[a][i] *= al[i];
+    }
+
+    // ---- O += P . V -----------------------------------------------------------------------------
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+        for (int c = 0; c < VC; ++c) {
+          const half4_t bv = {vr[tw][sg][0][c], vr[tw][sg][1][c], vr[tw][sg][2][c], vr[tw][sg][3][c]};
+          o_acc[sg * VC + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * VC + c], 0, 0, 0);
+        }
+  }
+
+  // ---- merge: lane groups (row sum), then the 4 waves through LDS -------------------------------
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  __shared__ float lds_m[4][16], lds_l[4][16];
+  __shared__ float lds_acc[4][SH::MAXH][D + 4];
+  if (j == 0) {
+    lds_m[wave][r] = m_run;
+    lds_l[wave][r] = l_run;
+  }
+#pragma unroll
+  for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+    for (int c = 0; c < VC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][16 * VC * sg + VC * r + c] = o_acc[sg * VC + c][i];
+  __syncthreads();
+
+  for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+    const int g = idx / D, c = idx % D;
+    const int h = kvh * G + g;
+    const float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
+    const float m_ref = (mm == kNegInf) ? 0.0f : mm;
+    float o = 0.0f, ll = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = __builtin_amdgcn_exp2f(lds_m[w][g] - m_ref);
+      o += lds_acc[w][g][c] * f;
+      ll += lds_l[w][g] * f;
+    }
+    // Partials are handed to the combine pass in natural-log units.
+    const int64_t pidx = ((int64_t)b * p.n_heads_q + h) * p.nsplit + split;
+    p.ws_o[pidx * D + c] = o;
+    if (c == 0) {
+      p.ws_ml[pidx * 2 + 0] = mm * kLn2;
+      p.ws_ml[pidx * 2 + 1] = ll;
+    }
+  }
+}
+
+template <int D>
+int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
+  constexpr int TW = (D <= 128) ? 2 : 1;
+  constexpr int tile_rows = 4 * 16 * TW;
+  const int pairs = batch * p.n_heads_kv;
+  const int target_wgs = ctx->compute_units * 24;
+  const int max_splits = (p.len + tile_rows - 1) / tile_rows;
+  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, kMaxSplits}));
+  int chunk = (p.len + nsplit - 1) / nsplit;
+  chunk = (chunk + tile_rows - 1) / tile_rows * tile_rows;
+  nsplit = (p.len + chunk - 1) / chunk;
+  p.chunk = chunk;
+  p.nsplit = nsplit;
+  p.direct = 0;
+  const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
+  const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
+  int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+  if (rc != ARGUS_HIP_OK) return rc;
+  p.ws_ml = ctx->ws;
+  p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
+  {
+    KernelTimer timer(ctx, stream);
+    hipLaunchKernelGGL((decode_mfma_kernel<D, TW>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, p);
+  }
+  ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
+  ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  return ARGUS_HIP_OK;
+}
+
+}  // namespace
+
+bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
+  return kv_dtype == ARGUS_HIP_F16 && !p.kv_index && !(p.softcap > 0.0f) && p.group <= (D == 256 ? 8 : 16) &&
+         (D == 64 || D == 128 || D == 256) && p.len >= 64;
+}
+
+int launch_decode_mfma(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hipStream_t stream) {
+  switch (D) {
+    case 64: return launch_mfma<64>(ctx, p, batch, stream);
+    case 128: return launch_mfma<128>(ctx, p, batch, stream);
+    default: return launch_mfma<256>(ctx, p, batch, stream);
+  }
+}
+
+}  // namespace argus_decode
