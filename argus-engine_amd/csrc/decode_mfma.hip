@@ -227,10 +227,20 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
 
 template <int D>
 int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
+#ifdef ARGUS_MFMA_TW
+  constexpr int TW = ARGUS_MFMA_TW;
+#else
   constexpr int TW = (D <= 128) ? 2 : 1;
+#endif
   constexpr int tile_rows = 4 * 16 * TW;
   const int pairs = batch * p.n_heads_kv;
-  const int target_wgs = ctx->compute_units * 24;
+#ifdef ARGUS_MFMA_WGMUL
+  const int target_wgs = ctx->compute_units * ARGUS_MFMA_WGMUL;
+#else
+  // About one round of resident workgroups (3 per CU at this register count) measured best:
+  // long chunks amortise the Q set-up and the cross-wave merge.
+  const int target_wgs = ctx->compute_units * 4;
+#endif
   const int max_splits = (p.len + tile_rows - 1) / tile_rows;
   int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, kMaxSplits}));
   int chunk = (p.len + nsplit - 1) / nsplit;
