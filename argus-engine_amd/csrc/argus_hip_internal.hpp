@@ -108,4 +108,14 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr float kNegInf = -__builtin_huge_valf();
+
+// x == hi + lo to ~2^-22 relative, both f16.  The value goes through an empty asm so the compiler
+// sees one f32 number, not the expression that made it: otherwise it may round `hi` once straight
+// from a fused product (fma_mix) for one use and twice (f32, then f16) for another, and at a
+// rounding tie the two copies differ by an ulp, which makes `lo` belong to the wrong `hi`.
+__device__ __forceinline__ void split_f16(float x, _Float16 &hi, _Float16 &lo) {
+  asm("" : "+v"(x));
+  hi = (_Float16)x;
+  lo = (_Float16)(x - (float)hi);
+}
 #endif

@@ -75,9 +75,10 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float x = (r < G) ? qp[(4 * kk + j) * 8 + e] * c : 0.0f;
-        const _Float16 hi = (_Float16)x;
+        _Float16 hi, lo;
+        split_f16(x, hi, lo);
         qh[kk][e] = hi;
-        ql[kk][e] = (_Float16)(x - (float)hi);
+        ql[kk][e] = lo;
       }
     }
   }

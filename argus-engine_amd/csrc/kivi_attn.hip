@@ -16,28 +16,16 @@
 // channels of its token, reading its code byte and the block header from LDS), an online
 // softmax step runs over the 32 tokens, and the V phase runs with lanes = channels.  All GQA
 // query heads of the KV head share the single pass over the blocks.
-#include "decode_common.hpp"
+#include "kivi_common.hpp"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 
 namespace {
 
 using namespace argus_decode;
-
-constexpr int kUnit = 32;  // tokens per unit == codec group size (QKKV)
-
-struct KiviParams {
-  DecodeParams d;          // q/out/scores/ws/nsplit/scale/softcap/group/heads as for decode
-  const uint8_t *qk;
-  const uint8_t *qv;
-  const void *res_k;
-  const void *res_v;
-  int32_t head_dim, q_tokens, res_tokens, res_cap;
-  int32_t units_total, units_per_split;
-  int32_t res_f16;
-  int64_t qk_bs, qv_bs;  // bytes between consecutive sequences' block streams
-  int64_t res_bs;        // elements between consecutive sequences' residual windows
-};
+using namespace argus_kivi;
 
 template <int BITS>
 __device__ __forceinline__ float kivi_code(const uint8_t *qs, int i) {
@@ -320,6 +308,12 @@ __global__ __launch_bounds__(128) void kivi_flush_v_kernel(const float *__restri
 
 template <int BITS>
 int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
+  // ARGUS_HIP_KIVI=valu keeps the vector-ALU kernel for A/B measurements.
+  static const bool force_valu = [] {
+    const char *e = getenv("ARGUS_HIP_KIVI");
+    return e && strcmp(e, "valu") == 0;
+  }();
+  if (!force_valu && kivi_mfma_supported(kp)) return launch_kivi_mfma(ctx, kp, BITS, batch, stream);
   DecodeParams &p = kp.d;
   const int D = kp.head_dim;
   const int target_wgs = ctx->compute_units * 4;
