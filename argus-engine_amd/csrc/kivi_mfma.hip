@@ -1,25 +1,37 @@
 // KIVI fused dequant + decode attention on the matrix cores (Q2 / Q4 / Q8, head_dim 64 / 128).
 //
 // Same arithmetic as kivi_attn.hip (dequant `code*d + m`, crates/techniques/kivi/src/kivi_attn.cu:
-// 213-218, block layouts kivi_attn.cu:256-262 / 357-361), reorganised so the per-element work is
-// an unpack, not `Hq/Hkv` FMAs:
+// 213-218, block layouts kivi_attn.cu:256-262 / 357-361), reorganised so the per-code work is a
+// mask, not `Hq/Hkv` FMAs:
 //
 //   logits  S[t][h] = sum_ch code[ch][t] * (q[h][ch] * d[ch])  +  sum_ch m[ch] * q[h][ch]
 //   output  O[h][c] = sum_t (p[h][t] * d[t][cb]) * code[t][c]   +  sum_t p[h][t] * m[t][cb]
 //
-// Every term is a 16x16x32 f16 MFMA.  The codes are the operand that has 8 contraction values per
+// The code sums are 16x16x32 f16 MFMAs.  The codes are the operand with 8 contraction values per
 // lane (8 channels of one token for the logits, 8 tokens of one channel for the output); KIVI
 // stores K per channel and V per token, i.e. both transposed relative to that, so each wave copies
-// its unit's K and V tiles (32 tokens) into a private LDS region and gathers the codes with byte
-// reads.  A code is turned into an exact f16 integer with one mask-or (1024 + code << shift) and one
-// packed subtract; the sub-byte shift is undone as a power-of-two factor on the MFMA result.  The
-// block scales go to the *other* operand in f32 (q*d split into f16 hi + lo, p*d in f16), and the
-// zero-point terms are MFMAs whose operand is the f16 `m` header itself.  Waves are autonomous:
-// no workgroup barrier inside the unit loop.  Residual rows (F32 or F16) run through the same
-// MFMAs with the row split into f16 hi + lo.
+// its unit's K and V tiles (32 tokens) into a private LDS region and gathers code bytes from there.
+//
+//  * A code field masked out of its byte *is* an f16 operand: an integer n < 1024 in the low bits
+//    of a half is the subnormal n * 2^-24, which the MFMA multiplies exactly.  No conversion; the
+//    field's bit position and the 2^-24 come back as one power-of-two factor on the result.
+//  * One byte (two for Q8) holds the codes of two neighbouring tokens (K) or channels (V).  A lane
+//    owns both: rows 2r and 2r+1 of the logits go to two accumulators fed from the same read.
+//  * The block scales ride on the other operand: q*d in f32, split into f16 hi + lo (the logits
+//    keep ~2^-22 relative accuracy, the 1e-4 bound on emitted scores needs it), and p*d in f16.
+//    Only `group` of the 16 operand columns are real heads, so the q*d work of a unit is spread
+//    over all 16 lanes of a row (each prepares one 32-channel slice for its head) and moved to the
+//    head's lane with a DPP row shift when the slice's MFMA is issued.
+//  * The zero-point terms: sum m*q on the vector ALU while the scales are read, sum p*m as one
+//    more MFMA whose operand is the f16 `m` header itself.
+//
+// Waves are autonomous: a wave prefetches its next unit into registers while it works on the
+// current one, and there is no workgroup barrier inside the unit loop.  The residual window (F32
+// or F16 rows) is a second loop over the same MFMAs with the K rows split into f16 hi + lo.
 #include "kivi_common.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace argus_kivi {
 
@@ -27,7 +39,6 @@ using namespace argus_decode;
 
 namespace {
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ void wave_lds_fence() {
@@ -36,35 +47,88 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Two bytes -> two exact f16 integers (code << shift), via 1024 + x in the f16 mantissa.
-__device__ __forceinline__ half2_t codes_to_half2(uint32_t b0, uint32_t b1, uint32_t mask2) {
-  const uint32_t v = ((b0 | (b1 << 16)) & mask2) | 0x64006400u;
-  const half2_t h = __builtin_bit_cast(half2_t, v);
-  const half2_t k = {(_Float16)1024.0f, (_Float16)1024.0f};
-  return h - k;
+// Lane i of a 16-lane row takes the value of lane i + SHIFT (zero past the row end).
+template <int SHIFT>
+__device__ __forceinline__ uint32_t row_shl(uint32_t x) {
+  if constexpr (SHIFT == 0) return x;
+  else return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x100 + SHIFT, 0xf, 0xf, true);
+}
+template <int SHIFT>
+__device__ __forceinline__ half8_t row_shl(half8_t v) {
+  u32x4_t w = __builtin_bit_cast(u32x4_t, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = row_shl<SHIFT>(w[i]);
+  return __builtin_bit_cast(half8_t, w);
+}
+template <int SHIFT>
+__device__ __forceinline__ float row_shl_add(float x) {
+  if constexpr (SHIFT > 0 && SHIFT < 16) x += __builtin_bit_cast(float, row_shl<SHIFT>(__builtin_bit_cast(uint32_t, x)));
+  return x;
 }
 
-__device__ __forceinline__ half8_t make_half8(half2_t a, half2_t b, half2_t c, half2_t d) {
-  return half8_t{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+// The lane's code field: 2*BITS bits holding two neighbouring codes (tokens 2r, 2r+1 of a K
+// channel block, channels 2r, 2r+1 of a V token block).
+template <int BITS>
+__device__ __forceinline__ int field_offset(int r) {
+  return 4 + (BITS == 8 ? 2 * r : BITS == 4 ? r : (r >> 1));
+}
+template <int BITS>
+__device__ __forceinline__ uint32_t field_read(const uint8_t *p) {
+  if constexpr (BITS == 8) return *(const uint16_t *)p;
+  else return *p;
+}
+// Two reads (consecutive contraction slots) -> one packed f16x2 operand word per owned code.
+// The matrix core multiplies subnormal halves exactly but keeps product bits relative to the
+// operand's exponent, not its leading one: a field in the lowest mantissa bits loses that many bits
+// of the sum (measured: 2^-20 relative for a 4-bit field at bit 0, 2^-24 at bit 4).  So every field
+// is moved up to end at mantissa bit 7 or 9 first; `presh` is that left shift (lane-dependent for Q2,
+// whose field sits in either nibble of its byte).
+template <int BITS>
+__device__ __forceinline__ void field_pair(uint32_t x0, uint32_t x1, int presh, uint32_t &w0, uint32_t &w1) {
+  if constexpr (BITS == 8) {
+    w0 = __builtin_amdgcn_perm(x1, x0, 0x0c040c00u);  // [x0.b0, 0, x1.b0, 0]
+    w1 = __builtin_amdgcn_perm(x1, x0, 0x0c050c01u);  // [x0.b1, 0, x1.b1, 0]
+  } else if constexpr (BITS == 4) {
+    const uint32_t v = x0 | (x1 << 16);
+    w0 = (v << 4) & 0x00f000f0u;
+    w1 = v & 0x00f000f0u;
+  } else {
+    const uint32_t v = (x0 | (x1 << 16)) << presh;
+    w0 = v & 0x00c000c0u;
+    w1 = v & 0x03000300u;
+  }
+}
+// Bit position of code `which` (0 / 1) inside the operand half.
+template <int BITS>
+__host__ __device__ constexpr int field_shift(int which) {
+  return BITS == 8 ? 0 : BITS == 4 ? 4 : 6 + 2 * which;
 }
 
-template <int BITS, int D>
-__global__ __launch_bounds__(256) void kivi_mfma_kernel(const KiviParams kp) {
+constexpr float kLn2 = 0.6931471805599453f;
+// Power of two on the f16 operands that carry block scales: keeps the low halves of the hi + lo
+// splits and small p*d products out of the f16 subnormal range.
+constexpr float kOpScale = 64.0f;
+constexpr float kCodeUnit = 16777216.0f;  // a raw code field n is the half n * 2^-24
+
+template <int BITS, int D, int GT>
+__global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) {
   constexpr int BB = 4 + 32 * BITS / 8;  // block bytes
-  constexpr int KK = D / 32;             // 32-channel steps == V blocks per token
+  constexpr int KK = D / 32;             // 32-channel slices == V blocks per token
   constexpr int TILE_BYTES = D * BB;     // one K tile == one V tile
+  constexpr int TILE_VEC = TILE_BYTES / 16;
+  constexpr int NCH = (TILE_VEC + 63) / 64;
   constexpr int WAVE_BYTES = 2 * TILE_BYTES;
   constexpr int MERGE_BYTES = 4 * 16 * (D + 4) * 4 + 4 * 16 * KK * 4 + 2 * 4 * 16 * 4;
   constexpr int SMEM = (4 * WAVE_BYTES > MERGE_BYTES) ? 4 * WAVE_BYTES : MERGE_BYTES;
-  constexpr uint32_t CMASK = (1u << BITS) - 1u;
-  constexpr float kLn2 = 0.6931471805599453f;
-  constexpr float kOpScale = 64.0f;  // power of two applied to the f16 operands that carry scales
+  constexpr int NREP = 16 / GT;               // lanes of a row that share one head
+  constexpr int NS = (KK + NREP - 1) / NREP;  // slices each lane prepares
   __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM];
 
   const DecodeParams &p = kp.d;
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane >> 4, r = lane & 15;
+  const int ra = r / GT, rh = r % GT;  // slice owner index and head of this lane during preparation
   const int G = p.group;
   const int gpf = kp.res_cap / kUnit;
   const int q_units = kp.q_tokens / kUnit;
@@ -73,170 +137,47 @@ __global__ __launch_bounds__(256) void kivi_mfma_kernel(const KiviParams kp) {
   uint8_t *sV = sK + TILE_BYTES;
   const uint8_t *qk_b = kp.qk + (int64_t)b * kp.qk_bs;
   const uint8_t *qv_b = kp.qv + (int64_t)b * kp.qv_bs;
+  const float qscale = p.scale * 1.4426950408889634f * kOpScale;  // log2 domain
 
-  // ---- constant Q operands: lane (h = r, j) holds channels 32kk + 8j + e -------------------------
-  // log2 domain, times kOpScale: the low halves of the f16 hi + lo splits (q, and q*d with d as
-  // small as range/255) would otherwise sit in the f16 subnormal range and lose their bits.
-  float qf[KK][8];
-  half8_t qh[KK], ql[KK];
-  {
-    const float c = p.scale * 1.4426950408889634f * kOpScale;
-    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(kvh * G + min(r, G - 1)) * D;
+  // q of head rh for the slices this lane prepares: slice s -> channels 32*(ra + s*NREP) + 8j + e
+  float qf[NS][8];
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
+  for (int s = 0; s < NS; ++s) {
+    const int kk = ra + s * NREP;
+    const bool ok = kk < KK && rh < G;
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(kvh * G + min(rh, G - 1)) * D + 32 * min(kk, KK - 1) + 8 * j;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float x = (r < G) ? qp[32 * kk + 8 * j + e] * c : 0.0f;
-        qf[kk][e] = x;
-        _Float16 hi, lo;
-        split_f16(x, hi, lo);
-        qh[kk][e] = hi;
-        ql[kk][e] = lo;
-      }
+    for (int e = 0; e < 8; ++e) qf[s][e] = ok ? qp[e] * qscale : 0.0f;
   }
 
-  // Sub-byte position of this lane's token (logit side, token = 16*half + r) and channel (output
-  // side, channel = 16*sub + r): both depend on r only.
-  const int sh_r = (r * BITS) % 8;
-  const uint32_t mask_r = (CMASK << sh_r) * 0x00010001u;
-  // undoes the shift on this lane's output columns and the operand scale on p*d
-  const float fv = 1.0f / ((float)(1 << sh_r) * kOpScale);
+  const int foff = field_offset<BITS>(r);
+  const int presh = 6 - 4 * (r & 1);  // Q2 only: the lane's field is the low or the high nibble of its byte
 
-  float4_t o_acc[2 * KK];  // [cb*2 + sub]: lane (j, n=r) reg i -> head 4j+i, channel 32cb+16sub+r
-  float4_t m_acc = {0.0f, 0.0f, 0.0f, 0.0f};  // zero-point term: lane (j, n=cb) reg i -> head 4j+i
+  // o_acc[2cb + sub]: lane (j, n = r) reg i -> head 4j + i, channel 32cb + 2r + sub
+  float4_t o_acc[2 * KK];
+  float4_t m_acc = {0.0f, 0.0f, 0.0f, 0.0f};  // zero-point term: lane (j, n = cb) reg i -> head 4j + i
 #pragma unroll
   for (int a = 0; a < 2 * KK; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;
-  bool shift_pending = true;  // o_acc still carries the per-lane 2^shift factor
 
-  // token owned by k-slot e of lane group jj (the lane's own logits, in MFMA output order)
-  auto tok_of = [](int jj, int e) { return (e < 4) ? (4 * jj + e) : (16 + 4 * jj + (e - 4)); };
-
-  const int u_begin = split * kp.units_per_split;
-  const int u_end = min(kp.units_total, u_begin + kp.units_per_split);
-  for (int u = u_begin + wave; u < u_end; u += 4) {
-    const bool quant = u < q_units;
-    float4_t s[2];
-    s[0] = s[1] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    int tok0, n_valid;
-
-    if (quant) {
-      tok0 = u * kUnit;
-      n_valid = kUnit;
-      // ---- stage the unit's K and V tiles into this wave's LDS region ---------------------------
-      {
-        const int flush = u / gpf, gif = u % gpf;
-        const int64_t kblk = ((int64_t)flush * p.n_heads_kv * gpf + (int64_t)kvh * gpf + gif) * D;
-        const int tif0 = (u * kUnit) % kp.res_cap;
-        const int64_t vblk = (((int64_t)flush * p.n_heads_kv + kvh) * kp.res_cap + tif0) * KK;
-        const u32x4_t *ksrc = (const u32x4_t *)(qk_b + kblk * BB);
-        const u32x4_t *vsrc = (const u32x4_t *)(qv_b + vblk * BB);
-        wave_lds_fence();  // the previous unit's reads are done
-#pragma unroll
-        for (int c = 0; c < (TILE_BYTES / 16 + 63) / 64; ++c) {
-          const int i = lane + 64 * c;
-          if (i < TILE_BYTES / 16) {
-            ((u32x4_t *)sK)[i] = __builtin_nontemporal_load(ksrc + i);
-            ((u32x4_t *)sV)[i] = __builtin_nontemporal_load(vsrc + i);
-          }
-        }
-        wave_lds_fence();
-      }
-
-      // ---- q*d operands (B, lane = head r) and zero-point operands (A, any row) -----------------
-      half8_t qdh[KK], qdl[KK], mk[KK];
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint8_t *blk = sK + (32 * kk + 8 * j + e) * BB;
-          const float dd = (float)*(const _Float16 *)blk;
-          mk[kk][e] = *(const _Float16 *)(blk + 2);
-          _Float16 hi, lo;
-          split_f16(qf[kk][e] * dd, hi, lo);
-          qdh[kk][e] = hi;
-          qdl[kk][e] = lo;
-        }
-
-      // ---- logits: two halves of 16 tokens (row m = r -> token 16*half + r) ---------------------
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const int byte_off = 4 + ((16 * hf + r) * BITS) / 8;
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          const uint8_t *cp = sK + (32 * kk + 8 * j) * BB + byte_off;
-          const half8_t a = make_half8(codes_to_half2(cp[0], cp[BB], mask_r), codes_to_half2(cp[2 * BB], cp[3 * BB], mask_r),
-                                       codes_to_half2(cp[4 * BB], cp[5 * BB], mask_r), codes_to_half2(cp[6 * BB], cp[7 * BB], mask_r));
-          s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qdh[kk], s[hf], 0, 0, 0);
-          s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qdl[kk], s[hf], 0, 0, 0);
-        }
-      }
-      // result register i belongs to token 16*half + 4j + i: undo that token's sub-byte shift
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float f = 1.0f / (float)(1 << ((i * BITS) % 8));
-        s[0][i] *= f;
-        s[1][i] *= f;
-      }
-      // zero-point term sum_ch m[ch] q[h][ch]: identical for every token row
-      float4_t c0 = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(mk[kk], qh[kk], c0, 0, 0, 0);
-        c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(mk[kk], ql[kk], c0, 0, 0, 0);
-      }
-      s[0] = (s[0] + c0) * (1.0f / kOpScale);
-      s[1] = (s[1] + c0) * (1.0f / kOpScale);
-    } else {
-      // ---- residual rows: [kv_heads, res_cap, D] F32 or F16 -------------------------------------
-      const int ru = u - q_units;
-      tok0 = kp.q_tokens + ru * kUnit;
-      n_valid = min(kUnit, kp.res_tokens - ru * kUnit);
-      if (shift_pending) {
-#pragma unroll
-        for (int a = 0; a < 2 * KK; ++a) o_acc[a] *= fv;
-        shift_pending = false;
-      }
-      const int64_t rbase = (int64_t)b * kp.res_bs + (int64_t)kvh * kp.res_cap * D;
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const int rt = ru * kUnit + min(16 * hf + r, n_valid - 1);
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          half8_t ah, al;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const int64_t idx = rbase + (int64_t)rt * D + 32 * kk + 8 * j + e;
-            const float x = kp.res_f16 ? (float)((const _Float16 *)kp.res_k)[idx] : ((const float *)kp.res_k)[idx];
-            _Float16 hi, lo;
-            split_f16(x, hi, lo);
-            ah[e] = hi;
-            al[e] = lo;
-          }
-          s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, qh[kk], s[hf], 0, 0, 0);
-          s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, ql[kk], s[hf], 0, 0, 0);
-          s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, qh[kk], s[hf], 0, 0, 0);
-        }
-        s[hf] *= 1.0f / kOpScale;
-      }
-    }
-
-    // ---- online softmax over the unit's 32 tokens; lane (j, h = r) owns tokens tok_of(j, e) ------
+  // Online-softmax step for one unit.  In: s[w][i] = logit (log2 units) of token 8j + 2i + w for
+  // head r.  Out: pa[e] = probability of token 8j + e relative to the running maximum.
+  auto softmax_step = [&](float4_t(&s)[2], int tok0, int n_valid) -> half8_t {
     float mt = kNegInf;
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (16 * hf + 4 * j + i >= n_valid) s[hf][i] = kNegInf;
-        mt = fmaxf(mt, s[hf][i]);  // a NaN logit propagates (the reference kernels have no guard)
+      for (int w = 0; w < 2; ++w) {
+        if (8 * j + 2 * i + w >= n_valid) s[w][i] = kNegInf;
+        mt = fmaxf(mt, s[w][i]);  // a NaN logit propagates (the reference kernels have no guard)
       }
     if (p.scores && r < G) {
-      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + r) * p.score_stride + tok0;
+      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + r) * p.score_stride + tok0 + 8 * j;
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf)
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (16 * hf + 4 * j + i < n_valid) srow[16 * hf + 4 * j + i] = s[hf][i] * kLn2;
+        for (int w = 0; w < 2; ++w)
+          if (8 * j + 2 * i + w < n_valid) srow[2 * i + w] = s[w][i] * kLn2;
     }
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
@@ -247,11 +188,13 @@ __global__ __launch_bounds__(256) void kivi_mfma_kernel(const KiviParams kp) {
     half8_t pa;
     float lsum = 0.0f;  // f32 sum: the emitted probabilities are normalised by it
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float pw = __builtin_amdgcn_exp2f(s[e / 4][e % 4] - m_ref);  // NaN stays NaN
-      lsum += pw;
-      pa[e] = (_Float16)pw;
-    }
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const float pw = __builtin_amdgcn_exp2f(s[w][i] - m_ref);  // NaN stays NaN
+        lsum += pw;
+        pa[2 * i + w] = (_Float16)pw;
+      }
     l_run = l_run * alpha + lsum;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
       float al[4];
@@ -264,55 +207,203 @@ __global__ __launch_bounds__(256) void kivi_mfma_kernel(const KiviParams kp) {
         m_acc[i] *= al[i];
       }
     }
+    return pa;
+  };
 
-    // ---- output ----------------------------------------------------------------------------------
-    if (quant) {
-      const half8_t pa_s = pa * (_Float16)kOpScale;  // keeps small p*d out of the f16 subnormals
+  const int u_begin = split * kp.units_per_split;
+  const int u_end = min(kp.units_total, u_begin + kp.units_per_split);
+  const int uq_end = min(u_end, q_units);
+  int u = u_begin + wave;
+
+  // ================================ quantised units ===============================================
+  u32x4_t pk[NCH], pv[NCH];
+  auto fetch = [&](int uu) {
+    const int flush = uu / gpf, gif = uu % gpf;
+    const int64_t kblk = ((int64_t)flush * p.n_heads_kv * gpf + (int64_t)kvh * gpf + gif) * D;
+    const int tif0 = (uu * kUnit) % kp.res_cap;
+    const int64_t vblk = (((int64_t)flush * p.n_heads_kv + kvh) * kp.res_cap + tif0) * KK;
+    const u32x4_t *ksrc = (const u32x4_t *)(qk_b + kblk * BB);
+    const u32x4_t *vsrc = (const u32x4_t *)(qv_b + vblk * BB);
 #pragma unroll
-      for (int cb = 0; cb < KK; ++cb) {
-        // A operand: p * d[token][cb] (lane = head r, k-slot e -> token tok_of(j, e))
-        half8_t dv;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dv[e] = *(const _Float16 *)(sV + (tok_of(j, e) * KK + cb) * BB);
-        const half8_t pd = pa_s * dv;
-#pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-          // B operand: codes of channel 32cb + 16sub + r for tokens tok_of(j, e)
-          const int byte_off = cb * BB + 4 + ((16 * sub + r) * BITS) / 8;
-          uint32_t bt[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) bt[e] = sV[tok_of(j, e) * KK * BB + byte_off];
-          const half8_t bc = make_half8(codes_to_half2(bt[0], bt[1], mask_r), codes_to_half2(bt[2], bt[3], mask_r),
-                                        codes_to_half2(bt[4], bt[5], mask_r), codes_to_half2(bt[6], bt[7], mask_r));
-          o_acc[2 * cb + sub] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, bc, o_acc[2 * cb + sub], 0, 0, 0);
-        }
-      }
-      // zero-point term: column n = cb holds sum_t p[h][t] m[t][cb]
-      half8_t mv = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (r < KK) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) mv[e] = *(const _Float16 *)(sV + (tok_of(j, e) * KK + r) * BB + 2);
-      }
-      m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, mv, m_acc, 0, 0, 0);
-    } else {
-      const int ru = u - q_units;
-      const int64_t rbase = (int64_t)b * kp.res_bs + (int64_t)kvh * kp.res_cap * D;
-#pragma unroll
-      for (int cs = 0; cs < 2 * KK; ++cs) {
-        half8_t bv;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int rt = ru * kUnit + min(tok_of(j, e), n_valid - 1);
-          const int64_t idx = rbase + (int64_t)rt * D + 16 * cs + r;
-          bv[e] = kp.res_f16 ? ((const _Float16 *)kp.res_v)[idx] : (_Float16)((const float *)kp.res_v)[idx];
-        }
-        o_acc[cs] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, bv, o_acc[cs], 0, 0, 0);
+    for (int c = 0; c < NCH; ++c) {
+      const int i = lane + 64 * c;
+      if (i < TILE_VEC) {
+        pk[c] = __builtin_nontemporal_load(ksrc + i);
+        pv[c] = __builtin_nontemporal_load(vsrc + i);
       }
     }
-  }
-  if (shift_pending) {
+  };
+  if (u < uq_end) fetch(u);
+
+  for (; u < uq_end; u += 4) {
+    wave_lds_fence();  // the previous unit's reads are done
 #pragma unroll
-    for (int a = 0; a < 2 * KK; ++a) o_acc[a] *= fv;
+    for (int c = 0; c < NCH; ++c) {
+      const int i = lane + 64 * c;
+      if (i < TILE_VEC) {
+        ((u32x4_t *)sK)[i] = pk[c];
+        ((u32x4_t *)sV)[i] = pv[c];
+      }
+    }
+    wave_lds_fence();
+    if (u + 4 < uq_end) fetch(u + 4);
+
+    // ---- this lane's share of q*d (hi + lo) and of sum m*q ----------------------------------------
+    half8_t own_h[NS], own_l[NS];
+    float c0 = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int kk = min(ra + s * NREP, KK - 1);  // qf is zero where the slice does not exist
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t hd = *(const uint32_t *)(sK + (32 * kk + 8 * j + e) * BB);
+        const float dd = (float)__builtin_bit_cast(_Float16, (uint16_t)(hd & 0xffffu));
+        const float mm = (float)__builtin_bit_cast(_Float16, (uint16_t)(hd >> 16));
+        _Float16 hi, lo;
+        split_f16(qf[s][e] * dd, hi, lo);
+        own_h[s][e] = hi;
+        own_l[s][e] = lo;
+        c0 = fmaf(qf[s][e], mm, c0);
+      }
+    }
+    c0 += __shfl_xor(c0, 16, 64);
+    c0 += __shfl_xor(c0, 32, 64);
+    if constexpr (NREP >= 16) c0 = row_shl_add<8 * GT>(c0);
+    if constexpr (NREP >= 8) c0 = row_shl_add<4 * GT>(c0);
+    if constexpr (NREP >= 4) c0 = row_shl_add<2 * GT>(c0);
+    if constexpr (NREP >= 2) c0 = row_shl_add<GT>(c0);
+    c0 *= 1.0f / kOpScale;  // lanes r < GT now hold sum_ch m[ch] q[r][ch]
+
+    // ---- logits: rows m = r -> tokens 2r (s[0]) and 2r + 1 (s[1]) ----------------------------------
+    float4_t s[2];
+    s[0] = s[1] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    auto qk_slice = [&](auto kk_c) {
+      constexpr int kk = decltype(kk_c)::value;
+      uint32_t x[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = field_read<BITS>(sK + (32 * kk + 8 * j + e) * BB + foff);
+      uint32_t w0[4], w1[4];
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) field_pair<BITS>(x[2 * pr], x[2 * pr + 1], presh, w0[pr], w1[pr]);
+      const half8_t a0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
+      const half8_t a1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
+      const half8_t bh = row_shl<(kk % NREP) * GT>(own_h[kk / NREP]);
+      const half8_t bl = row_shl<(kk % NREP) * GT>(own_l[kk / NREP]);
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bh, s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bh, s[1], 0, 0, 0);
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bl, s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bl, s[1], 0, 0, 0);
+    };
+    qk_slice(std::integral_constant<int, 0>{});
+    qk_slice(std::integral_constant<int, 1>{});
+    if constexpr (KK > 2) {
+      qk_slice(std::integral_constant<int, 2>{});
+      qk_slice(std::integral_constant<int, 3>{});
+    }
+    // undo the field position and the operand units
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+        s[w][i] = fmaf(s[w][i], kCodeUnit / (kOpScale * (float)(1 << field_shift<BITS>(w))), c0);
+
+    const half8_t pa = softmax_step(s, u * kUnit, kUnit);
+
+    // ---- output: contraction slot e -> token 8j + e -------------------------------------------------
+    const half8_t pa_s = pa * (_Float16)kOpScale;
+#pragma unroll
+    for (int cb = 0; cb < KK; ++cb) {
+      u32x4_t dw;
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        const uint32_t d0 = *(const uint16_t *)(sV + ((8 * j + 2 * pr) * KK + cb) * BB);
+        const uint32_t d1 = *(const uint16_t *)(sV + ((8 * j + 2 * pr + 1) * KK + cb) * BB);
+        dw[pr] = d0 | (d1 << 16);
+      }
+      const half8_t pd = pa_s * __builtin_bit_cast(half8_t, dw);  // rows = heads: p * d[token][cb]
+      uint32_t y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = field_read<BITS>(sV + ((8 * j + e) * KK + cb) * BB + foff);
+      uint32_t w0[4], w1[4];
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) field_pair<BITS>(y[2 * pr], y[2 * pr + 1], presh, w0[pr], w1[pr]);
+      const half8_t b0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
+      const half8_t b1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
+      o_acc[2 * cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b0, o_acc[2 * cb], 0, 0, 0);
+      o_acc[2 * cb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b1, o_acc[2 * cb + 1], 0, 0, 0);
+    }
+    // zero-point term: column n = cb holds sum_t p[h][t] m[t][cb]
+    u32x4_t mw = {0u, 0u, 0u, 0u};
+    if (r < KK) {
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        const uint32_t m0 = *(const uint16_t *)(sV + ((8 * j + 2 * pr) * KK + r) * BB + 2);
+        const uint32_t m1 = *(const uint16_t *)(sV + ((8 * j + 2 * pr + 1) * KK + r) * BB + 2);
+        mw[pr] = m0 | (m1 << 16);
+      }
+    }
+    m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(half8_t, mw), m_acc, 0, 0, 0);
+  }
+
+  // The code sums carry the field position and the operand units.
+#pragma unroll
+  for (int cb = 0; cb < KK; ++cb) {
+    o_acc[2 * cb] *= kCodeUnit / (kOpScale * (float)(1 << field_shift<BITS>(0)));
+    o_acc[2 * cb + 1] *= kCodeUnit / (kOpScale * (float)(1 << field_shift<BITS>(1)));
+  }
+
+  // ================================ residual window ===============================================
+  // Rows [kv_heads, res_cap, D], F32 or F16; same lane roles (rows 2r / 2r+1, columns 2r / 2r+1).
+  auto residual_unit = [&](auto tag, int ru) {
+    using RES_T = decltype(tag);
+    const int n_valid = min(kUnit, kp.res_tokens - ru * kUnit);
+    const int64_t rbase = (int64_t)b * kp.res_bs + (int64_t)kvh * kp.res_cap * D + (int64_t)ru * kUnit * D;
+    const RES_T *rk = (const RES_T *)kp.res_k + rbase;
+    const RES_T *rv = (const RES_T *)kp.res_v + rbase;
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(kvh * G + min(r, G - 1)) * D + 8 * j;
+    float4_t s[2];
+    s[0] = s[1] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      half8_t qh, ql;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        _Float16 hi, lo;
+        split_f16((r < G) ? qp[32 * kk + e] * qscale : 0.0f, hi, lo);
+        qh[e] = hi;
+        ql[e] = lo;
+      }
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const RES_T *row = rk + (int64_t)min(2 * r + w, n_valid - 1) * D + 32 * kk + 8 * j;
+        half8_t ah, al;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          _Float16 hi, lo;
+          split_f16((float)row[e], hi, lo);
+          ah[e] = hi;
+          al[e] = lo;
+        }
+        s[w] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, qh, s[w], 0, 0, 0);
+        s[w] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, ql, s[w], 0, 0, 0);
+        s[w] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, qh, s[w], 0, 0, 0);
+      }
+    }
+    s[0] *= 1.0f / kOpScale;
+    s[1] *= 1.0f / kOpScale;
+    const half8_t pa = softmax_step(s, kp.q_tokens + ru * kUnit, n_valid);
+#pragma unroll
+    for (int cs = 0; cs < 2 * KK; ++cs) {
+      half8_t bv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        bv[e] = (_Float16)(float)rv[(int64_t)min(8 * j + e, n_valid - 1) * D + 32 * (cs / 2) + 2 * r + (cs & 1)];
+      o_acc[cs] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, bv, o_acc[cs], 0, 0, 0);
+    }
+  };
+  for (; u < u_end; u += 4) {
+    if (kp.res_f16) residual_unit((_Float16)0, u - q_units);
+    else residual_unit(0.0f, u - q_units);
   }
 
   // ---- merge: lane groups (row sum), then the 4 waves through LDS --------------------------------
@@ -328,9 +419,10 @@ __global__ __launch_bounds__(256) void kivi_mfma_kernel(const KiviParams kp) {
     lds_l[wave][r] = l_run;
   }
 #pragma unroll
-  for (int a = 0; a < 2 * KK; ++a)
+  for (int cb = 0; cb < KK; ++cb)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_acc[wave][4 * j + i][16 * a + r] = o_acc[a][i];
+    for (int i = 0; i < 4; ++i)
+      *(float2 *)&lds_acc[wave][4 * j + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
   if (r < KK) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
@@ -364,8 +456,7 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   DecodeParams &p = kp.d;
   const int pairs = p.n_heads_kv * batch;
   const int target_wgs = ctx->compute_units * 4;
-  // at least one unit per wave
-  const int max_splits = (kp.units_total + 3) / 4;
+  const int max_splits = (kp.units_total + 3) / 4;  // at least one unit per wave
   int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, kMaxSplits}));
   kp.units_per_split = (kp.units_total + nsplit - 1) / nsplit;
   nsplit = (kp.units_total + kp.units_per_split - 1) / kp.units_per_split;
@@ -377,9 +468,11 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   if (rc != ARGUS_HIP_OK) return rc;
   p.ws_ml = ctx->ws;
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
+  const dim3 grid(nsplit, p.n_heads_kv, batch);
   {
     KernelTimer timer(ctx, stream);
-    hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, kp);
+    if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4>), grid, dim3(256), 0, stream, kp);
+    else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8>), grid, dim3(256), 0, stream, kp);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<NoFallback, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -397,7 +490,7 @@ int launch_dim(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream
 bool kivi_mfma_supported(const KiviParams &kp) {
   const DecodeParams &p = kp.d;
   if (kp.head_dim != 64 && kp.head_dim != 128) return false;
-  if (p.group > 16 || p.softcap > 0.0f) return false;
+  if (p.group > 8 || p.softcap > 0.0f) return false;
   // tiles are copied as 16-byte vectors
   if ((((uintptr_t)kp.qk | (uintptr_t)kp.qv) & 15) || (kp.qk_bs & 15) || (kp.qv_bs & 15)) return false;
   return true;
