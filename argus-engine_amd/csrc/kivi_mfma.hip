@@ -60,6 +60,14 @@ __device__ __forceinline__ half8_t row_shl(half8_t v) {
   for (int i = 0; i < 4; ++i) w[i] = row_shl<SHIFT>(w[i]);
   return __builtin_bit_cast(half8_t, w);
 }
+// Lanes of the banks (groups of 4 lanes) in BANKS take the value of lane i - SHIFT; the rest keep theirs.
+template <int SHIFT, int BANKS>
+__device__ __forceinline__ half8_t row_shr_into(half8_t v) {
+  u32x4_t w = __builtin_bit_cast(u32x4_t, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)w[i], (int)w[i], 0x110 + SHIFT, 0xf, BANKS, false);
+  return __builtin_bit_cast(half8_t, w);
+}
 template <int SHIFT>
 __device__ __forceinline__ float row_shl_add(float x) {
   if constexpr (SHIFT > 0 && SHIFT < 16) x += __builtin_bit_cast(float, row_shl<SHIFT>(__builtin_bit_cast(uint32_t, x)));
@@ -72,28 +80,42 @@ template <int BITS>
 __device__ __forceinline__ int field_offset(int r) {
   return 4 + (BITS == 8 ? 2 * r : BITS == 4 ? r : (r >> 1));
 }
+// Reads of two consecutive contraction slots land in the two halves of one register (the second
+// as a load into the high half), ready to be masked into a packed f16x2 operand word per owned code.
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
 template <int BITS>
-__device__ __forceinline__ uint32_t field_read(const uint8_t *p) {
-  if constexpr (BITS == 8) return *(const uint16_t *)p;
-  else return *p;
+__device__ __forceinline__ uint32_t field_read2(const uint8_t *p0, const uint8_t *p1) {
+  u16x2_t t;
+  if constexpr (BITS == 8) {
+    t[0] = *(const uint16_t *)p0;
+    t[1] = *(const uint16_t *)p1;
+  } else {
+    t[0] = *p0;
+    t[1] = *p1;
+  }
+  return __builtin_bit_cast(uint32_t, t);
 }
-// Two reads (consecutive contraction slots) -> one packed f16x2 operand word per owned code.
+__device__ __forceinline__ uint32_t half_read2(const uint8_t *p0, const uint8_t *p1) {
+  u16x2_t t;
+  t[0] = *(const uint16_t *)p0;
+  t[1] = *(const uint16_t *)p1;
+  return __builtin_bit_cast(uint32_t, t);
+}
 // The matrix core multiplies subnormal halves exactly but keeps product bits relative to the
 // operand's exponent, not its leading one: a field in the lowest mantissa bits loses that many bits
 // of the sum (measured: 2^-20 relative for a 4-bit field at bit 0, 2^-24 at bit 4).  So every field
 // is moved up to end at mantissa bit 7 or 9 first; `presh` is that left shift (lane-dependent for Q2,
 // whose field sits in either nibble of its byte).
 template <int BITS>
-__device__ __forceinline__ void field_pair(uint32_t x0, uint32_t x1, int presh, uint32_t &w0, uint32_t &w1) {
+__device__ __forceinline__ void field_pair(uint32_t v, int presh, uint32_t &w0, uint32_t &w1) {
   if constexpr (BITS == 8) {
-    w0 = __builtin_amdgcn_perm(x1, x0, 0x0c040c00u);  // [x0.b0, 0, x1.b0, 0]
-    w1 = __builtin_amdgcn_perm(x1, x0, 0x0c050c01u);  // [x0.b1, 0, x1.b1, 0]
+    w0 = v & 0x00ff00ffu;
+    w1 = __builtin_amdgcn_perm(v, v, 0x0c030c01u);  // [v.b1, 0, v.b3, 0]
   } else if constexpr (BITS == 4) {
-    const uint32_t v = x0 | (x1 << 16);
     w0 = (v << 4) & 0x00f000f0u;
     w1 = v & 0x00f000f0u;
   } else {
-    const uint32_t v = (x0 | (x1 << 16)) << presh;
+    v <<= presh;
     w0 = v & 0x00c000c0u;
     w1 = v & 0x03000300u;
   }
@@ -111,7 +133,7 @@ constexpr float kOpScale = 64.0f;
 constexpr float kCodeUnit = 16777216.0f;  // a raw code field n is the half n * 2^-24
 
 template <int BITS, int D, int GT>
-__global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) {
+__global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) {
   constexpr int BB = 4 + 32 * BITS / 8;  // block bytes
   constexpr int KK = D / 32;             // 32-channel slices == V blocks per token
   constexpr int TILE_BYTES = D * BB;     // one K tile == one V tile
@@ -126,7 +148,8 @@ __global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) 
 
   const DecodeParams &p = kp.d;
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // keeps unit indices and tile addresses scalar
   const int j = lane >> 4, r = lane & 15;
   const int ra = r / GT, rh = r % GT;  // slice owner index and head of this lane during preparation
   const int G = p.group;
@@ -217,11 +240,11 @@ __global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) 
 
   // ================================ quantised units ===============================================
   u32x4_t pk[NCH], pv[NCH];
-  auto fetch = [&](int uu) {
-    const int flush = uu / gpf, gif = uu % gpf;
-    const int64_t kblk = ((int64_t)flush * p.n_heads_kv * gpf + (int64_t)kvh * gpf + gif) * D;
-    const int tif0 = (uu * kUnit) % kp.res_cap;
-    const int64_t vblk = (((int64_t)flush * p.n_heads_kv + kvh) * kp.res_cap + tif0) * KK;
+  // The unit to fetch next, as (flush, 32-token group inside the flush); stepped without divisions.
+  int f_flush = u / gpf, f_gif = u % gpf;
+  auto fetch = [&]() {
+    const int64_t kblk = ((int64_t)f_flush * p.n_heads_kv * gpf + (int64_t)kvh * gpf + f_gif) * D;
+    const int64_t vblk = (((int64_t)f_flush * p.n_heads_kv + kvh) * kp.res_cap + f_gif * kUnit) * KK;
     const u32x4_t *ksrc = (const u32x4_t *)(qk_b + kblk * BB);
     const u32x4_t *vsrc = (const u32x4_t *)(qv_b + vblk * BB);
 #pragma unroll
@@ -232,8 +255,13 @@ __global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) 
         pv[c] = __builtin_nontemporal_load(vsrc + i);
       }
     }
+    f_gif += 4;
+    while (f_gif >= gpf) {
+      f_gif -= gpf;
+      ++f_flush;
+    }
   };
-  if (u < uq_end) fetch(u);
+  if (u < uq_end) fetch();
 
   for (; u < uq_end; u += 4) {
     wave_lds_fence();  // the previous unit's reads are done
@@ -246,7 +274,7 @@ __global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) 
       }
     }
     wave_lds_fence();
-    if (u + 4 < uq_end) fetch(u + 4);
+    if (u + 4 < uq_end) fetch();
 
     // ---- this lane's share of q*d (hi + lo) and of sum m*q ----------------------------------------
     half8_t own_h[NS], own_l[NS];
@@ -279,12 +307,12 @@ __global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) 
     s[0] = s[1] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     auto qk_slice = [&](auto kk_c) {
       constexpr int kk = decltype(kk_c)::value;
-      uint32_t x[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = field_read<BITS>(sK + (32 * kk + 8 * j + e) * BB + foff);
       uint32_t w0[4], w1[4];
 #pragma unroll
-      for (int pr = 0; pr < 4; ++pr) field_pair<BITS>(x[2 * pr], x[2 * pr + 1], presh, w0[pr], w1[pr]);
+      for (int pr = 0; pr < 4; ++pr) {
+        const uint8_t *cp = sK + (32 * kk + 8 * j + 2 * pr) * BB + foff;
+        field_pair<BITS>(field_read2<BITS>(cp, cp + BB), presh, w0[pr], w1[pr]);
+      }
       const half8_t a0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
       const half8_t a1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
       const half8_t bh = row_shl<(kk % NREP) * GT>(own_h[kk / NREP]);
@@ -310,36 +338,51 @@ __global__ __launch_bounds__(256, 2) void kivi_mfma_kernel(const KiviParams kp) 
     const half8_t pa = softmax_step(s, u * kUnit, kUnit);
 
     // ---- output: contraction slot e -> token 8j + e -------------------------------------------------
-    const half8_t pa_s = pa * (_Float16)kOpScale;
+    // Like q*d, the p*d operand only has `group` real rows: every lane of the row gets its head's
+    // probabilities, scales them for the V blocks it owns, and hands the result to the head's lane.
+    half8_t pa_all = pa;
+    if constexpr (GT <= 4) pa_all = row_shr_into<4, 0x2>(pa_all);
+    if constexpr (GT <= 8) pa_all = row_shr_into<8, 0xc>(pa_all);
+    const half8_t pa_s = pa_all * (_Float16)kOpScale;
+    half8_t pd_own[NS];
 #pragma unroll
-    for (int cb = 0; cb < KK; ++cb) {
+    for (int s2 = 0; s2 < NS; ++s2) {
+      const int cb = min(ra + s2 * NREP, KK - 1);
       u32x4_t dw;
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint32_t d0 = *(const uint16_t *)(sV + ((8 * j + 2 * pr) * KK + cb) * BB);
-        const uint32_t d1 = *(const uint16_t *)(sV + ((8 * j + 2 * pr + 1) * KK + cb) * BB);
-        dw[pr] = d0 | (d1 << 16);
+        const uint8_t *dp = sV + ((8 * j + 2 * pr) * KK + cb) * BB;
+        dw[pr] = half_read2(dp, dp + KK * BB);
       }
-      const half8_t pd = pa_s * __builtin_bit_cast(half8_t, dw);  // rows = heads: p * d[token][cb]
-      uint32_t y[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) y[e] = field_read<BITS>(sV + ((8 * j + e) * KK + cb) * BB + foff);
+      pd_own[s2] = pa_s * __builtin_bit_cast(half8_t, dw);  // p * d[token][cb]
+    }
+    auto pv_block = [&](auto cb_c) {
+      constexpr int cb = decltype(cb_c)::value;
+      const half8_t pd = row_shl<(cb % NREP) * GT>(pd_own[cb / NREP]);
       uint32_t w0[4], w1[4];
 #pragma unroll
-      for (int pr = 0; pr < 4; ++pr) field_pair<BITS>(y[2 * pr], y[2 * pr + 1], presh, w0[pr], w1[pr]);
+      for (int pr = 0; pr < 4; ++pr) {
+        const uint8_t *cp = sV + ((8 * j + 2 * pr) * KK + cb) * BB + foff;
+        field_pair<BITS>(field_read2<BITS>(cp, cp + KK * BB), presh, w0[pr], w1[pr]);
+      }
       const half8_t b0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
       const half8_t b1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
       o_acc[2 * cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b0, o_acc[2 * cb], 0, 0, 0);
       o_acc[2 * cb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b1, o_acc[2 * cb + 1], 0, 0, 0);
+    };
+    pv_block(std::integral_constant<int, 0>{});
+    pv_block(std::integral_constant<int, 1>{});
+    if constexpr (KK > 2) {
+      pv_block(std::integral_constant<int, 2>{});
+      pv_block(std::integral_constant<int, 3>{});
     }
     // zero-point term: column n = cb holds sum_t p[h][t] m[t][cb]
     u32x4_t mw = {0u, 0u, 0u, 0u};
     if (r < KK) {
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint32_t m0 = *(const uint16_t *)(sV + ((8 * j + 2 * pr) * KK + r) * BB + 2);
-        const uint32_t m1 = *(const uint16_t *)(sV + ((8 * j + 2 * pr + 1) * KK + r) * BB + 2);
-        mw[pr] = m0 | (m1 << 16);
+        const uint8_t *mp = sV + ((8 * j + 2 * pr) * KK + r) * BB + 2;
+        mw[pr] = half_read2(mp, mp + KK * BB);
       }
     }
     m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(half8_t, mw), m_acc, 0, 0, 0);
@@ -455,9 +498,17 @@ template <int BITS, int D>
 int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   DecodeParams &p = kp.d;
   const int pairs = p.n_heads_kv * batch;
-  const int target_wgs = ctx->compute_units * 4;
+  // One round of co-resident workgroups: a second, partly filled round would run at a fraction of
+  // the occupancy the unit loop needs to hide its LDS and HBM latency.
+  static const int wgs_per_cu = [] {
+    int n4 = 0, n8 = 0;
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n4, kivi_mfma_kernel<BITS, D, 4>, 256, 0);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n8, kivi_mfma_kernel<BITS, D, 8>, 256, 0);
+    return std::max(1, std::min(n4, n8));
+  }();
+  const int slots = ctx->compute_units * wgs_per_cu;
   const int max_splits = (kp.units_total + 3) / 4;  // at least one unit per wave
-  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, kMaxSplits}));
+  int nsplit = std::max(1, std::min({slots / pairs, max_splits, kMaxSplits}));
   kp.units_per_split = (kp.units_total + nsplit - 1) / nsplit;
   nsplit = (kp.units_total + kp.units_per_split - 1) / kp.units_per_split;
   p.nsplit = nsplit;
