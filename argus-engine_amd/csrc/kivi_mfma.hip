@@ -80,11 +80,12 @@ template <int BITS>
 __device__ __forceinline__ int field_offset(int r) {
   return 4 + (BITS == 8 ? 2 * r : BITS == 4 ? r : (r >> 1));
 }
-// Reads of two consecutive contraction slots land in the two halves of one register (the second
-// as a load into the high half), ready to be masked into a packed f16x2 operand word per owned code.
-typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+// Reads of two consecutive contraction slots, packed into the two halves of one word.  (Loads
+// into the high half of a register do not keep the low half on this target, so the pair is
+// packed with a byte permute.)
 template <int BITS>
 __device__ __forceinline__ uint32_t field_read2(const uint8_t *p0, const uint8_t *p1) {
+  typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
   u16x2_t t;
   if constexpr (BITS == 8) {
     t[0] = *(const uint16_t *)p0;
@@ -96,34 +97,47 @@ __device__ __forceinline__ uint32_t field_read2(const uint8_t *p0, const uint8_t
   return __builtin_bit_cast(uint32_t, t);
 }
 __device__ __forceinline__ uint32_t half_read2(const uint8_t *p0, const uint8_t *p1) {
+  typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
   u16x2_t t;
   t[0] = *(const uint16_t *)p0;
   t[1] = *(const uint16_t *)p1;
   return __builtin_bit_cast(uint32_t, t);
 }
+// Packed pair word -> the f16x2 operand words of the two codes of the field.
 // The matrix core multiplies subnormal halves exactly but keeps product bits relative to the
 // operand's exponent, not its leading one: a field in the lowest mantissa bits loses that many bits
-// of the sum (measured: 2^-20 relative for a 4-bit field at bit 0, 2^-24 at bit 4).  So every field
-// is moved up to end at mantissa bit 7 or 9 first; `presh` is that left shift (lane-dependent for Q2,
-// whose field sits in either nibble of its byte).
-template <int BITS>
+// of the sum (measured: 2^-20 relative for a 4-bit field at bit 0, 2^-24 at bit 4).  The logits need
+// the full f32 accuracy, so with PRECISE every field is first moved up to end at mantissa bit 7 or
+// 9 (`presh`: that left shift, lane-dependent for Q2, whose field sits in either nibble of its
+// byte); the output sums do not, and take the fields where they are.
+template <int BITS, bool PRECISE>
 __device__ __forceinline__ void field_pair(uint32_t v, int presh, uint32_t &w0, uint32_t &w1) {
   if constexpr (BITS == 8) {
     w0 = v & 0x00ff00ffu;
     w1 = __builtin_amdgcn_perm(v, v, 0x0c030c01u);  // [v.b1, 0, v.b3, 0]
   } else if constexpr (BITS == 4) {
-    w0 = (v << 4) & 0x00f000f0u;
+    w0 = PRECISE ? ((v << 4) & 0x00f000f0u) : (v & 0x000f000fu);
     w1 = v & 0x00f000f0u;
-  } else {
+  } else if constexpr (PRECISE) {
     v <<= presh;
     w0 = v & 0x00c000c0u;
     w1 = v & 0x03000300u;
+  } else {
+    // presh = 6 (low nibble) or 2 (high nibble): masks 0x3 / 0xc shifted to the field's nibble
+    const uint32_t m0 = (0x00c000c0u >> presh), m1 = (0x03000300u >> presh);
+    w0 = v & m0;
+    w1 = v & m1;
   }
 }
 // Bit position of code `which` (0 / 1) inside the operand half.
 template <int BITS>
 __host__ __device__ constexpr int field_shift(int which) {
   return BITS == 8 ? 0 : BITS == 4 ? 4 : 6 + 2 * which;
+}
+// Same for the fields of the output sums, which stay in place (Q2: on top of the lane's 2^-presh).
+template <int BITS>
+__host__ __device__ constexpr int field_shift_v(int which) {
+  return BITS == 8 ? 0 : BITS == 4 ? 4 * which : 6 + 2 * which;
 }
 
 constexpr float kLn2 = 0.6931471805599453f;
@@ -139,7 +153,12 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
   constexpr int TILE_BYTES = D * BB;     // one K tile == one V tile
   constexpr int TILE_VEC = TILE_BYTES / 16;
   constexpr int NCH = (TILE_VEC + 63) / 64;
-  constexpr int WAVE_BYTES = 2 * TILE_BYTES;
+  // In LDS the V tile gets 16 bytes of padding after every 8 tokens: a lane group j reads tokens
+  // 8j..8j+7, and the unpadded stride of 8 tokens is a multiple of 128 bytes for head_dim 128, which
+  // would put groups j and j+2 on the same banks.
+  constexpr int VPAD = 16;
+  constexpr int V8_VEC = 8 * KK * BB / 16;  // 16-byte vectors per 8 tokens
+  constexpr int WAVE_BYTES = 2 * TILE_BYTES + 4 * VPAD;
   constexpr int MERGE_BYTES = 4 * 16 * (D + 4) * 4 + 4 * 16 * KK * 4 + 2 * 4 * 16 * 4;
   constexpr int SMEM = (4 * WAVE_BYTES > MERGE_BYTES) ? 4 * WAVE_BYTES : MERGE_BYTES;
   constexpr int NREP = 16 / GT;               // lanes of a row that share one head
@@ -158,6 +177,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
 
   uint8_t *sK = smem + wave * WAVE_BYTES;
   uint8_t *sV = sK + TILE_BYTES;
+  const uint8_t *sVj = sV + j * (8 * KK * BB + VPAD);  // this lane group's 8 tokens
   const uint8_t *qk_b = kp.qk + (int64_t)b * kp.qk_bs;
   const uint8_t *qv_b = kp.qv + (int64_t)b * kp.qv_bs;
   const float qscale = p.scale * 1.4426950408889634f * kOpScale;  // log2 domain
@@ -270,7 +290,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
       const int i = lane + 64 * c;
       if (i < TILE_VEC) {
         ((u32x4_t *)sK)[i] = pk[c];
-        ((u32x4_t *)sV)[i] = pv[c];
+        ((u32x4_t *)sV)[i + i / V8_VEC] = pv[c];
       }
     }
     wave_lds_fence();
@@ -311,7 +331,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
         const uint8_t *cp = sK + (32 * kk + 8 * j + 2 * pr) * BB + foff;
-        field_pair<BITS>(field_read2<BITS>(cp, cp + BB), presh, w0[pr], w1[pr]);
+        field_pair<BITS, true>(field_read2<BITS>(cp, cp + BB), presh, w0[pr], w1[pr]);
       }
       const half8_t a0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
       const half8_t a1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
@@ -351,7 +371,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
       u32x4_t dw;
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint8_t *dp = sV + ((8 * j + 2 * pr) * KK + cb) * BB;
+        const uint8_t *dp = sVj + (2 * pr * KK + cb) * BB;
         dw[pr] = half_read2(dp, dp + KK * BB);
       }
       pd_own[s2] = pa_s * __builtin_bit_cast(half8_t, dw);  // p * d[token][cb]
@@ -362,8 +382,8 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
       uint32_t w0[4], w1[4];
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint8_t *cp = sV + ((8 * j + 2 * pr) * KK + cb) * BB + foff;
-        field_pair<BITS>(field_read2<BITS>(cp, cp + KK * BB), presh, w0[pr], w1[pr]);
+        const uint8_t *cp = sVj + (2 * pr * KK + cb) * BB + foff;
+        field_pair<BITS, false>(field_read2<BITS>(cp, cp + KK * BB), presh, w0[pr], w1[pr]);
       }
       const half8_t b0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
       const half8_t b1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
@@ -381,7 +401,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
     if (r < KK) {
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint8_t *mp = sV + ((8 * j + 2 * pr) * KK + r) * BB + 2;
+        const uint8_t *mp = sVj + (2 * pr * KK + r) * BB + 2;
         mw[pr] = half_read2(mp, mp + KK * BB);
       }
     }
@@ -389,10 +409,11 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
   }
 
   // The code sums carry the field position and the operand units.
+  const float v_unit = (BITS == 2) ? (float)(1 << presh) : 1.0f;  // Q2 fields sit 2^-presh below bit 6
 #pragma unroll
   for (int cb = 0; cb < KK; ++cb) {
-    o_acc[2 * cb] *= kCodeUnit / (kOpScale * (float)(1 << field_shift<BITS>(0)));
-    o_acc[2 * cb + 1] *= kCodeUnit / (kOpScale * (float)(1 << field_shift<BITS>(1)));
+    o_acc[2 * cb] *= v_unit * (kCodeUnit / (kOpScale * (float)(1 << field_shift_v<BITS>(0))));
+    o_acc[2 * cb + 1] *= v_unit * (kCodeUnit / (kOpScale * (float)(1 << field_shift_v<BITS>(1))));
   }
 
   // ================================ residual window ===============================================
