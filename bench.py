@@ -196,6 +196,12 @@ def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
                       "restated CpuBackendAVX2::attention_gen, one task per Q head" % (len(times), med * 1e6)}
 
 
+# HBM bytes per launch of the primary workload's kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs
+# scaled by what the same counters read for a plain 1 GiB copy (x2.000 and x1.000); the runs and
+# their commands are summarised in profiles/decode_mfma_cfg3_L32768_b16_hbm_traffic.md.
+DECODE_TRAFFIC_BYTES = 2_191_763_046
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -204,7 +210,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
-                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5"],
+                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "copy_calib"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -222,7 +228,15 @@ def main():
 
     if args.workload != "primary":
         w = args.workload
-        if w == "decode_b1":
+        if w == "copy_calib":
+            # plain 1 GiB device copy: the known-size reference the HBM traffic counters are scaled by
+            src = torch.ones(1 << 28, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(args.warmup + args.steps):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            res = {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}
+        elif w == "decode_b1":
             res = bench_decode(ctx, 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=4)
         elif w == "prefill":
             res = bench_prefill(ctx, args.steps, args.warmup)
@@ -257,8 +271,8 @@ def main():
                    "us_per_call": round(r["ms_per_step"] * 1e3, 2),
                    "tokens_per_s": round(batch / (r["ms_per_step"] * 1e-3), 1)},
         "roofline": {"bound": "hbm", "achieved": round(r["gbps_kernel"], 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(r["gbps_kernel"] / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "decode_split_kernel<128,4,f16>", "kernel_ms": round(r["kernel_ms"], 5),
+                     "unit": "GB/s", "frac": round(r["gbps_kernel"] / HBM_PEAK_GBPS, 4), "traffic": DECODE_TRAFFIC_BYTES,
+                     "kernel": "decode_mfma_kernel<128,2>", "kernel_ms": round(r["kernel_ms"], 5),
                      "algorithmic_bytes": r["bytes"]},
         "device": {"name": info.name.decode(), "arch": info.gcn_arch.decode(), "cus": info.compute_units,
                    "clock_mhz": info.clock_mhz},
@@ -287,9 +301,9 @@ def main():
         add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")
         add("cfg4_kivi_q4_L8192_res128_f16", bench_kivi(ctx, 4, es, ew, res_f16=True), "F16 residual window")
         add("cfg4_kivi_q4_x32_caches", bench_kivi(ctx, 4, es, ew, batch=32, rotate=2),
-            "32 caches (layers) per launch, 365 MB: amortised rate")
+            "32 caches (sequences) per launch, 365 MB: amortised rate")
         add("cfg4_kivi_q8_x32_caches", bench_kivi(ctx, 8, es, ew, batch=32, rotate=2),
-            "32 caches (layers) per launch, 629 MB: amortised rate")
+            "32 caches (sequences) per launch, 629 MB: amortised rate")
         ex["cfg2_prefill_llama1b_S2048_f16"] = bench_prefill(ctx, es, ew)
         ex["cfg2_prefill_llama1b_S2048_f32io"] = bench_prefill(ctx, es, ew, f16_io=False)
         ex["prefill_llama8b_d128_S8192_f16"] = bench_prefill(ctx, max(5, es // 4), 2, hq=32, hkv=8, d=128, s=8192)
