@@ -38,6 +38,13 @@ struct PrefillParams {
   float scale_log2e;
 };
 
+// Transposing LDS read (ds_read_b64_tr_b16), see its use below.
+__device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *p) {
+  typedef short short4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+  return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)p));
+}
+
 template <typename KV_T>
 __device__ __forceinline__ half8_t load_kv_chunk(const KV_T *p);
 template <>
@@ -61,8 +68,11 @@ template <int D>
 struct PrefillTile {
   static constexpr int BN = (D <= 128) ? 64 : 32;  // keys per tile
   static constexpr int KP = D + 8;                 // K tile row pitch (halfs)
-  static constexpr int VP = BN + 4;                // V^T tile row pitch (halfs), keeps 8-byte alignment
-  static constexpr int HALFS = BN * KP + D * VP;   // halfs per (K, V^T) tile pair
+  // V tile row pitch (halfs): an odd multiple of 16 dwords, so that the 4 rows x 32 bytes a
+  // 16-lane group touches in one transposing read, and the neighbouring group's 32 bytes next to
+  // them, all fall on different banks.
+  static constexpr int VP = D + 32;
+  static constexpr int HALFS = BN * KP + BN * VP;  // halfs per (K, V) tile pair
 };
 
 template <int D, int HPW, int NG, typename KV_T>
@@ -136,132 +146,178 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
   const KV_T *vbase = (const KV_T *)p.v + ((int64_t)b * p.n_heads_kv + kvh) * p.capacity * D;
 
   // Iteration `it` covers tiles kt_begin + it*NG + g for g < NG (tile g is consumed by KV group g).
+  // Software pipeline inside each wave: the S^T MFMAs of iteration it+1 are issued before the
+  // softmax of iteration it, so the matrix core works while the vector ALU does the exponentials.
+  // That needs K one iteration further ahead than V: K tiles are staged two iterations ahead into
+  // sKb[it & 1], V^T tiles one ahead into sVb[it & 1]; in iteration `it` the waves read
+  // sKb[(it+1) & 1] and sVb[it & 1] and fill sKb[it & 1] and sVb[(it+1) & 1], so one barrier per
+  // iteration still separates every fill from the reads before and after it.
+  _Float16 *const sKb = smem;                         // [2][NG][BN * KP]
+  _Float16 *const sVb = smem + 2 * NG * BN * KP;      // [2][NG][BN * VP]
   half8_t kpre[CH], vpre[CH];
-  auto fetch = [&](int it) {
+  auto fetch_k = [&](int it) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int cid = threadIdx.x + NT * c;
       const int key = (kt_begin + it * NG) * BN + cid / (D / 8), dc = cid % (D / 8);
-      half8_t kx = {0, 0, 0, 0, 0, 0, 0, 0}, vx = kx;
-      if (key < kv_end) {
-        kx = load_kv_chunk<KV_T>(kbase + (int64_t)key * D + 8 * dc);
-        vx = load_kv_chunk<KV_T>(vbase + (int64_t)key * D + 8 * dc);
-      }
+      half8_t kx = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (key < kv_end) kx = load_kv_chunk<KV_T>(kbase + (int64_t)key * D + 8 * dc);
       kpre[c] = kx;
+    }
+  };
+  auto fetch_v = [&](int it) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int cid = threadIdx.x + NT * c;
+      const int key = (kt_begin + it * NG) * BN + cid / (D / 8), dc = cid % (D / 8);
+      half8_t vx = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (key < kv_end) vx = load_kv_chunk<KV_T>(vbase + (int64_t)key * D + 8 * dc);
       vpre[c] = vx;
     }
   };
-  auto stage = [&](int buf) {
+  auto stage_k = [&](int buf) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int cid = threadIdx.x + NT * c;
       const int trow = cid / (D / 8), dc = cid % (D / 8);
       const int g = trow / BN, key = trow % BN;
-      _Float16 *sK = smem + (buf * NG + g) * TL::HALFS;
-      _Float16 *sVt = sK + BN * KP;
-      *(half8_t *)(sK + key * KP + 8 * dc) = kpre[c];
+      *(half8_t *)(sKb + (buf * NG + g) * (BN * KP) + key * KP + 8 * dc) = kpre[c];
+    }
+  };
+  auto stage_v = [&](int buf) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sVt[(8 * dc + e) * VP + key] = vpre[c][e];
+    for (int c = 0; c < CH; ++c) {
+      const int cid = threadIdx.x + NT * c;
+      const int trow = cid / (D / 8), dc = cid % (D / 8);
+      const int g = trow / BN, key = trow % BN;
+      *(half8_t *)(sVb + (buf * NG + g) * (BN * VP) + key * VP + 8 * dc) = vpre[c];
     }
   };
 
-  if (n_it > 0) {
-    fetch(0);
-    stage(0);
-  }
-  __syncthreads();
-  for (int it = 0; it < n_it; ++it) {
-    if (it + 1 < n_it) fetch(it + 1);
-
+  // Does this wave have anything to do with its tile of iteration `it`?
+  const int wave_hi = r0 + 31 + p.q_start;  // largest visible key of the wave
+  const int wave_lo = p.window > 0 ? (r0 + p.q_start - p.window + 1) : 0;
+  auto tile_active = [&](int it) {
     const int kt = kt_begin + it * NG + kvg;
     const int key0 = kt * BN;
-    // Waves whose rows cannot see their tile skip the math (they still take part in the barrier).
-    const int wave_hi = r0 + 31 + p.q_start;  // largest visible key of the wave
-    const int wave_lo = p.window > 0 ? (r0 + p.q_start - p.window + 1) : 0;
-    if (kt < kt_end && r0 < p.seq_len && key0 <= wave_hi && key0 + BN > wave_lo) {
-      const _Float16 *sK = smem + ((it & 1) * NG + kvg) * TL::HALFS;
-      const _Float16 *sVt = sK + BN * KP;
-
-      // ---- S^T = K . Q^T ----------------------------------------------------------------------
-      float16_t s_acc[KB];
+    return it < n_it && kt < kt_end && r0 < p.seq_len && key0 <= wave_hi && key0 + BN > wave_lo;
+  };
+  // S^T = K . Q^T for this wave's tile of iteration `it`
+  auto qk_tile = [&](int it, float16_t(&s_acc)[KB]) {
+    const _Float16 *sK = sKb + ((it & 1) * NG + kvg) * (BN * KP);
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_acc[kb][i] = 0.0f;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
+        s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
+      }
+  };
+  // mask, online softmax and O^T += V^T . P^T for the tile of iteration `it`, whose logits are in s_acc
+  auto softmax_pv_tile = [&](int it, float16_t(&s_acc)[KB]) {
+    const int key0 = (kt_begin + it * NG + kvg) * BN;
+    // V stays row major in LDS.  The A operand of O^T = V^T . P^T wants, per lane, 8 keys of one
+    // channel: ds_read_b64_tr_b16 delivers exactly that transposition.  In a group of 16 lanes,
+    // lane 4q + c receives element c of the 8-byte rows addressed by lanes q, 4 + q, 8 + q, 12 + q;
+    // with lane s addressing V[key0 + s / 4][ch0 + 4 (s % 4) ..], lane i gets channel ch0 + i of
+    // keys key0 .. key0 + 3.  Lane groups 0..3 are (channels 0-15 | 16-31) x (lane half 0 | 1); P^T has
+    // keys 4 hl + {0..3} and 8 + 4 hl + {0..3} of each 16 in the contraction slots of lane half hl.
+    const _Float16 *sV = sVb + ((it & 1) * NG + kvg) * (BN * VP);
+    const int g16 = lane >> 4, s16 = lane & 15;
+    const _Float16 *vlane = sV + (4 * (g16 >> 1) + (s16 >> 2)) * VP + 16 * (g16 & 1) + 4 * (s16 & 3);
+    // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) ---------
+    const int q_pos = row + p.q_start;
+    const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
+                           (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
+    if (need_mask) {
+      const int lo = p.window > 0 ? q_pos - p.window : -1;  // keys <= lo are outside the window
+      const int hi = min(q_pos, p.cache_len - 1);
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_acc[kb][i] = 0.0f;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
-          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + 32 * kb + 8 * (i / 4) + 4 * hl + (i % 4);
+          s_acc[kb][i] = (key <= hi && key > lo) ? s_acc[kb][i] : kNegInf;
         }
-
-      // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) -------
-      const int q_pos = row + p.q_start;
-      const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
-                             (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
-      if (need_mask) {
-        const int lo = p.window > 0 ? q_pos - p.window : -1;  // keys <= lo are outside the window
-        const int hi = min(q_pos, p.cache_len - 1);
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = key0 + 32 * kb + 8 * (i / 4) + 4 * hl + (i % 4);
-            s_acc[kb][i] = (key <= hi && key > lo) ? s_acc[kb][i] : kNegInf;
-          }
-      }
-
-      // ---- online softmax for this lane's query column --------------------------------------
-      float mt = kNegInf;
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-      const float m_new = fmaxf(m_run, mt * p.scale_log2e);
-      const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-      m_run = m_new;
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          s_acc[kb][i] = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][i], p.scale_log2e, -m_ref));
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
-      }
-
-      // ---- O^T += V^T . P^T ------------------------------------------------------------------
-      // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
-      // rounding cancels in the final normalisation.
-      float lsum = 0.0f;
-#pragma unroll
-      for (int jn = 0; jn < BN / 16; ++jn) {
-        half8_t pb;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pb[e] = (_Float16)s_acc[jn / 2][8 * (jn % 2) + e];
-#pragma unroll
-        for (int e = 0; e < 8; e += 2) {
-          const half2_t pr = {pb[e], pb[e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
-          lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
-        }
-#pragma unroll
-        for (int r = 0; r < RB; ++r) {
-          const _Float16 *vrow = sVt + (32 * r + ln) * VP + 16 * jn + 4 * hl;
-          const half4_t lo = *(const half4_t *)vrow, hi = *(const half4_t *)(vrow + 8);
-          const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, o_acc[r], 0, 0, 0);
-        }
-      }
-      l_run = l_run * alpha + lsum;
     }
+    // ---- online softmax for this lane's query column ----------------------------------------
+    float mt = kNegInf;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m_run, mt * p.scale_log2e);
+    const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+    m_run = m_new;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        s_acc[kb][i] = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][i], p.scale_log2e, -m_ref));
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
+    }
+    // ---- O^T += V^T . P^T --------------------------------------------------------------------
+    // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
+    // rounding cancels in the final normalisation.
+    float lsum = 0.0f;
+#pragma unroll
+    for (int jn = 0; jn < BN / 16; ++jn) {
+      half8_t pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pb[e] = (_Float16)s_acc[jn / 2][8 * (jn % 2) + e];
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const half2_t pr = {pb[e], pb[e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
+        lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
+      }
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const _Float16 *vp = vlane + (16 * jn) * VP + 32 * r;
+        const half4_t lo = lds_read_tr16(vp), hi = lds_read_tr16(vp + 8 * VP);
+        const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, o_acc[r], 0, 0, 0);
+      }
+    }
+    l_run = l_run * alpha + lsum;
+  };
+  // One pipeline step: logits of iteration it+1 into s_next while iteration it is finished from s_cur.
+  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB]) {
+    if (it + 2 < n_it) fetch_k(it + 2);
+    if (it + 1 < n_it) fetch_v(it + 1);
+    if (tile_active(it + 1)) qk_tile(it + 1, s_next);
+    if (tile_active(it)) softmax_pv_tile(it, s_cur);
+    if (it + 2 < n_it) stage_k(it & 1);
+    if (it + 1 < n_it) stage_v((it + 1) & 1);
+    __syncthreads();  // fills are visible; every wave is done with the buffers the next step refills
+  };
 
-    if (it + 1 < n_it) stage((it + 1) & 1);
-    __syncthreads();  // next buffer is filled; every wave is done with the current one
+  float16_t s_a[KB], s_b[KB];
+  if (n_it > 0) {
+    fetch_k(0);
+    fetch_v(0);
+    stage_k(0);
+    stage_v(0);
+    if (n_it > 1) {
+      fetch_k(1);
+      stage_k(1);
+    }
+  }
+  __syncthreads();
+  if (tile_active(0)) qk_tile(0, s_a);
+  __syncthreads();  // sKb[0] is refilled by the first step
+  for (int it = 0; it < n_it; it += 2) {
+    step(it, s_a, s_b);
+    if (it + 1 < n_it) step(it + 1, s_b, s_a);
   }
 
   // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
