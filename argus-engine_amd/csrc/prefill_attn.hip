@@ -21,6 +21,8 @@
 //    pairing a long and a short tile on each compute unit.
 #include "argus_hip_internal.hpp"
 
+#include <type_traits>
+
 namespace {
 
 typedef float float16_t __attribute__((ext_vector_type(16)));
@@ -85,6 +87,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
   constexpr int KB = BN / 32;                // S^T row blocks (32 keys each)
   constexpr int RB = D / 32;                 // O^T row blocks (32 channels each)
   constexpr int CH = NG * BN * D / 8 / NT;   // 16-byte chunks per thread per iteration
+  constexpr int kLdsAhead = 4;               // MFMA operand reads kept in flight
 
   // [2 buffers][NG tiles][K tile | V^T tile]; reused at the end for the cross-group merge.
   extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
@@ -216,9 +219,19 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
         const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
         s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
       }
+    // Keep kLdsAhead operand reads in flight ahead of the MFMA that consumes them: one LDS round
+    // trip per MFMA is several times the MFMA's own 32 cycles.
+    __builtin_amdgcn_sched_group_barrier(0x100, kLdsAhead, 0);
+#pragma unroll
+    for (int i = 0; i < KK * KB - kLdsAhead; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLdsAhead, 0);
   };
   // mask, online softmax and O^T += V^T . P^T for the tile of iteration `it`, whose logits are in s_acc
-  auto softmax_pv_tile = [&](int it, float16_t(&s_acc)[KB]) {
+  auto softmax_pv_tile = [&](int it, float16_t(&s_acc)[KB], auto interior_c) {
+    constexpr bool INTERIOR = decltype(interior_c)::value;
     const int key0 = (kt_begin + it * NG + kvg) * BN;
     // V stays row major in LDS.  The A operand of O^T = V^T . P^T wants, per lane, 8 keys of one
     // channel: ds_read_b64_tr_b16 delivers exactly that transposition.  In a group of 16 lanes,
@@ -231,8 +244,8 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
     const _Float16 *vlane = sV + (4 * (g16 >> 1) + (s16 >> 2)) * VP + 16 * (g16 & 1) + 4 * (s16 & 3);
     // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) ---------
     const int q_pos = row + p.q_start;
-    const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
-                           (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
+    const bool need_mask = !INTERIOR && ((key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
+                                         (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1));
     if (need_mask) {
       const int lo = p.window > 0 ? q_pos - p.window : -1;  // keys <= lo are outside the window
       const int hi = min(q_pos, p.cache_len - 1);
@@ -291,11 +304,15 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
     l_run = l_run * alpha + lsum;
   };
   // One pipeline step: logits of iteration it+1 into s_next while iteration it is finished from s_cur.
-  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB]) {
+  // Interior steps (every tile of the iteration lies below the diagonal of every wave, inside the
+  // cache and the window, and there is a next iteration) have no per-wave conditions: the logits
+  // MFMAs of the next tile and the softmax of the current one sit in one basic block and interleave.
+  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], auto interior_c) {
+    constexpr bool INTERIOR = decltype(interior_c)::value;
     if (it + 2 < n_it) fetch_k(it + 2);
-    if (it + 1 < n_it) fetch_v(it + 1);
-    if (tile_active(it + 1)) qk_tile(it + 1, s_next);
-    if (tile_active(it)) softmax_pv_tile(it, s_cur);
+    if (INTERIOR || it + 1 < n_it) fetch_v(it + 1);
+    if (INTERIOR || it + 1 < n_it) qk_tile(it + 1, s_next);  // harmless on a tile the wave cannot see
+    if (INTERIOR || tile_active(it)) softmax_pv_tile(it, s_cur, interior_c);
     if (it + 2 < n_it) stage_k(it & 1);
     if (it + 1 < n_it) stage_v((it + 1) & 1);
     __syncthreads();  // fills are visible; every wave is done with the buffers the next step refills
@@ -313,11 +330,22 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
     }
   }
   __syncthreads();
-  if (tile_active(0)) qk_tile(0, s_a);
+  if (n_it > 0) qk_tile(0, s_a);
   __syncthreads();  // sKb[0] is refilled by the first step
-  for (int it = 0; it < n_it; it += 2) {
-    step(it, s_a, s_b);
-    if (it + 1 < n_it) step(it + 1, s_b, s_a);
+  // leading interior iterations, rounded down to pairs so that s_a holds the current logits after them
+  int n_int = 0;
+  if (p.window == 0) {
+    const int full_keys = min(qt * QPW * 32 + p.q_start + 1, p.cache_len);  // keys every row of the workgroup sees
+    n_int = max(0, min(n_it - 1, (full_keys / BN - kt_begin) / NG)) & ~1;
+  }
+  int it = 0;
+  for (; it < n_int; it += 2) {
+    step(it, s_a, s_b, std::true_type{});
+    step(it + 1, s_b, s_a, std::true_type{});
+  }
+  for (; it < n_it; it += 2) {
+    step(it, s_a, s_b, std::false_type{});
+    if (it + 1 < n_it) step(it + 1, s_b, s_a, std::false_type{});
   }
 
   // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
