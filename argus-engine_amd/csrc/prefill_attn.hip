@@ -229,20 +229,19 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
     }
     __builtin_amdgcn_sched_group_barrier(0x008, kLdsAhead, 0);
   };
-  // mask, online softmax and O^T += V^T . P^T for the tile of iteration `it`, whose logits are in s_acc
-  auto softmax_pv_tile = [&](int it, float16_t(&s_acc)[KB], auto interior_c) {
+  // Per-tile softmax state handed from the phase that finds the maximum to the one that exponentiates.
+  struct TileMax {
+    float m_ref;  // reference the tile's probabilities are taken against (log2 units)
+    float alpha;  // factor the running sums take before this tile is added
+  };
+  // Mask (edge tiles only) and row maximum of the tile of iteration `it`.  The running maximum is
+  // only moved when a row's maximum exceeds it by more than kLazy (log2 units): probabilities then
+  // reach at most 2^kLazy, which f16 and the f32 sums hold easily, and almost every tile leaves the
+  // accumulators unscaled.
+  constexpr float kLazy = 8.0f;
+  auto mask_max = [&](int it, float16_t(&s_acc)[KB], auto interior_c) -> TileMax {
     constexpr bool INTERIOR = decltype(interior_c)::value;
     const int key0 = (kt_begin + it * NG + kvg) * BN;
-    // V stays row major in LDS.  The A operand of O^T = V^T . P^T wants, per lane, 8 keys of one
-    // channel: ds_read_b64_tr_b16 delivers exactly that transposition.  In a group of 16 lanes,
-    // lane 4q + c receives element c of the 8-byte rows addressed by lanes q, 4 + q, 8 + q, 12 + q;
-    // with lane s addressing V[key0 + s / 4][ch0 + 4 (s % 4) ..], lane i gets channel ch0 + i of
-    // keys key0 .. key0 + 3.  Lane groups 0..3 are (channels 0-15 | 16-31) x (lane half 0 | 1); P^T has
-    // keys 4 hl + {0..3} and 8 + 4 hl + {0..3} of each 16 in the contraction slots of lane half hl.
-    const _Float16 *sV = sVb + ((it & 1) * NG + kvg) * (BN * VP);
-    const int g16 = lane >> 4, s16 = lane & 15;
-    const _Float16 *vlane = sV + (4 * (g16 >> 1) + (s16 >> 2)) * VP + 16 * (g16 & 1) + 4 * (s16 & 3);
-    // ---- mask (only tiles that touch the diagonal, the window edge or the cache end) ---------
     const int q_pos = row + p.q_start;
     const bool need_mask = !INTERIOR && ((key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
                                          (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1));
@@ -257,64 +256,87 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
           s_acc[kb][i] = (key <= hi && key > lo) ? s_acc[kb][i] : kNegInf;
         }
     }
-    // ---- online softmax for this lane's query column ----------------------------------------
     float mt = kNegInf;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m_run, mt * p.scale_log2e);
-    const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * p.scale_log2e;
+    const float m_new = (mt > m_run + kLazy) ? mt : m_run;  // also takes the first finite maximum
+    TileMax t;
+    t.m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+    t.alpha = __builtin_amdgcn_exp2f(m_run - t.m_ref);
     m_run = m_new;
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        s_acc[kb][i] = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][i], p.scale_log2e, -m_ref));
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+    return t;
+  };
+  // Probabilities of the current tile (exp2 against t.m_ref), rounded to f16 in P^T operand order.
+  half8_t pb[BN / 16];
+  auto exp_tile = [&](float16_t(&s_acc)[KB], const TileMax &t) {
+    if (__builtin_amdgcn_ballot_w64(t.alpha != 1.0f) != 0) {
 #pragma unroll
       for (int r = 0; r < RB; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
+        for (int i = 0; i < 16; ++i) o_acc[r][i] *= t.alpha;
+      l_run *= t.alpha;
     }
-    // ---- O^T += V^T . P^T --------------------------------------------------------------------
     // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
     // rounding cancels in the final normalisation.
     float lsum = 0.0f;
 #pragma unroll
     for (int jn = 0; jn < BN / 16; ++jn) {
-      half8_t pb;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pb[e] = (_Float16)s_acc[jn / 2][8 * (jn % 2) + e];
+      for (int e = 0; e < 8; ++e)
+        pb[jn][e] = (_Float16)__builtin_amdgcn_exp2f(fmaf(s_acc[jn / 2][8 * (jn % 2) + e], p.scale_log2e, -t.m_ref));
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
-        const half2_t pr = {pb[e], pb[e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
+        const half2_t pr = {pb[jn][e], pb[jn][e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
         lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
       }
+    }
+    l_run += lsum;
+  };
+  // O^T += V^T . P^T for the tile of iteration `it`.
+  // V stays row major in LDS.  The A operand wants, per lane, 8 keys of one channel:
+  // ds_read_b64_tr_b16 delivers exactly that transposition.  In a group of 16 lanes, lane 4q + c
+  // receives element c of the 8-byte rows addressed by lanes q, 4 + q, 8 + q, 12 + q; with lane s
+  // addressing V[key0 + s / 4][ch0 + 4 (s % 4) ..], lane i gets channel ch0 + i of keys key0 ..
+  // key0 + 3.  Lane groups 0..3 are (channels 0-15 | 16-31) x (lane half 0 | 1); P^T has keys
+  // 4 hl + {0..3} and 8 + 4 hl + {0..3} of each 16 in the contraction slots of lane half hl.
+  const int g16 = lane >> 4, s16 = lane & 15;
+  const int vlane_off = (4 * (g16 >> 1) + (s16 >> 2)) * VP + 16 * (g16 & 1) + 4 * (s16 & 3);
+  auto pv_tile = [&](int it) {
+    const _Float16 *vlane = sVb + ((it & 1) * NG + kvg) * (BN * VP) + vlane_off;
+#pragma unroll
+    for (int jn = 0; jn < BN / 16; ++jn)
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const _Float16 *vp = vlane + (16 * jn) * VP + 32 * r;
         const half4_t lo = lds_read_tr16(vp), hi = lds_read_tr16(vp + 8 * VP);
         const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, o_acc[r], 0, 0, 0);
+        o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[jn], o_acc[r], 0, 0, 0);
       }
-    }
-    l_run = l_run * alpha + lsum;
   };
-  // One pipeline step: logits of iteration it+1 into s_next while iteration it is finished from s_cur.
-  // Interior steps (every tile of the iteration lies below the diagonal of every wave, inside the
-  // cache and the window, and there is a next iteration) have no per-wave conditions: the logits
-  // MFMAs of the next tile and the softmax of the current one sit in one basic block and interleave.
-  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], auto interior_c) {
+
+  // One pipeline step.  On entry s_cur holds the logits of iteration `it` and t_cur their maximum
+  // data.  Phase A issues the logits MFMAs of iteration it+1 while the vector ALU exponentiates
+  // tile `it`; phase B issues the output MFMAs of tile `it` while the vector ALU finds the maximum
+  // of tile it+1.  Interior steps (every tile of the iteration lies below the diagonal of every
+  // wave, inside the cache and the window, and there is a next iteration) have no per-wave
+  // conditions, so each phase is one basic block the scheduler can interleave.
+  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], TileMax &t_cur, auto interior_c) {
     constexpr bool INTERIOR = decltype(interior_c)::value;
+    const bool act = INTERIOR || tile_active(it);
+    const bool has_next = INTERIOR || it + 1 < n_it;
     if (it + 2 < n_it) fetch_k(it + 2);
-    if (INTERIOR || it + 1 < n_it) fetch_v(it + 1);
-    if (INTERIOR || it + 1 < n_it) qk_tile(it + 1, s_next);  // harmless on a tile the wave cannot see
-    if (INTERIOR || tile_active(it)) softmax_pv_tile(it, s_cur, interior_c);
+    if (has_next) fetch_v(it + 1);
+    // ---- phase A
+    if (has_next) qk_tile(it + 1, s_next);  // harmless on a tile the wave cannot see
+    if (act) exp_tile(s_cur, t_cur);
+    // ---- phase B
+    if (act) pv_tile(it);
+    if (INTERIOR || tile_active(it + 1)) t_cur = mask_max(it + 1, s_next, interior_c);
     if (it + 2 < n_it) stage_k(it & 1);
-    if (it + 1 < n_it) stage_v((it + 1) & 1);
+    if (has_next) stage_v((it + 1) & 1);
     __syncthreads();  // fills are visible; every wave is done with the buffers the next step refills
   };
 
@@ -330,22 +352,24 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
     }
   }
   __syncthreads();
+  TileMax t_cur = {0.0f, 1.0f};
   if (n_it > 0) qk_tile(0, s_a);
+  if (tile_active(0)) t_cur = mask_max(0, s_a, std::false_type{});
   __syncthreads();  // sKb[0] is refilled by the first step
   // leading interior iterations, rounded down to pairs so that s_a holds the current logits after them
   int n_int = 0;
   if (p.window == 0) {
     const int full_keys = min(qt * QPW * 32 + p.q_start + 1, p.cache_len);  // keys every row of the workgroup sees
-    n_int = max(0, min(n_it - 1, (full_keys / BN - kt_begin) / NG)) & ~1;
+    n_int = max(0, min(n_it - 1, (full_keys / BN - kt_begin) / NG - 1)) & ~1;
   }
   int it = 0;
   for (; it < n_int; it += 2) {
-    step(it, s_a, s_b, std::true_type{});
-    step(it + 1, s_b, s_a, std::true_type{});
+    step(it, s_a, s_b, t_cur, std::true_type{});
+    step(it + 1, s_b, s_a, t_cur, std::true_type{});
   }
   for (; it < n_it; it += 2) {
-    step(it, s_a, s_b, std::false_type{});
-    if (it + 1 < n_it) step(it + 1, s_b, s_a, std::false_type{});
+    step(it, s_a, s_b, t_cur, std::false_type{});
+    if (it + 1 < n_it) step(it + 1, s_b, s_a, t_cur, std::false_type{});
   }
 
   // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
