@@ -21,6 +21,7 @@
 //    pairing a long and a short tile on each compute unit.
 #include "argus_hip_internal.hpp"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -78,7 +79,7 @@ struct PrefillTile {
 };
 
 template <int D, int HPW, int NG, typename KV_T>
-__global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefill_kernel(const PrefillParams p) {
   using TL = PrefillTile<D>;
   constexpr int BN = TL::BN, KP = TL::KP, VP = TL::VP;
   constexpr int NT = 256 * NG;               // threads
@@ -88,6 +89,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
   constexpr int RB = D / 32;                 // O^T row blocks (32 channels each)
   constexpr int CH = NG * BN * D / 8 / NT;   // 16-byte chunks per thread per iteration
   constexpr int kLdsAhead = 4;               // MFMA operand reads kept in flight
+  constexpr int kVAhead = (D <= 64) ? 4 : 3;
 
   // [2 buffers][NG tiles][K tile | V^T tile]; reused at the end for the cross-group merge.
   extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
@@ -158,26 +160,27 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
   _Float16 *const sKb = smem;                         // [2][NG][BN * KP]
   _Float16 *const sVb = smem + 2 * NG * BN * KP;      // [2][NG][BN * VP]
   half8_t kpre[CH], vpre[CH];
-  auto fetch_k = [&](int it) {
+  // Chunk cid of an iteration's NG tiles is the 16 bytes at element 8*cid from the first tile's
+  // first row (the tiles are adjacent in the cache), so a fetch is a uniform base plus a per-thread
+  // offset; only an iteration that reaches past the visible keys needs per-chunk bounds checks.
+  auto fetch_tiles = [&](const KV_T *base, int it, half8_t(&pre)[CH]) {
+    const int key_first = (kt_begin + it * NG) * BN;
+    const KV_T *tile = base + (int64_t)key_first * D;
+    if (key_first + NG * BN <= kv_end) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int cid = threadIdx.x + NT * c;
-      const int key = (kt_begin + it * NG) * BN + cid / (D / 8), dc = cid % (D / 8);
-      half8_t kx = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (key < kv_end) kx = load_kv_chunk<KV_T>(kbase + (int64_t)key * D + 8 * dc);
-      kpre[c] = kx;
+      for (int c = 0; c < CH; ++c) pre[c] = load_kv_chunk<KV_T>(tile + (size_t)c * (NT * 8) + threadIdx.x * 8);
+    } else {
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int cid = threadIdx.x + NT * c;
+        half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (key_first + cid / (D / 8) < kv_end) x = load_kv_chunk<KV_T>(tile + (size_t)cid * 8);
+        pre[c] = x;
+      }
     }
   };
-  auto fetch_v = [&](int it) {
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int cid = threadIdx.x + NT * c;
-      const int key = (kt_begin + it * NG) * BN + cid / (D / 8), dc = cid % (D / 8);
-      half8_t vx = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (key < kv_end) vx = load_kv_chunk<KV_T>(vbase + (int64_t)key * D + 8 * dc);
-      vpre[c] = vx;
-    }
-  };
+  auto fetch_k = [&](int it) { fetch_tiles(kbase, it, kpre); };
+  auto fetch_v = [&](int it) { fetch_tiles(vbase, it, vpre); };
   auto stage_k = [&](int buf) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -271,7 +274,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
   };
   // Probabilities of the current tile (exp2 against t.m_ref), rounded to f16 in P^T operand order.
   half8_t pb[BN / 16];
-  auto exp_tile = [&](float16_t(&s_acc)[KB], const TileMax &t) {
+  auto rescale = [&](const TileMax &t) {
     if (__builtin_amdgcn_ballot_w64(t.alpha != 1.0f) != 0) {
 #pragma unroll
       for (int r = 0; r < RB; ++r)
@@ -279,6 +282,8 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
         for (int i = 0; i < 16; ++i) o_acc[r][i] *= t.alpha;
       l_run *= t.alpha;
     }
+  };
+  auto exp_tile = [&](float16_t(&s_acc)[KB], const TileMax &t) {
     // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
     // rounding cancels in the final normalisation.
     float lsum = 0.0f;
@@ -315,6 +320,14 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
         const half8_t a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[jn], o_acc[r], 0, 0, 0);
       }
+    // two transposing reads per MFMA, kept kVAhead MFMAs ahead
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kVAhead, 0);
+#pragma unroll
+    for (int i = 0; i < (BN / 16) * RB - kVAhead; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kVAhead, 0);
   };
 
   // One pipeline step.  On entry s_cur holds the logits of iteration `it` and t_cur their maximum
@@ -327,6 +340,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_kernel(const PrefillParams p
     constexpr bool INTERIOR = decltype(interior_c)::value;
     const bool act = INTERIOR || tile_active(it);
     const bool has_next = INTERIOR || it + 1 < n_it;
+    if (act) rescale(t_cur);  // its branch stays out of the phases below
     if (it + 2 < n_it) fetch_k(it + 2);
     if (has_next) fetch_v(it + 1);
     // ---- phase A
@@ -455,8 +469,9 @@ int launch(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
   // (8 waves, <= 256 VGPRs each) measured best; four groups need a 128-VGPR cap that spills.
   const size_t tile_bytes = (size_t)PrefillTile<D>::HALFS * sizeof(_Float16);
   const size_t lds_limit = ctx->props.sharedMemPerBlock;
+  static const bool one_group = getenv("ARGUS_PREFILL_NG1") != nullptr;
   if constexpr (D <= 128) {
-    if (2 * 2 * tile_bytes <= lds_limit) return launch_ng<D, HPW, 2, KV_T>(ctx, p, stream, 2 * 2 * tile_bytes);
+    if (!one_group && 2 * 2 * tile_bytes <= lds_limit) return launch_ng<D, HPW, 2, KV_T>(ctx, p, stream, 2 * 2 * tile_bytes);
   }
   if (2 * tile_bytes > lds_limit)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: %zu bytes of LDS needed, %zu available", 2 * tile_bytes, lds_limit);
