@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = [
     "argus_hip_attention_gen", "argus_hip_flash_attention_prefill",
     "argus_hip_has_quant_attn_kernel", "argus_hip_attention_gen_quant",
     "argus_hip_attention_gen_quant_ex", "argus_hip_gather_update_quant", "argus_hip_quant_flush",
+    "argus_hip_quant_dequant_flush", "argus_hip_quant_scatter_residual",
     "argus_hip_score_reduce", "argus_hip_score_reduce_per_layer",
     "argus_hip_kv_scatter_f32_to_f16", "argus_hip_kv_scatter_f32_to_f16_batch",
     "argus_hip_kv_scatter_f32_batch",
@@ -100,6 +101,19 @@ class QuantFlushArgs(C.Structure):
                 ("k_block_start", C.c_size_t), ("v_block_start", C.c_size_t), ("bits", C.c_uint8)]
 
 
+class QuantDequantFlushArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("q_blocks_mem", C.c_uint64), ("attn_mem", C.c_uint64),
+                ("kv_heads", C.c_size_t), ("head_dim", C.c_size_t), ("n_groups_or_tokens", C.c_size_t),
+                ("tok_base", C.c_size_t), ("block_start", C.c_size_t), ("bits", C.c_uint8),
+                ("is_key", C.c_uint8)]
+
+
+class QuantScatterResidualArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("res_mem", C.c_uint64), ("attn_mem", C.c_uint64),
+                ("kv_heads", C.c_size_t), ("res_cap", C.c_size_t), ("head_dim", C.c_size_t),
+                ("res_pos", C.c_size_t), ("tok_base", C.c_size_t)]
+
+
 class ScoreReduceArgs(C.Structure):
     _fields_ = [("stream", C.c_void_p), ("score_buf", C.c_uint64), ("importance", C.c_uint64),
                 ("head_importance", C.c_uint64), ("decay_factor", C.c_float),
@@ -131,6 +145,8 @@ def _bind():
     lib.argus_hip_attention_gen_quant_ex.argtypes = [vp, C.POINTER(QuantAttnArgs), C.POINTER(QuantAttnExt)]
     lib.argus_hip_gather_update_quant.argtypes = [vp, C.POINTER(QuantGatherArgs)]
     lib.argus_hip_quant_flush.argtypes = [vp, C.POINTER(QuantFlushArgs)]
+    lib.argus_hip_quant_dequant_flush.argtypes = [vp, C.POINTER(QuantDequantFlushArgs)]
+    lib.argus_hip_quant_scatter_residual.argtypes = [vp, C.POINTER(QuantScatterResidualArgs)]
     lib.argus_hip_score_reduce.argtypes = [vp, C.POINTER(ScoreReduceArgs)]
     lib.argus_hip_score_reduce_per_layer.argtypes = [vp, C.POINTER(ScoreReduceArgs)]
     sc16 = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32]
@@ -285,6 +301,21 @@ class Context:
                            head_dim=head_dim, flush_tokens=flush_tokens,
                            k_block_start=k_block_start, v_block_start=v_block_start, bits=bits)
         return self._check(lib.argus_hip_quant_flush(self.handle, C.byref(a)), check)
+
+    def quant_dequant_flush(self, blocks, attn, kv_heads, head_dim, n_groups_or_tokens, tok_base,
+                            block_start, bits, is_key, check=True):
+        a = QuantDequantFlushArgs(stream=_stream(), q_blocks_mem=_ptr(blocks), attn_mem=_ptr(attn),
+                                  kv_heads=kv_heads, head_dim=head_dim,
+                                  n_groups_or_tokens=n_groups_or_tokens, tok_base=tok_base,
+                                  block_start=block_start, bits=bits, is_key=1 if is_key else 0)
+        return self._check(lib.argus_hip_quant_dequant_flush(self.handle, C.byref(a)), check)
+
+    def quant_scatter_residual(self, residual, attn, kv_heads, res_cap, head_dim, res_pos, tok_base,
+                               check=True):
+        a = QuantScatterResidualArgs(stream=_stream(), res_mem=_ptr(residual), attn_mem=_ptr(attn),
+                                     kv_heads=kv_heads, res_cap=res_cap, head_dim=head_dim,
+                                     res_pos=res_pos, tok_base=tok_base)
+        return self._check(lib.argus_hip_quant_scatter_residual(self.handle, C.byref(a)), check)
 
     # -- (a-4) ---------------------------------------------------------------------------
     def _score_args(self, scores, importance, head_importance, decay_factor, n_layers, n_heads_q,

@@ -169,9 +169,9 @@ class HipQuantAttnBackend {
   bool is_nosub_device() const { return true; }
   int attention_gen_quant(const argus_hip_quant_attn_args &a) const { return ctx_ ? argus_hip_attention_gen_quant(ctx_, &a) : -1; }
   int gather_update_quant(const argus_hip_quant_gather_args &a) const { return ctx_ ? argus_hip_gather_update_quant(ctx_, &a) : -1; }
-  // Q2 F16-view helpers are not built: the trait defaults return -1 (lib.rs:3096-3103).
-  int dequant_flush() const { return -1; }
-  int scatter_residual() const { return -1; }
+  // F16-view helpers (lib.rs:3096-3103): negative on failure like the reference (-1 .. -4).
+  int dequant_flush(const argus_hip_quant_dequant_flush_args &a) const { return ctx_ ? argus_hip_quant_dequant_flush(ctx_, &a) : -1; }
+  int scatter_residual(const argus_hip_quant_scatter_residual_args &a) const { return ctx_ ? argus_hip_quant_scatter_residual(ctx_, &a) : -1; }
 
  private:
   argus_hip_ctx *ctx_;

@@ -241,6 +241,42 @@ typedef struct argus_hip_quant_flush_args {
 } argus_hip_quant_flush_args;
 int argus_hip_quant_flush(argus_hip_ctx *ctx, const argus_hip_quant_flush_args *args);
 
+/* Dequantise flushed blocks into the F16 attention view [max_seq, kv_heads, head_dim] (sequence
+ * major).  Field-for-field twin of CudaQuantDequantFlushArgs,
+ * crates/argus-extension-api/src/lib.rs:3045-3063; CudaQuantAttnBackend::dequant_flush 3096-3099;
+ * kernels crates/techniques/kivi/src/kivi_q2.cu:18-92 (keys: block (h, g, ch) = 32 tokens of one
+ * channel, n_groups_or_tokens = groups per flush; values: block (h, t, b) = 32 channels of one
+ * token, n_groups_or_tokens = flush tokens).  The reference serves bits == 2 only
+ * (gpu_kivi_cuda.rs:251-254); 2, 4 and 8 are served here.  attn_mem 16-byte aligned. */
+typedef struct argus_hip_quant_dequant_flush_args {
+  void *stream;
+  uint64_t q_blocks_mem;
+  uint64_t attn_mem;
+  size_t kv_heads;
+  size_t head_dim;
+  size_t n_groups_or_tokens;
+  size_t tok_base;
+  size_t block_start; /* index of the first block in q_blocks_mem */
+  uint8_t bits;
+  uint8_t is_key; /* Rust bool */
+} argus_hip_quant_dequant_flush_args;
+int argus_hip_quant_dequant_flush(argus_hip_ctx *ctx, const argus_hip_quant_dequant_flush_args *args);
+
+/* Copy the first res_pos rows of the F32 residual ring [kv_heads, res_cap, head_dim] to rows
+ * tok_base.. of the F16 attention view.  Twin of CudaQuantScatterResidualArgs, lib.rs:3065-3081;
+ * CudaQuantAttnBackend::scatter_residual 3100-3103; kernel kivi_q2.cu:94-116. */
+typedef struct argus_hip_quant_scatter_residual_args {
+  void *stream;
+  uint64_t res_mem;
+  uint64_t attn_mem;
+  size_t kv_heads;
+  size_t res_cap;
+  size_t head_dim;
+  size_t res_pos;
+  size_t tok_base;
+} argus_hip_quant_scatter_residual_args;
+int argus_hip_quant_scatter_residual(argus_hip_ctx *ctx, const argus_hip_quant_scatter_residual_args *args);
+
 /* ---- (a-4) attention-score reduce for H2O / D2O --------------------------------------------- */
 /* Field-for-field twin of CudaScoreReduceArgs, crates/argus-extension-api/src/lib.rs:2909-2933;
  * CudaScoreReduceBackend::{reduce, reduce_per_layer} 2938-2948; kernel semantics

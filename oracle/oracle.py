@@ -223,6 +223,42 @@ def kivi_assemble_view(c):
     return ak[:total], av[:total]
 
 
+def kivi_dequant_flush_f16(blocks, attn, kv_heads, head_dim, n_groups_or_tokens, tok_base, block_start,
+                           bits, is_key):
+    """F16-view dequant of one flush (crates/techniques/kivi/src/kivi_q2.cu:18-92, generalised from
+    Q2 to the 4- and 8-bit codecs): attn is [max_seq, kv_heads, head_dim] float16, written in place.
+    Keys: block (h, g, ch) -> tokens tok_base + 32 g + i of channel ch; values: block (h, t, b) ->
+    channels 32 b + i of token tok_base + t.  out = f16(code * d + m) in float32."""
+    bb = kivi_block_bytes(bits)
+    blocks = np.ascontiguousarray(blocks, np.uint8).reshape(-1, bb)
+    n = n_groups_or_tokens
+    nblk = kv_heads * n * (head_dim if is_key else head_dim // 32)
+    blk = blocks[block_start:block_start + nblk]
+    d = blk[:, 0:2].copy().view(np.float16).astype(np.float32)      # [nblk, 1]
+    m = blk[:, 2:4].copy().view(np.float16).astype(np.float32)
+    qs = blk[:, 4:]
+    per = 8 // bits
+    idx = np.arange(32)
+    codes = (qs[:, idx // per] >> ((idx % per) * bits).astype(np.uint8)) & ((1 << bits) - 1)
+    vals = (codes.astype(np.float32) * d + m).astype(np.float16)     # [nblk, 32]
+    if is_key:
+        v = vals.reshape(kv_heads, n, head_dim, 32)                  # [h, g, ch, i]
+        for g in range(n):
+            attn[tok_base + 32 * g:tok_base + 32 * g + 32] = v[:, g].transpose(2, 0, 1)
+    else:
+        v = vals.reshape(kv_heads, n, head_dim // 32, 32)            # [h, t, b, i]
+        attn[tok_base:tok_base + n] = v.transpose(1, 0, 2, 3).reshape(n, kv_heads, head_dim)
+    return attn
+
+
+def kivi_scatter_residual_f16(residual, attn, kv_heads, res_cap, head_dim, res_pos, tok_base):
+    """kivi_q2.cu:94-116: rows 0..res_pos of the F32 ring [kv_heads, res_cap, head_dim] -> rows
+    tok_base.. of the F16 view."""
+    r = np.asarray(residual, np.float32).reshape(kv_heads, res_cap, head_dim)
+    attn[tok_base:tok_base + res_pos] = r[:, :res_pos].transpose(1, 0, 2).astype(np.float16)
+    return attn
+
+
 def kivi_attention(q, c, scale, scores=False, score_stride=None):
     q = np.ascontiguousarray(q, np.float32)
     hq, d = q.shape

@@ -218,8 +218,10 @@ static void test_quant_attn(HipBackend &be) {
   HipQuantAttnBackend degraded(nullptr);
   argus_hip_quant_attn_args za{};
   argus_hip_quant_gather_args zg{};
+  argus_hip_quant_dequant_flush_args zd{};
+  argus_hip_quant_scatter_residual_args zs{};
   CHECK(!degraded.has_quant_attn_kernel(2) && degraded.attention_gen_quant(za) == -1 && degraded.gather_update_quant(zg) == -1 &&
-            degraded.dequant_flush() == -1 && degraded.scatter_residual() == -1,
+            degraded.dequant_flush(zd) == -1 && degraded.scatter_residual(zs) == -1,
         "degraded handle returns -1 everywhere");
   HipQuantAttnBackend cap(be.ctx());
   CHECK(cap.has_quant_attn_kernel(2) && cap.has_quant_attn_kernel(4) && cap.has_quant_attn_kernel(8) && !cap.has_quant_attn_kernel(3), "kernels present");

@@ -33,6 +33,8 @@ def test_struct_layouts_match_header_field_order():
     pairs = {"argus_hip_attention_gen_args": A.AttentionGenArgs, "argus_hip_prefill_args": A.PrefillArgs,
              "argus_hip_quant_attn_args": A.QuantAttnArgs, "argus_hip_quant_attn_ext": A.QuantAttnExt,
              "argus_hip_quant_gather_args": A.QuantGatherArgs, "argus_hip_quant_flush_args": A.QuantFlushArgs,
+             "argus_hip_quant_dequant_flush_args": A.QuantDequantFlushArgs,
+             "argus_hip_quant_scatter_residual_args": A.QuantScatterResidualArgs,
              "argus_hip_score_reduce_args": A.ScoreReduceArgs, "argus_hip_device_info": A.DeviceInfo}
     for cname, cls in pairs.items():
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), text, re.S).group(1)

@@ -247,3 +247,41 @@ def test_kivi_argument_errors():
     assert c.attention_gen_quant(q, z, z, z, z, q.clone(), 2, 33, 0, 32, 0.1, 4, check=False) == A.ERR_INVALID
     assert c.gather_update_quant(z, z, 2, 32, 128, 4, 30, check=False) == A.ERR_INVALID
     assert c.quant_flush(z, z, z, z, 2, 32, 128, 48, 0, 0, 4, check=False) == A.ERR_INVALID
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("hkv,d,R,n", [(3, 64, 64, 64 * 3 + 17), (8, 128, 128, 128 * 2 + 128), (2, 256, 32, 97)])
+def test_f16_view_dequant_flush_and_scatter_bit_exact(bits, hkv, d, R, n):
+    # CudaQuantAttnBackend::{dequant_flush, scatter_residual}: the F16 attention view built on the
+    # device flush by flush equals the oracle's, bit for bit, and nothing outside the rows is touched.
+    import torch
+    rng = np.random.default_rng(300 + bits + n)
+    k = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    k[:, 0, 1] *= 10.0
+    c = O.kivi_build(k, v, R, bits)
+    gpf = R // 32
+    ref_k = np.full((n + 2, hkv, d), 7.0, np.float16)
+    ref_v = ref_k.copy()
+    dev_k = torch.full((n + 2, hkv, d), 7.0, device="cuda", dtype=torch.float16)
+    dev_v = dev_k.clone()
+    qk, qv, rk, rv = dev(c["qk"]), dev(c["qv"]), dev(c["res_k"]), dev(c["res_v"])
+    for f in range(c["q_tokens"] // R):
+        kb, vb = f * hkv * gpf * d, f * hkv * R * (d // 32)
+        O.kivi_dequant_flush_f16(c["qk"], ref_k, hkv, d, gpf, f * R, kb, bits, True)
+        O.kivi_dequant_flush_f16(c["qv"], ref_v, hkv, d, R, f * R, vb, bits, False)
+        ctx().quant_dequant_flush(qk, dev_k, hkv, d, gpf, f * R, kb, bits, True)
+        ctx().quant_dequant_flush(qv, dev_v, hkv, d, R, f * R, vb, bits, False)
+    O.kivi_scatter_residual_f16(c["res_k"], ref_k, hkv, R, d, c["res_tokens"], c["q_tokens"])
+    O.kivi_scatter_residual_f16(c["res_v"], ref_v, hkv, R, d, c["res_tokens"], c["q_tokens"])
+    ctx().quant_scatter_residual(rk, dev_k, hkv, R, d, c["res_tokens"], c["q_tokens"])
+    ctx().quant_scatter_residual(rv, dev_v, hkv, R, d, c["res_tokens"], c["q_tokens"])
+    got_k, got_v = host(dev_k), host(dev_v)
+    assert np.array_equal(got_k.view(np.uint16), ref_k.view(np.uint16))
+    assert np.array_equal(got_v.view(np.uint16), ref_v.view(np.uint16))
+    # empty calls and error behaviour
+    import argus_hip as A
+    assert ctx().quant_dequant_flush(qk, dev_k, hkv, d, 0, 0, 0, bits, True) == 0
+    assert ctx().quant_scatter_residual(rk, dev_k, hkv, R, d, 0, 0) == 0
+    assert ctx().quant_dequant_flush(qk, dev_k, hkv, d, 1, 0, 0, 3, True, check=False) == A.ERR_UNSUPPORTED
+    assert ctx().quant_scatter_residual(rk, dev_k, hkv, R, d, R + 1, 0, check=False) == A.ERR_INVALID

@@ -277,3 +277,25 @@ def test_compaction_and_scatter_vs_naive_model():
     assert np.array_equal(kd[:, 11:16], ks.transpose(1, 0, 2).astype(np.float16))
     assert np.array_equal(vd[:, 11:16], vs.transpose(1, 0, 2).astype(np.float16))
     assert not kd[:, :11].any() and not kd[:, 16:].any()
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_f16_view_dequant_flush_and_scatter_match_assembled_view(bits):
+    # The F16 attention view built flush by flush (kivi_q2.cu:18-116) must equal the C oracle's
+    # dequantised view (an independent walk over the same container) rounded to f16.
+    hkv, d, R, n = 3, 64, 64, 64 * 3 + 17
+    rng = np.random.default_rng(90 + bits)
+    k = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    c = O.kivi_build(k, v, R, bits)
+    ak, av = O.kivi_assemble_view(c)
+    vk = np.full((n + 3, hkv, d), 7.0, np.float16)
+    vv = np.full((n + 3, hkv, d), 7.0, np.float16)
+    gpf = R // 32
+    for f in range(c["q_tokens"] // R):
+        O.kivi_dequant_flush_f16(c["qk"], vk, hkv, d, gpf, f * R, f * hkv * gpf * d, bits, True)
+        O.kivi_dequant_flush_f16(c["qv"], vv, hkv, d, R, f * R, f * hkv * R * (d // 32), bits, False)
+    O.kivi_scatter_residual_f16(c["res_k"], vk, hkv, R, d, c["res_tokens"], c["q_tokens"])
+    O.kivi_scatter_residual_f16(c["res_v"], vv, hkv, R, d, c["res_tokens"], c["q_tokens"])
+    assert np.array_equal(vk[:n], ak.astype(np.float16)) and np.array_equal(vv[:n], av.astype(np.float16))
+    assert (vk[n:] == 7.0).all() and (vv[n:] == 7.0).all()
