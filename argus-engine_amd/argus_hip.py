@@ -21,7 +21,7 @@ EXPORTED_SYMBOLS = [
     "argus_hip_get_device_info", "argus_hip_kernel_timing_begin", "argus_hip_kernel_timing_end",
     "argus_hip_malloc", "argus_hip_free", "argus_hip_write_buffer",
     "argus_hip_read_buffer", "argus_hip_copy_slice", "argus_hip_synchronize",
-    "argus_hip_attention_gen", "argus_hip_flash_attention_prefill",
+    "argus_hip_attention_gen", "argus_hip_flash_attention_prefill", "argus_hip_prefill_attention_scores",
     "argus_hip_has_quant_attn_kernel", "argus_hip_attention_gen_quant",
     "argus_hip_attention_gen_quant_ex", "argus_hip_gather_update_quant", "argus_hip_quant_flush",
     "argus_hip_quant_dequant_flush", "argus_hip_quant_scatter_residual",
@@ -70,6 +70,15 @@ class PrefillArgs(C.Structure):
                 ("cache_seq_len", C.c_int32), ("head_dim", C.c_int32), ("kv_capacity", C.c_int32),
                 ("batch_size", C.c_int32), ("is_head_major", C.c_int32), ("q_dtype", C.c_int32),
                 ("kv_dtype", C.c_int32), ("out_dtype", C.c_int32), ("window", C.c_int32)]
+
+
+class PfaArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("q", C.c_void_p), ("k", C.c_void_p), ("k_dtype", C.c_int32),
+                ("n_heads_q", C.c_int32), ("n_heads_kv", C.c_int32), ("head_dim", C.c_int32),
+                ("seq_len", C.c_int32), ("cache_seq_len", C.c_int32), ("k_pos_stride", C.c_int64),
+                ("kv_head_stride", C.c_int64), ("q_start_pos", C.c_int32), ("q_window", C.c_int32),
+                ("has_window", C.c_int32), ("window", C.c_int32), ("sum_out", C.c_void_p),
+                ("per_row_out", C.c_void_p), ("per_row_per_head", C.c_int32)]
 
 
 class QuantAttnArgs(C.Structure):
@@ -140,6 +149,7 @@ def _bind():
     lib.argus_hip_synchronize.argtypes = [vp, vp]
     lib.argus_hip_attention_gen.argtypes = [vp, C.POINTER(AttentionGenArgs)]
     lib.argus_hip_flash_attention_prefill.argtypes = [vp, C.POINTER(PrefillArgs)]
+    lib.argus_hip_prefill_attention_scores.argtypes = [vp, C.POINTER(PfaArgs)]
     lib.argus_hip_has_quant_attn_kernel.argtypes = [vp, C.c_uint8]
     lib.argus_hip_attention_gen_quant.argtypes = [vp, C.POINTER(QuantAttnArgs)]
     lib.argus_hip_attention_gen_quant_ex.argtypes = [vp, C.POINTER(QuantAttnArgs), C.POINTER(QuantAttnExt)]
@@ -258,6 +268,20 @@ class Context:
             batch_size=batch_size, is_head_major=int(is_head_major), q_dtype=_kv_dtype(q),
             kv_dtype=_kv_dtype(k), out_dtype=_kv_dtype(out), window=window)
         return self._check(lib.argus_hip_flash_attention_prefill(self.handle, C.byref(a)), check)
+
+    # -- (a-6) ---------------------------------------------------------------------------
+    def prefill_attention_scores(self, q, k, n_heads_q, n_heads_kv, head_dim, seq_len, cache_seq_len,
+                                 k_pos_stride, kv_head_stride, q_start_pos, q_window, window=None,
+                                 sum_out=None, per_row=None, per_head=False, check=True):
+        a = PfaArgs(stream=_stream(), q=_ptr(q), k=_ptr(k), k_dtype=_kv_dtype(k), n_heads_q=n_heads_q,
+                    n_heads_kv=n_heads_kv, head_dim=head_dim, seq_len=seq_len,
+                    cache_seq_len=cache_seq_len, k_pos_stride=k_pos_stride,
+                    kv_head_stride=kv_head_stride, q_start_pos=q_start_pos, q_window=q_window,
+                    has_window=0 if window is None else 1, window=0 if window is None else window,
+                    sum_out=_ptr(sum_out) if sum_out is not None else None,
+                    per_row_out=_ptr(per_row) if per_row is not None else None,
+                    per_row_per_head=1 if per_head else 0)
+        return self._check(lib.argus_hip_prefill_attention_scores(self.handle, C.byref(a)), check)
 
     # -- (a-3) ---------------------------------------------------------------------------
     def has_quant_attn_kernel(self, bits):

@@ -115,6 +115,24 @@ class HipBackend {
     return Result<bool>::Ok(rc == 1);
   }
 
+  // ---- PFA side channel (prefill_attention_scores, engine/src/kv/standard_format.rs:1400-1510) ----
+  // Same argument order as the host mirror; q and k are device tensors, sum_out / per_row device F32
+  // buffers (nullptr = not armed).  has_window mirrors Option<usize>.
+  Status prefill_attention_scores(const Tensor &q, const Tensor &k, size_t n_heads_q, size_t n_heads_kv, size_t head_dim,
+                                  size_t seq_len, size_t cache_seq_len, size_t k_pos_stride, size_t kv_head_stride,
+                                  size_t q_start_pos, size_t q_window, bool has_window, size_t window, float *sum_out,
+                                  float *per_row_out, bool per_row_per_head) {
+    argus_hip_pfa_args a{};
+    a.q = q.ptr; a.k = k.ptr; a.k_dtype = (int32_t)k.dtype;
+    a.n_heads_q = (int32_t)n_heads_q; a.n_heads_kv = (int32_t)n_heads_kv; a.head_dim = (int32_t)head_dim;
+    a.seq_len = (int32_t)seq_len; a.cache_seq_len = (int32_t)cache_seq_len;
+    a.k_pos_stride = (int64_t)k_pos_stride; a.kv_head_stride = (int64_t)kv_head_stride;
+    a.q_start_pos = (int32_t)q_start_pos; a.q_window = (int32_t)q_window;
+    a.has_window = has_window ? 1 : 0; a.window = (int32_t)window;
+    a.sum_out = sum_out; a.per_row_out = per_row_out; a.per_row_per_head = per_row_per_head ? 1 : 0;
+    return wrap(argus_hip_prefill_attention_scores(ctx_, &a));
+  }
+
   // ---- Backend::kv_scatter_f32_to_f16 / _batch (engine/src/backend.rs:425-545) ----------------
   Status kv_scatter_f32_to_f16(const Tensor &k_src, const Tensor &v_src, Tensor &k_dst, Tensor &v_dst,
                                size_t head_dim, size_t capacity, size_t write_pos) {

@@ -277,6 +277,38 @@ typedef struct argus_hip_quant_scatter_residual_args {
 } argus_hip_quant_scatter_residual_args;
 int argus_hip_quant_scatter_residual(argus_hip_ctx *ctx, const argus_hip_quant_scatter_residual_args *args);
 
+/* ---- (a-6) PFA side channel: prefill attention scores on the device --------------------------
+ * Stands in for the host mirror prefill_attention_scores, engine/src/kv/standard_format.rs:
+ * 1400-1510 (arguments in the same order and meaning; PerRowScores { out, per_head } becomes
+ * per_row_out / per_row_per_head), which the reference can only run after reading K back from
+ * VRAM (standard_format.rs:1137-1173).  q: device F32 [seq_len, n_heads_q, head_dim]; k: device
+ * F32 or F16 addressed as k[key * k_pos_stride + kv_head * kv_head_stride + d] (elements), so both
+ * cache layouts work.  sum_out [n_heads_q, cache_seq_len] is accumulated in place (+=);
+ * per_row_out is [q_window, n_heads_q, cache_seq_len] written (per head) or
+ * [q_window, cache_seq_len] accumulated with 1/n_heads_q (head mean).  Either may be NULL.
+ * Single sequence, like the reference. */
+typedef struct argus_hip_pfa_args {
+  void *stream;
+  const void *q;
+  const void *k;
+  int32_t k_dtype; /* ARGUS_HIP_F32 / ARGUS_HIP_F16 */
+  int32_t n_heads_q;
+  int32_t n_heads_kv;
+  int32_t head_dim;
+  int32_t seq_len;
+  int32_t cache_seq_len;
+  int64_t k_pos_stride;
+  int64_t kv_head_stride;
+  int32_t q_start_pos;
+  int32_t q_window;
+  int32_t has_window; /* Option<usize>: 0 = None */
+  int32_t window;
+  void *sum_out;
+  void *per_row_out;
+  int32_t per_row_per_head;
+} argus_hip_pfa_args;
+int argus_hip_prefill_attention_scores(argus_hip_ctx *ctx, const argus_hip_pfa_args *args);
+
 /* ---- (a-4) attention-score reduce for H2O / D2O --------------------------------------------- */
 /* Field-for-field twin of CudaScoreReduceArgs, crates/argus-extension-api/src/lib.rs:2909-2933;
  * CudaScoreReduceBackend::{reduce, reduce_per_layer} 2938-2948; kernel semantics

@@ -904,3 +904,70 @@ ORACLE_API void oracle_kv_scatter(const float *k_src, const float *v_src, void *
         }
       }
 }
+
+/* ---- PFA side channel ----------------------------------------------------------------------
+ * prefill_attention_scores, engine/src/kv/standard_format.rs:1400-1510: for the trailing q_window
+ * query rows of a prefill chunk, the post-softmax probability of every visible key, (a) summed
+ * over the rows into sum_out[h][key] (+=) and/or (b) per row: per_head -> out[step][h][key] = p,
+ * else out[step][key] += p / n_heads_q.  Scalar f32 dot (mul then add), logit = dot * scale,
+ * row maximum, e = exp(logit - max), denom summed in key order, p = e / denom.  K is F32 with the
+ * caller's strides (elements).  window < 0 means no window; lo = p - (window - 1), saturating. */
+ORACLE_API int oracle_prefill_attention_scores(const float *q, const float *k, int n_heads_q,
+                                               int n_heads_kv, int head_dim, int seq_len,
+                                               int cache_seq_len, int64_t k_pos_stride,
+                                               int64_t kv_head_stride, int q_start_pos, int q_window,
+                                               int window, float *sum_out, float *per_row_out,
+                                               int per_row_per_head) {
+  if (n_heads_kv <= 0 || n_heads_q % n_heads_kv) return -1;
+  const int prefix_len = cache_seq_len;
+  const float scale = 1.0f / sqrtf((float)head_dim);
+  const int gqa = n_heads_q / n_heads_kv;
+  const int64_t q_row_stride = (int64_t)n_heads_q * head_dim;
+  const int qwin = q_window < seq_len ? q_window : seq_len;
+  const int qwin_start = seq_len - qwin;
+  const float inv_heads = 1.0f / (float)n_heads_q;
+  float *scratch = (float *)malloc(sizeof(float) * (size_t)(prefix_len > 0 ? prefix_len : 1));
+  if (!scratch) return -2;
+  for (int h = 0; h < n_heads_q; ++h) {
+    const int kv_head = h / gqa;
+    const int64_t out_row_base = (int64_t)h * prefix_len;
+    for (int r = qwin_start; r < seq_len; ++r) {
+      const int p = q_start_pos + r;
+      int lo = 0;
+      if (window >= 0) {
+        const int w1 = window > 0 ? window - 1 : 0;
+        lo = p > w1 ? p - w1 : 0;
+      }
+      const float *qv = q + (int64_t)r * q_row_stride + (int64_t)h * head_dim;
+      float maxv = -INFINITY;
+      for (int key = lo; key <= p; ++key) {
+        const float *kv = k + (int64_t)key * k_pos_stride + (int64_t)kv_head * kv_head_stride;
+        float dot = 0.0f;
+        for (int d = 0; d < head_dim; ++d) dot += qv[d] * kv[d];
+        const float logit = dot * scale;
+        scratch[key] = logit;
+        if (logit > maxv) maxv = logit;
+      }
+      float denom = 0.0f;
+      for (int key = lo; key <= p; ++key) {
+        const float e = expf(scratch[key] - maxv);
+        scratch[key] = e;
+        denom += e;
+      }
+      if (sum_out)
+        for (int key = lo; key <= p; ++key) sum_out[out_row_base + key] += scratch[key] / denom;
+      if (per_row_out) {
+        const int step = r - qwin_start;
+        if (per_row_per_head) {
+          float *dst = per_row_out + (int64_t)step * n_heads_q * prefix_len + out_row_base;
+          for (int key = lo; key <= p; ++key) dst[key] = scratch[key] / denom;
+        } else {
+          float *dst = per_row_out + (int64_t)step * prefix_len;
+          for (int key = lo; key <= p; ++key) dst[key] += (scratch[key] / denom) * inv_heads;
+        }
+      }
+    }
+  }
+  free(scratch);
+  return 0;
+}

@@ -86,6 +86,9 @@ _keep = _sig("oracle_compile_keep_top_k", C.c_int, [C.c_int, C.c_int, C.c_int, C
 _skeep = _sig("oracle_streaming_keep", C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, _i32p])
 _compact = _sig("oracle_compact_keep", None, [
     C.c_void_p, C.c_void_p, _i32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int])
+_pfa = _sig("oracle_prefill_attention_scores", C.c_int, [
+    _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_int,
+    C.c_int, _f32p, _f32p, C.c_int])
 _scatter = _sig("oracle_kv_scatter", None, [
     _f32p, _f32p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int])
 
@@ -348,3 +351,17 @@ def kv_scatter(k_src, v_src, k_dst, v_dst, write_pos_start):
     cap = k_dst.shape[1]
     _scatter(_p(k_src, _f32p), _p(v_src, _f32p), _p(k_dst), _p(v_dst), hkv, d, cap,
              write_pos_start, s, int(k_dst.dtype != np.float32))
+
+
+def prefill_attention_scores(q, k, n_heads_q, n_heads_kv, head_dim, seq_len, cache_seq_len, k_pos_stride,
+                             kv_head_stride, q_start_pos, q_window, window=None, sum_out=None,
+                             per_row=None, per_head=False):
+    """PFA side channel (standard_format.rs:1400-1510).  q [seq_len, n_heads_q, head_dim] f32, k a flat
+    f32 array addressed by the strides; sum_out / per_row are float32 arrays updated in place."""
+    q = np.ascontiguousarray(q, np.float32)
+    k = np.ascontiguousarray(k, np.float32)
+    rc = _pfa(_p(q, _f32p), _p(k, _f32p), n_heads_q, n_heads_kv, head_dim, seq_len, cache_seq_len,
+              k_pos_stride, kv_head_stride, q_start_pos, q_window, -1 if window is None else window,
+              _p(sum_out, _f32p), _p(per_row, _f32p), 1 if per_head else 0)
+    if rc != 0:
+        raise ValueError("oracle prefill_attention_scores rc=%d" % rc)
