@@ -27,7 +27,7 @@ EXPORTED_SYMBOLS = [
     "argus_hip_quant_dequant_flush", "argus_hip_quant_scatter_residual",
     "argus_hip_score_reduce", "argus_hip_score_reduce_per_layer",
     "argus_hip_kv_scatter_f32_to_f16", "argus_hip_kv_scatter_f32_to_f16_batch",
-    "argus_hip_kv_scatter_f32_batch",
+    "argus_hip_kv_scatter_f32_batch", "argus_hip_kv_decode_descriptor", "argus_hip_kv_encode_descriptor",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -123,6 +123,11 @@ class QuantScatterResidualArgs(C.Structure):
                 ("res_pos", C.c_size_t), ("tok_base", C.c_size_t)]
 
 
+class KvLayoutDesc(C.Structure):
+    _fields_ = [("block_elems", C.c_uint32), ("bits", C.c_uint8), ("scale_layout", C.c_uint32),
+                ("packing", C.c_uint32)]
+
+
 class ScoreReduceArgs(C.Structure):
     _fields_ = [("stream", C.c_void_p), ("score_buf", C.c_uint64), ("importance", C.c_uint64),
                 ("head_importance", C.c_uint64), ("decay_factor", C.c_float),
@@ -150,6 +155,8 @@ def _bind():
     lib.argus_hip_attention_gen.argtypes = [vp, C.POINTER(AttentionGenArgs)]
     lib.argus_hip_flash_attention_prefill.argtypes = [vp, C.POINTER(PrefillArgs)]
     lib.argus_hip_prefill_attention_scores.argtypes = [vp, C.POINTER(PfaArgs)]
+    lib.argus_hip_kv_decode_descriptor.argtypes = [vp, vp, C.POINTER(KvLayoutDesc), vp, vp, C.c_int32, C.c_int64]
+    lib.argus_hip_kv_encode_descriptor.argtypes = [vp, vp, C.POINTER(KvLayoutDesc), vp, vp, C.c_int64]
     lib.argus_hip_has_quant_attn_kernel.argtypes = [vp, C.c_uint8]
     lib.argus_hip_attention_gen_quant.argtypes = [vp, C.POINTER(QuantAttnArgs)]
     lib.argus_hip_attention_gen_quant_ex.argtypes = [vp, C.POINTER(QuantAttnArgs), C.POINTER(QuantAttnExt)]
@@ -340,6 +347,17 @@ class Context:
                                      kv_heads=kv_heads, res_cap=res_cap, head_dim=head_dim,
                                      res_pos=res_pos, tok_base=tok_base)
         return self._check(lib.argus_hip_quant_scatter_residual(self.handle, C.byref(a)), check)
+
+    # -- (f-4) ---------------------------------------------------------------------------
+    def kv_decode_descriptor(self, desc, src, dst, n_elems, check=True):
+        d = KvLayoutDesc(*desc)
+        return self._check(lib.argus_hip_kv_decode_descriptor(self.handle, _stream(), C.byref(d), _ptr(src), _ptr(dst),
+                                                              _kv_dtype(dst), n_elems), check)
+
+    def kv_encode_descriptor(self, desc, src, dst, n_elems, check=True):
+        d = KvLayoutDesc(*desc)
+        return self._check(lib.argus_hip_kv_encode_descriptor(self.handle, _stream(), C.byref(d), _ptr(src), _ptr(dst),
+                                                              n_elems), check)
 
     # -- (a-4) ---------------------------------------------------------------------------
     def _score_args(self, scores, importance, head_importance, decay_factor, n_layers, n_heads_q,

@@ -309,6 +309,26 @@ typedef struct argus_hip_pfa_args {
 } argus_hip_pfa_args;
 int argus_hip_prefill_attention_scores(argus_hip_ctx *ctx, const argus_hip_pfa_args *args);
 
+/* ---- (f-4) descriptor-driven block formats: the device-side floor of --kv-format -------------
+ * KVLayoutDesc twin (crates/argus-extension-api/src/lib.rs:1111-1159): scale_layout 0 None,
+ * 1 PerBlockF16, 2 PerBlockF16WithMin; packing 0 Dense, 1 Nibble, 2 Byte, 3 Quad.
+ * kv_decode_descriptor = decode_via_descriptor / unpack_block_via_descriptor
+ * (engine/src/format/dtype_layout.rs:102-166, 285-300) into F32 or F16, bit-identical;
+ * kv_encode_descriptor = encode_via_descriptor (302-396), q4_0- and q2_0-style only, other
+ * descriptors return ARGUS_HIP_ERR_UNSUPPORTED like the reference's Err.  n_elems is a multiple of
+ * block_elems (<= 64); block buffers are 2-byte aligned.  They replace the host dequant-to-F32 of
+ * standard_format.rs:538-643 by a device pass followed by the F16/F32 attention entry points. */
+typedef struct argus_hip_kv_layout_desc {
+  uint32_t block_elems;
+  uint8_t bits;
+  uint32_t scale_layout;
+  uint32_t packing;
+} argus_hip_kv_layout_desc;
+int argus_hip_kv_decode_descriptor(argus_hip_ctx *ctx, void *stream, const argus_hip_kv_layout_desc *desc, const void *src,
+                                   void *dst, int32_t dst_dtype, int64_t n_elems);
+int argus_hip_kv_encode_descriptor(argus_hip_ctx *ctx, void *stream, const argus_hip_kv_layout_desc *desc, const void *src,
+                                   void *dst, int64_t n_elems);
+
 /* ---- (a-4) attention-score reduce for H2O / D2O --------------------------------------------- */
 /* Field-for-field twin of CudaScoreReduceArgs, crates/argus-extension-api/src/lib.rs:2909-2933;
  * CudaScoreReduceBackend::{reduce, reduce_per_layer} 2938-2948; kernel semantics

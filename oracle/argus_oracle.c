@@ -971,3 +971,113 @@ ORACLE_API int oracle_prefill_attention_scores(const float *q, const float *k, i
   free(scratch);
   return 0;
 }
+
+/* ---- descriptor-driven block formats (--kv-format floor) ---------------------------------------
+ * unpack_block_via_descriptor / decode_via_descriptor, engine/src/format/dtype_layout.rs:102-166,
+ * 285-300, and encode_via_descriptor with its two canonical encoders, 302-396.
+ * scale_layout: 0 None, 1 PerBlockF16, 2 PerBlockF16WithMin; packing: 0 Dense, 1 Nibble, 2 Byte,
+ * 3 Quad (argus-extension-api lib.rs:1111-1138).  Block = [f16 scale][f16 min?][packed quants]. */
+static int desc_block_bytes(int block_elems, int scale_layout, int packing) {
+  int q;
+  switch (packing) {
+    case 1: q = block_elems / 2; break;
+    case 2: q = block_elems; break;
+    case 3: q = block_elems / 4; break;
+    default: return -1;
+  }
+  return q + (scale_layout == 1 ? 2 : scale_layout == 2 ? 4 : 0);
+}
+
+ORACLE_API int oracle_desc_block_bytes(int block_elems, int scale_layout, int packing) {
+  return desc_block_bytes(block_elems, scale_layout, packing);
+}
+
+ORACLE_API int oracle_decode_via_descriptor(int block_elems, int bits, int scale_layout, int packing,
+                                            const uint8_t *src, float *dst, int64_t n_elems) {
+  const int bb = desc_block_bytes(block_elems, scale_layout, packing);
+  if (bb <= 0 || block_elems <= 0 || n_elems % block_elems) return -1;
+  const int n = block_elems;
+  for (int64_t bi = 0; bi < n_elems / n; ++bi) {
+    const uint8_t *block = src + bi * bb;
+    float *out = dst + bi * n;
+    uint16_t sb, mb = 0;
+    memcpy(&sb, block, 2);
+    const float scale = h2f(sb);
+    float min = 0.0f;
+    const uint8_t *quants = block + 2;
+    if (scale_layout == 2) {
+      memcpy(&mb, block + 2, 2);
+      min = h2f(mb);
+      quants = block + 4;
+    }
+    if (packing == 1) {
+      const int half = n / 2, is_signed = scale_layout == 1, zp = 1 << (bits - 1);
+      for (int i = 0; i < half; ++i) {
+        const int lo = quants[i] & 0x0f, hi = quants[i] >> 4;
+        if (is_signed) {
+          out[i] = (float)(lo - zp) * scale;
+          out[i + half] = (float)(hi - zp) * scale;
+        } else {
+          out[i] = (float)lo * scale + min;
+          out[i + half] = (float)hi * scale + min;
+        }
+      }
+    } else if (packing == 2) {
+      for (int i = 0; i < n; ++i) out[i] = (float)(int)(int8_t)quants[i] * scale;
+    } else {
+      for (int i = 0; i < n / 4; ++i)
+        for (int j = 0; j < 4; ++j) out[i * 4 + j] = (float)((quants[i] >> (j * 2)) & 3) * scale + min;
+    }
+  }
+  return 0;
+}
+
+ORACLE_API int oracle_encode_via_descriptor(int block_elems, int bits, int scale_layout, int packing,
+                                            const float *src, uint8_t *dst, int64_t n_elems) {
+  const int quad = (scale_layout == 2 && packing == 3);
+  if (!quad && !(scale_layout == 1 && packing == 1)) return -2;  /* outside the writable floor */
+  const int bb = desc_block_bytes(block_elems, scale_layout, packing);
+  if (block_elems <= 0 || n_elems % block_elems) return -1;
+  const int n = block_elems;
+  for (int64_t bi = 0; bi < n_elems / n; ++bi) {
+    const float *s = src + bi * n;
+    uint8_t *d8 = dst + bi * bb;
+    if (!quad) {
+      const float qmax = (float)((1 << (bits - 1)) - 1), qmin = -(float)(1 << (bits - 1));
+      const int zp = 1 << (bits - 1), half = n / 2;
+      float max_abs = 0.0f;
+      for (int i = 0; i < n; ++i) max_abs = fmaxf(max_abs, fabsf(s[i]));  /* f32::max ignores NaN like fmaxf */
+      const float d = max_abs / qmax;
+      const float id = d == 0.0f ? 0.0f : 1.0f / d;
+      const uint16_t db = f2h(d);
+      memcpy(d8, &db, 2);
+      for (int i = 0; i < half; ++i) {
+        const int v0 = (int)fminf(fmaxf(roundf(s[i] * id), qmin), qmax);
+        const int v1 = (int)fminf(fmaxf(roundf(s[i + half] * id), qmin), qmax);
+        d8[2 + i] = (uint8_t)((uint8_t)(v0 + zp) | ((uint8_t)(v1 + zp) << 4));
+      }
+    } else {
+      const float qmax = (float)((1u << bits) - 1u);
+      const int per_byte = 8 / bits;
+      float mn = INFINITY, mx = -INFINITY;
+      for (int i = 0; i < n; ++i) {
+        mn = fminf(mn, s[i]);
+        mx = fmaxf(mx, s[i]);
+      }
+      const float d = (mx - mn) / qmax;
+      const float id = d == 0.0f ? 0.0f : 1.0f / d;
+      const uint16_t db = f2h(d), mb = f2h(mn);
+      memcpy(d8, &db, 2);
+      memcpy(d8 + 2, &mb, 2);
+      for (int i = 0; i < n / per_byte; ++i) {
+        uint8_t byte = 0;
+        for (int j = 0; j < per_byte; ++j) {
+          const uint8_t qv = (uint8_t)fminf(fmaxf(roundf((s[i * per_byte + j] - mn) * id), 0.0f), qmax);
+          byte |= (uint8_t)(qv << (j * bits));
+        }
+        d8[4 + i] = byte;
+      }
+    }
+  }
+  return 0;
+}

@@ -89,6 +89,9 @@ _compact = _sig("oracle_compact_keep", None, [
 _pfa = _sig("oracle_prefill_attention_scores", C.c_int, [
     _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_int,
     C.c_int, _f32p, _f32p, C.c_int])
+_desc_bb = _sig("oracle_desc_block_bytes", C.c_int, [C.c_int, C.c_int, C.c_int])
+_desc_dec = _sig("oracle_decode_via_descriptor", C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, _u8p, _f32p, C.c_int64])
+_desc_enc = _sig("oracle_encode_via_descriptor", C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _u8p, C.c_int64])
 _scatter = _sig("oracle_kv_scatter", None, [
     _f32p, _f32p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int])
 
@@ -365,3 +368,37 @@ def prefill_attention_scores(q, k, n_heads_q, n_heads_kv, head_dim, seq_len, cac
               _p(sum_out, _f32p), _p(per_row, _f32p), 1 if per_head else 0)
     if rc != 0:
         raise ValueError("oracle prefill_attention_scores rc=%d" % rc)
+
+
+# KVLayoutDesc vocabulary (argus-extension-api lib.rs:1111-1159): (block_elems, bits, scale_layout, packing)
+SCALE_NONE, SCALE_F16, SCALE_F16_MIN = 0, 1, 2
+PACK_DENSE, PACK_NIBBLE, PACK_BYTE, PACK_QUAD = 0, 1, 2, 3
+DESC_Q4_0 = (32, 4, SCALE_F16, PACK_NIBBLE)
+DESC_Q4_1 = (32, 4, SCALE_F16_MIN, PACK_NIBBLE)
+DESC_Q8_0 = (32, 8, SCALE_F16, PACK_BYTE)
+DESC_Q2_0 = (32, 2, SCALE_F16_MIN, PACK_QUAD)
+
+
+def desc_block_bytes(desc):
+    return _desc_bb(desc[0], desc[2], desc[3])
+
+
+def decode_via_descriptor(desc, raw, n_elems):
+    """decode_via_descriptor / unpack_block_via_descriptor (format/dtype_layout.rs:102-166, 285-300)."""
+    raw = np.ascontiguousarray(raw, np.uint8)
+    out = np.zeros(n_elems, np.float32)
+    rc = _desc_dec(desc[0], desc[1], desc[2], desc[3], _p(raw, _u8p), _p(out, _f32p), n_elems)
+    if rc != 0:
+        raise ValueError("oracle decode_via_descriptor rc=%d" % rc)
+    return out
+
+
+def encode_via_descriptor(desc, src):
+    """encode_via_descriptor (format/dtype_layout.rs:302-396): q4_0 (PerBlockF16 + Nibble) and q2_0
+    (PerBlockF16WithMin + Quad) only; anything else raises like the reference's Err."""
+    src = np.ascontiguousarray(src, np.float32).reshape(-1)
+    out = np.zeros(src.size // desc[0] * max(desc_block_bytes(desc), 1), np.uint8)
+    rc = _desc_enc(desc[0], desc[1], desc[2], desc[3], _p(src, _f32p), _p(out, _u8p), src.size)
+    if rc != 0:
+        raise ValueError("oracle encode_via_descriptor rc=%d" % rc)
+    return out

@@ -31,7 +31,7 @@ def test_struct_layouts_match_header_field_order():
     text = open(os.path.join(ROOT, "include", "argus_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     pairs = {"argus_hip_attention_gen_args": A.AttentionGenArgs, "argus_hip_prefill_args": A.PrefillArgs,
-             "argus_hip_pfa_args": A.PfaArgs,
+             "argus_hip_pfa_args": A.PfaArgs, "argus_hip_kv_layout_desc": A.KvLayoutDesc,
              "argus_hip_quant_attn_args": A.QuantAttnArgs, "argus_hip_quant_attn_ext": A.QuantAttnExt,
              "argus_hip_quant_gather_args": A.QuantGatherArgs, "argus_hip_quant_flush_args": A.QuantFlushArgs,
              "argus_hip_quant_dequant_flush_args": A.QuantDequantFlushArgs,
