@@ -159,7 +159,10 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   // iteration still separates every fill from the reads before and after it.
   _Float16 *const sKb = smem;                         // [2][NG][BN * KP]
   _Float16 *const sVb = smem + 2 * NG * BN * KP;      // [2][NG][BN * VP]
-  half8_t kpre[CH], vpre[CH];
+  // kDeep: tiles are fetched one step earlier than they are staged (two register sets, alternating
+  // by step parity), so a fetch has a whole extra step to arrive; used where registers allow.
+  constexpr bool kDeep = D <= 64;
+  half8_t kpre[kDeep ? 2 : 1][CH], vpre[kDeep ? 2 : 1][CH];
   // Chunk cid of an iteration's NG tiles is the 16 bytes at element 8*cid from the first tile's
   // first row (the tiles are adjacent in the cache), so a fetch is a uniform base plus a per-thread
   // offset; only an iteration that reaches past the visible keys needs per-chunk bounds checks.
@@ -179,24 +182,26 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
       }
     }
   };
-  auto fetch_k = [&](int it) { fetch_tiles(kbase, it, kpre); };
-  auto fetch_v = [&](int it) { fetch_tiles(vbase, it, vpre); };
-  auto stage_k = [&](int buf) {
+  auto fetch_k = [&](int it, auto set_c) { fetch_tiles(kbase, it, kpre[decltype(set_c)::value]); };
+  auto fetch_v = [&](int it, auto set_c) { fetch_tiles(vbase, it, vpre[decltype(set_c)::value]); };
+  auto stage_k = [&](int buf, auto set_c) {
+    constexpr int SET = decltype(set_c)::value;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int cid = threadIdx.x + NT * c;
       const int trow = cid / (D / 8), dc = cid % (D / 8);
       const int g = trow / BN, key = trow % BN;
-      *(half8_t *)(sKb + (buf * NG + g) * (BN * KP) + key * KP + 8 * dc) = kpre[c];
+      *(half8_t *)(sKb + (buf * NG + g) * (BN * KP) + key * KP + 8 * dc) = kpre[SET][c];
     }
   };
-  auto stage_v = [&](int buf) {
+  auto stage_v = [&](int buf, auto set_c) {
+    constexpr int SET = decltype(set_c)::value;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int cid = threadIdx.x + NT * c;
       const int trow = cid / (D / 8), dc = cid % (D / 8);
       const int g = trow / BN, key = trow % BN;
-      *(half8_t *)(sVb + (buf * NG + g) * (BN * VP) + key * VP + 8 * dc) = vpre[c];
+      *(half8_t *)(sVb + (buf * NG + g) * (BN * VP) + key * VP + 8 * dc) = vpre[SET][c];
     }
   };
 
@@ -336,33 +341,45 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   // of tile it+1.  Interior steps (every tile of the iteration lies below the diagonal of every
   // wave, inside the cache and the window, and there is a next iteration) have no per-wave
   // conditions, so each phase is one basic block the scheduler can interleave.
-  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], TileMax &t_cur, auto interior_c) {
+  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], TileMax &t_cur, auto interior_c, auto parity_c) {
     constexpr bool INTERIOR = decltype(interior_c)::value;
+    // register set fetched into during this step, and the one staged at its end
+    typedef std::integral_constant<int, kDeep ? decltype(parity_c)::value : 0> FetchSet;
+    typedef std::integral_constant<int, kDeep ? 1 - decltype(parity_c)::value : 0> StageSet;
+    constexpr int AHEAD = kDeep ? 1 : 0;
     const bool act = INTERIOR || tile_active(it);
     const bool has_next = INTERIOR || it + 1 < n_it;
     if (act) rescale(t_cur);  // its branch stays out of the phases below
-    if (it + 2 < n_it) fetch_k(it + 2);
-    if (has_next) fetch_v(it + 1);
+    if (it + 2 + AHEAD < n_it) fetch_k(it + 2 + AHEAD, FetchSet{});
+    if (it + 1 + AHEAD < n_it) fetch_v(it + 1 + AHEAD, FetchSet{});
     // ---- phase A
     if (has_next) qk_tile(it + 1, s_next);  // harmless on a tile the wave cannot see
     if (act) exp_tile(s_cur, t_cur);
     // ---- phase B
     if (act) pv_tile(it);
     if (INTERIOR || tile_active(it + 1)) t_cur = mask_max(it + 1, s_next, interior_c);
-    if (it + 2 < n_it) stage_k(it & 1);
-    if (has_next) stage_v((it + 1) & 1);
+    if (it + 2 < n_it) stage_k(it & 1, StageSet{});
+    if (has_next) stage_v((it + 1) & 1, StageSet{});
     __syncthreads();  // fills are visible; every wave is done with the buffers the next step refills
   };
 
   float16_t s_a[KB], s_b[KB];
-  if (n_it > 0) {
-    fetch_k(0);
-    fetch_v(0);
-    stage_k(0);
-    stage_v(0);
-    if (n_it > 1) {
-      fetch_k(1);
-      stage_k(1);
+  {
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, kDeep ? 1 : 0> Set1;
+    if (n_it > 0) {
+      fetch_k(0, Set0{});
+      fetch_v(0, Set0{});
+      stage_k(0, Set0{});
+      stage_v(0, Set0{});
+      if (n_it > 1) {
+        fetch_k(1, Set0{});
+        stage_k(1, Set0{});
+      }
+    }
+    if constexpr (kDeep) {  // what step 0 stages at its end
+      if (n_it > 2) fetch_k(2, Set1{});
+      if (n_it > 1) fetch_v(1, Set1{});
     }
   }
   __syncthreads();
@@ -378,12 +395,12 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   }
   int it = 0;
   for (; it < n_int; it += 2) {
-    step(it, s_a, s_b, t_cur, std::true_type{});
-    step(it + 1, s_b, s_a, t_cur, std::true_type{});
+    step(it, s_a, s_b, t_cur, std::true_type{}, std::integral_constant<int, 0>{});
+    step(it + 1, s_b, s_a, t_cur, std::true_type{}, std::integral_constant<int, 1>{});
   }
   for (; it < n_it; it += 2) {
-    step(it, s_a, s_b, t_cur, std::false_type{});
-    if (it + 1 < n_it) step(it + 1, s_b, s_a, t_cur, std::false_type{});
+    step(it, s_a, s_b, t_cur, std::false_type{}, std::integral_constant<int, 0>{});
+    if (it + 1 < n_it) step(it + 1, s_b, s_a, t_cur, std::false_type{}, std::integral_constant<int, 1>{});
   }
 
   // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
