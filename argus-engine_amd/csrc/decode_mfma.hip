@@ -45,13 +45,14 @@ struct VPiece<8> { using type = half8_t; };
 template <>
 struct VPiece<4> { using type = half4_t; };
 
-template <int D, int TW>
+template <int D, int TW, bool SOFTCAP>
 __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) {
   using SH = MfmaShape<D>;
   constexpr int KK = SH::KK, VC = SH::VC, VSEG = SH::VSEG, NACC = SH::NACC;
   using vpiece_t = typename VPiece<VC>::type;
   constexpr int TILE = 16 * TW;  // tokens per wave iteration
-  constexpr float kLn2 = 0.6931471805599453f;
+  constexpr float kLn2 = 0.6931471805599453f, kLog2e = 1.4426950408889634f;
+  const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
 
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -127,7 +128,13 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
     for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float sv = fmaxf(s[tw][i], kNegInf);  // NaN logit counts as -inf (common.rs:555-560)
+        float sv = s[tw][i];
+        if constexpr (SOFTCAP) {
+          // cap * tanh(logit / cap) on the natural-unit logit (flash_attn_f32_f16.cl:563-565), back to log2 units
+          const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * kLog2e;
+          sv = (sv != sv) ? kNegInf : capped;
+        }
+        sv = fmaxf(sv, kNegInf);  // NaN logit counts as -inf (common.rs:555-560)
         if (!full && base + 16 * tw + 4 * j + i >= t_end) sv = kNegInf;
         s[tw][i] = sv;
         mt = fmaxf(mt, sv);
@@ -258,7 +265,8 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   {
     KernelTimer timer(ctx, stream);
-    hipLaunchKernelGGL((decode_mfma_kernel<D, TW>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, p);
+    if (p.softcap > 0.0f) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -269,8 +277,12 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
 }  // namespace
 
 bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
-  return kv_dtype == ARGUS_HIP_F16 && !p.kv_index && !(p.softcap > 0.0f) && p.group <= (D == 256 ? 8 : 16) &&
-         (D == 64 || D == 128 || D == 256) && p.len >= 64;
+  if (kv_dtype != ARGUS_HIP_F16 || p.kv_index || p.len < 64) return false;
+  if (D == 64 || D == 128) return p.group <= 16;
+  // head_dim 256: one 64-row tile per workgroup costs more set-up (Q split over 256 channels) than it
+  // saves; measured against the vector-ALU kernel it only pays for long rows and wider groups
+  // (Hq8/Hkv4, L 2048: 30 us vs 17 us; L 32768: equal).
+  return D == 256 && p.group >= 4 && p.group <= 8 && p.len >= 8192;
 }
 
 int launch_decode_mfma(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hipStream_t stream) {

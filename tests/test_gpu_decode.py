@@ -144,6 +144,29 @@ def test_softcap_index_and_window_start():
     check_attention_out(got, ref)
 
 
+@pytest.mark.parametrize("hq,hkv,d,L,cap", [(32, 8, 128, 1500, 1536), (14, 2, 64, 777, 800)])
+def test_softcap_on_the_matrix_core_path(hq, hkv, d, L, cap):
+    # F16 KV, no index list, d in {64, 128}: soft-capped logits run through the MFMA kernel; same
+    # definition (cap * tanh(logit / cap)), emitted scores included; a NaN key still counts as -inf.
+    q = normal((hq, d), 61) * 2.0
+    k = f16(normal((hkv, cap, d), 62))
+    v = f16(normal((hkv, cap, d), 63))
+    for softcap in (5.0, 50.0):
+        got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, softcap=softcap)
+        ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, softcap=softcap)
+        check_attention_out(got, ref)
+        check_scores(sc, p)
+        r64, p64 = T.decode_attention(q, k, v, hkv, L, softcap=softcap)
+        check_attention_out(got, r64)
+    k2 = k.copy()
+    k2[0, 5, 3] = np.float16(np.nan)
+    got, sc = run_decode(q, k2, v, hkv, L, cap, scores=True, softcap=5.0)
+    ref, p = O.attention_gen(q, k2, v, hkv, L, cap, scores=True, softcap=5.0)
+    check_attention_out(got, ref)
+    check_scores(sc, p)
+    assert (sc[:hq // hkv, 5] == 0).all()
+
+
 def test_batched_sequences_match_looped_calls():
     # the reference has no batch dimension (engine/src/backend.rs:277-295): batch == a loop.
     b, hq, hkv, d, L, cap = 5, 32, 8, 128, 1500, 1536
