@@ -140,6 +140,21 @@ __host__ __device__ constexpr int field_shift_v(int which) {
   return BITS == 8 ? 0 : BITS == 4 ? 4 * which : 6 + 2 * which;
 }
 
+// 8 consecutive residual elements (16-byte aligned) as floats
+__device__ __forceinline__ void load_row8(const float *p, float (&o)[8]) {
+  const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    o[e] = a[e];
+    o[4 + e] = b[e];
+  }
+}
+__device__ __forceinline__ void load_row8(const _Float16 *p, float (&o)[8]) {
+  const half8_t a = *(const half8_t *)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (float)a[e];
+}
+
 constexpr float kLn2 = 0.6931471805599453f;
 // Power of two on the f16 operands that carry block scales: keeps the low halves of the hi + lo
 // splits and small p*d products out of the f16 subnormal range.
@@ -440,11 +455,13 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
         const RES_T *row = rk + (int64_t)min(2 * r + w, n_valid - 1) * D + 32 * kk + 8 * j;
+        float rowv[8];
+        load_row8(row, rowv);
         half8_t ah, al;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           _Float16 hi, lo;
-          split_f16((float)row[e], hi, lo);
+          split_f16(rowv[e], hi, lo);
           ah[e] = hi;
           al[e] = lo;
         }
@@ -565,6 +582,8 @@ bool kivi_mfma_supported(const KiviParams &kp) {
   if (p.group > 8 || p.softcap > 0.0f) return false;
   // tiles are copied as 16-byte vectors
   if ((((uintptr_t)kp.qk | (uintptr_t)kp.qv) & 15) || (kp.qk_bs & 15) || (kp.qv_bs & 15)) return false;
+  // residual rows are read as 16-byte vectors
+  if ((((uintptr_t)kp.res_k | (uintptr_t)kp.res_v) & 15) || (kp.res_bs & 7)) return false;
   return true;
 }
 
