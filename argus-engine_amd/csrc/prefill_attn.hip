@@ -370,11 +370,14 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     if (n_it > 0) {
       fetch_k(0, Set0{});
       fetch_v(0, Set0{});
+      if constexpr (kDeep) {  // second register set: all three first tiles in one round trip
+        if (n_it > 1) fetch_k(1, Set1{});
+      }
       stage_k(0, Set0{});
       stage_v(0, Set0{});
       if (n_it > 1) {
-        fetch_k(1, Set0{});
-        stage_k(1, Set0{});
+        if constexpr (!kDeep) fetch_k(1, Set0{});
+        stage_k(1, Set1{});
       }
     }
     if constexpr (kDeep) {  // what step 0 stages at its end
