@@ -77,23 +77,46 @@ constexpr int kMaxSplits = 128;
 
 template <typename FALLBACK, int D>
 __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams p) {
-  constexpr int CQ = D / 4;      // float4 columns per row
-  constexpr int NSG = 256 / CQ;  // split groups
+  constexpr int CQ = D / 4;                // float4 columns per row
+  constexpr int NSG = 256 / CQ;            // split groups
+  constexpr int PER = kMaxSplits / NSG;    // splits per thread at most
   const int h = blockIdx.x, b = blockIdx.y;
   const int64_t pbase = ((int64_t)b * p.n_heads_q + h) * p.nsplit;
+  const int cq = threadIdx.x % CQ, sg = threadIdx.x / CQ;
   __shared__ float sh_w[kMaxSplits];
   __shared__ float sh_m, sh_l;
   __shared__ float4_t sh_o[NSG][CQ];
+  // The pass is one memory round trip long if nothing waits on anything else, so the partial
+  // outputs are requested before the (m, l) pairs that weight them.  Slots past the last split
+  // re-read it and get weight zero.
+  const int last = p.nsplit - 1;
+  float4_t part[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    if (i * NSG > last) break;  // uniform
+    part[i] = *(const float4_t *)(p.ws_o + (pbase + min(sg + i * NSG, last)) * D + 4 * cq);
+  }
   if (threadIdx.x < 64) {
+    constexpr int MLP = kMaxSplits / 64;
+    float pm[MLP], pl[MLP];
+#pragma unroll
+    for (int i = 0; i < MLP; ++i) {
+      const int s = min((int)threadIdx.x + 64 * i, last);
+      pm[i] = p.ws_ml[(pbase + s) * 2];
+      pl[i] = p.ws_ml[(pbase + s) * 2 + 1];
+    }
     float mm = kNegInf;
-    for (int s = threadIdx.x; s < p.nsplit; s += 64) mm = fmaxf(mm, p.ws_ml[(pbase + s) * 2]);
+#pragma unroll
+    for (int i = 0; i < MLP; ++i) mm = fmaxf(mm, pm[i]);
     mm = wave_allreduce_max(mm);
     const float m_ref = (mm == kNegInf) ? 0.0f : mm;
     float ll = 0.0f;
-    for (int s = threadIdx.x; s < p.nsplit; s += 64) {
-      const float w = __expf(p.ws_ml[(pbase + s) * 2] - m_ref);
+#pragma unroll
+    for (int i = 0; i < MLP; ++i) {
+      const int s = threadIdx.x + 64 * i;
+      const float w = (s <= last) ? __expf(pm[i] - m_ref) : 0.0f;
       sh_w[s] = w;
-      ll += p.ws_ml[(pbase + s) * 2 + 1] * w;
+      ll += pl[i] * w;
     }
     ll = wave_allreduce_sum(ll);
     if (threadIdx.x == 0) {
@@ -107,10 +130,12 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     if (FALLBACK::run(p, b, h, D)) return;
   }
   const float inv = 1.0f / ll;  // non-finite when the fallback declined: NaN propagates
-  const int cq = threadIdx.x % CQ, sg = threadIdx.x / CQ;
   float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int s = sg; s < p.nsplit; s += NSG)
-    o += *(const float4_t *)(p.ws_o + (pbase + s) * D + 4 * cq) * sh_w[s];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    if (i * NSG > last) break;
+    o += part[i] * sh_w[sg + i * NSG];
+  }
   sh_o[sg][cq] = o;
   __syncthreads();
   if (sg == 0) {

@@ -38,6 +38,22 @@ struct MfmaShape {
   static constexpr int MAXH = (D == 256) ? 8 : 16;  // query heads per KV head (bounds the merge LDS)
 };
 
+// dword 3 of a raw (untyped, unstrided) buffer descriptor on this target
+constexpr int kBufferFlags = 0x00020000;
+
+// Bounds-checked streaming (non-temporal) load of 8 or 16 bytes: byte offsets `voff` per lane,
+// `soff` wave-uniform.
+template <typename T>
+__device__ __forceinline__ T buffer_load_stream(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff);
+template <>
+__device__ __forceinline__ half8_t buffer_load_stream<half8_t>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 2));
+}
+template <>
+__device__ __forceinline__ half4_t buffer_load_stream<half4_t>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(half4_t, __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, soff, 2));
+}
+
 template <int VC>
 struct VPiece;
 template <>
@@ -45,8 +61,13 @@ struct VPiece<8> { using type = half8_t; };
 template <>
 struct VPiece<4> { using type = half4_t; };
 
+// Waves per workgroup, each taking every kWaves-th tile of the workgroup's chunk.  (Eight waves
+// drawing tiles from a counter in LDS evened out the finish times of the workgroups but moved
+// less data per microsecond: 27.4 us against 26.4 us on one 32K-token sequence.)
+constexpr int kWaves = 4;
+
 template <int D, int TW, bool SOFTCAP>
-__global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodeParams p) {
   using SH = MfmaShape<D>;
   constexpr int KK = SH::KK, VC = SH::VC, VSEG = SH::VSEG, NACC = SH::NACC;
   using vpiece_t = typename VPiece<VC>::type;
@@ -65,6 +86,43 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
   const _Float16 *kb = (const _Float16 *)p.k + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;
   const _Float16 *vb = (const _Float16 *)p.v + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;
 
+  // K/V rows are read through buffer descriptors that end at the chunk's last row: rows past it
+  // come back as zeros without touching memory, so every iteration issues the same loads (the
+  // compiler then waits for exactly the ones it needs) and a tile may be requested before it is
+  // known to exist.  Offsets: a per-lane constant plus the wave-uniform first row of the tile.
+  const int64_t rs = p.row_stride;
+  const uint32_t slab_bytes = (uint32_t)((int64_t)(p.kv_start + t_end) * rs * 2);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)kb, 0, slab_bytes, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)vb, 0, slab_bytes, kBufferFlags);
+  const uint32_t k_lane = (uint32_t)(((int64_t)(p.kv_start + r) * rs + 8 * j) * 2);
+  const uint32_t v_lane = (uint32_t)(((int64_t)(p.kv_start + 4 * j) * rs + VC * r) * 2);
+  const uint32_t row_bytes = (uint32_t)(rs * 2);
+  half8_t kr[TW][KK];
+  vpiece_t vr[TW][VSEG][4];
+  auto load_k = [&](int base) {  // TW tiles of 16 tokens starting at token `base`
+    const uint32_t tile = (uint32_t)base * row_bytes;
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+        kr[tw][kk] = buffer_load_stream<half8_t>(k_rsrc, k_lane + 16 * tw * row_bytes + 64 * kk, tile);
+  };
+  auto load_v = [&](int base) {
+    const uint32_t tile = (uint32_t)base * row_bytes;
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int sg = 0; sg < VSEG; ++sg)
+          vr[tw][sg][e] = buffer_load_stream<vpiece_t>(v_rsrc, v_lane + (16 * tw + e) * row_bytes + 32 * VC * sg, tile);
+  };
+  // The first tile is requested before the query is prepared, so both arrive together.
+  const int base0 = t_begin + __builtin_amdgcn_readfirstlane(wave) * TILE;
+  load_k(base0);
+  load_v(base0);
+  __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the query's
+
   // ---- Q operand: lane (j, h = r) holds chunk 4kk + j of head h, scaled to the log2 domain ------
   half8_t qh[KK], ql[KK];
   {
@@ -75,7 +133,8 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
     for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float x = (r < G) ? qp[(4 * kk + j) * 8 + e] * c : 0.0f;
+        const float qv = qp[(4 * kk + j) * 8 + e];  // unconditional: lanes past the group re-read its last head
+        const float x = (r < G) ? qv * c : 0.0f;
         _Float16 hi, lo;
         split_f16(x, hi, lo);
         qh[kk][e] = hi;
@@ -89,28 +148,7 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
   for (int a = 0; a < NACC; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
 
-  const int64_t rs = p.row_stride;
-  for (int base = t_begin + wave * TILE; base < t_end; base += 4 * TILE) {
-    // ---- loads: TW tiles of 16 tokens -----------------------------------------------------------
-    half8_t kr[TW][KK];
-    vpiece_t vr[TW][VSEG][4];
-#pragma unroll
-    for (int tw = 0; tw < TW; ++tw) {
-      const int t0 = base + 16 * tw;
-      const int krow = min(t0 + r, t_end - 1) + p.kv_start;
-      const _Float16 *kp = kb + (int64_t)krow * rs + 8 * j;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) kr[tw][kk] = __builtin_nontemporal_load((const half8_t *)(kp + 32 * kk));
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int vrow = min(t0 + 4 * j + e, t_end - 1) + p.kv_start;
-        const _Float16 *vp = vb + (int64_t)vrow * rs + VC * r;
-#pragma unroll
-        for (int sg = 0; sg < VSEG; ++sg)
-          vr[tw][sg][e] = __builtin_nontemporal_load((const vpiece_t *)(vp + 16 * VC * sg));
-      }
-    }
-
+  for (int base = base0; base < t_end; base += kWaves * TILE) {
     // ---- logits ---------------------------------------------------------------------------------
     float4_t s[TW];
 #pragma unroll
@@ -122,6 +160,8 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
         s[tw] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kr[tw][kk], ql[kk], s[tw], 0, 0, 0);
       }
     }
+    // The K registers are free again: request the wave's next tile (past the chunk: zeros, no traffic).
+    load_k(base + kWaves * TILE);
     const bool full = base + TILE <= t_end;
     float mt = kNegInf;
 #pragma unroll
@@ -191,13 +231,14 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
           const half4_t bv = {vr[tw][sg][0][c], vr[tw][sg][1][c], vr[tw][sg][2][c], vr[tw][sg][3][c]};
           o_acc[sg * VC + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * VC + c], 0, 0, 0);
         }
+    load_v(base + kWaves * TILE);
   }
 
-  // ---- merge: lane groups (row sum), then the 4 waves through LDS -------------------------------
+  // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  __shared__ float lds_m[4][16], lds_l[4][16];
-  __shared__ float lds_acc[4][SH::MAXH][D + 4];
+  __shared__ float lds_m[kWaves][16], lds_l[kWaves][16];
+  __shared__ float lds_acc[kWaves][SH::MAXH][D + 4];
   if (j == 0) {
     lds_m[wave][r] = m_run;
     lds_l[wave][r] = l_run;
@@ -211,14 +252,16 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
         if (4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][16 * VC * sg + VC * r + c] = o_acc[sg * VC + c][i];
   __syncthreads();
 
-  for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+  for (int idx = threadIdx.x; idx < G * D; idx += 64 * kWaves) {
     const int g = idx / D, c = idx % D;
     const int h = kvh * G + g;
-    const float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
+    float mm = lds_m[0][g];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, lds_m[w][g]);
     const float m_ref = (mm == kNegInf) ? 0.0f : mm;
     float o = 0.0f, ll = 0.0f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < kWaves; ++w) {
       const float f = __builtin_amdgcn_exp2f(lds_m[w][g] - m_ref);
       o += lds_acc[w][g][c] * f;
       ll += lds_l[w][g] * f;
@@ -235,25 +278,36 @@ __global__ __launch_bounds__(256) void decode_mfma_kernel(const DecodeParams p) 
 
 template <int D>
 int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
-#ifdef ARGUS_MFMA_TW
-  constexpr int TW = ARGUS_MFMA_TW;
-#else
   constexpr int TW = (D <= 128) ? 2 : 1;
-#endif
-  constexpr int tile_rows = 4 * 16 * TW;
+  constexpr int tile_rows = kWaves * 16 * TW;  // one tile per wave
   const int pairs = batch * p.n_heads_kv;
-#ifdef ARGUS_MFMA_WGMUL
-  const int target_wgs = ctx->compute_units * ARGUS_MFMA_WGMUL;
-#else
-  // About one round of resident workgroups (3 per CU at this register count) measured best:
-  // long chunks amortise the Q set-up and the cross-wave merge.
-  const int target_wgs = ctx->compute_units * 4;
-#endif
-  const int max_splits = (p.len + tile_rows - 1) / tile_rows;
-  int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, max_splits, kMaxSplits}));
-  int chunk = (p.len + nsplit - 1) / nsplit;
-  chunk = (chunk + tile_rows - 1) / tile_rows * tile_rows;
-  nsplit = (p.len + chunk - 1) / chunk;
+  // The grid is sized against the number of workgroups the device holds at once: when the splits
+  // fill it in one round every workgroup starts together and streams an equal share, each wave
+  // requesting its next tile while it works on the current one; a partial extra round runs thinly
+  // occupied (one 32K-token sequence: 2 rounds of 2-tile waves were 10 % slower than 1 round of
+  // 4-tile waves).  Cost model, in units of one tile step with the device full: rounds x (tile
+  // steps per workgroup + 0.75 for set-up, merge and partial write-out).
+  static int wgs_per_cu = 0;  // per head_dim instantiation; single inference thread
+  if (wgs_per_cu == 0) {
+    int n = 0;
+    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_mfma_kernel<D, TW, false>, 64 * kWaves, 0));
+    wgs_per_cu = std::max(1, n);
+  }
+  const int64_t slots = (int64_t)ctx->compute_units * wgs_per_cu;
+  const int max_splits = std::min((p.len + tile_rows - 1) / tile_rows, kMaxSplits);
+  int nsplit = 1, chunk = (p.len + tile_rows - 1) / tile_rows * tile_rows;
+  float best = 3.0e38f;
+  for (int n = 1; n <= max_splits; ++n) {
+    const int c = ((p.len + n - 1) / n + tile_rows - 1) / tile_rows * tile_rows;
+    const int ns = (p.len + c - 1) / c;
+    const int64_t rounds = ((int64_t)pairs * ns + slots - 1) / slots;
+    const float cost = (float)rounds * ((float)(c / tile_rows) + 0.75f);
+    if (cost < best) {
+      best = cost;
+      nsplit = ns;
+      chunk = c;
+    }
+  }
   p.chunk = chunk;
   p.nsplit = nsplit;
   p.direct = 0;
@@ -265,8 +319,8 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   {
     KernelTimer timer(ctx, stream);
-    if (p.softcap > 0.0f) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false>), dim3(nsplit, p.n_heads_kv, batch), dim3(256), 0, stream, p);
+    if (p.softcap > 0.0f) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true>), dim3(nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
+    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false>), dim3(nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -278,6 +332,8 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
 
 bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
   if (kv_dtype != ARGUS_HIP_F16 || p.kv_index || p.len < 64) return false;
+  // rows are addressed with 32-bit byte offsets from the head's first row, a few tiles past the end
+  if (((int64_t)p.kv_start + p.len + 1024) * p.row_stride * 2 > 0x7fffffffll) return false;
   if (D == 64 || D == 128) return p.group <= 16;
   // head_dim 256: one 64-row tile per workgroup costs more set-up (Q split over 256 channels) than it
   // saves; measured against the vector-ALU kernel it only pays for long rows and wider groups

@@ -48,14 +48,32 @@ __device__ __forceinline__ half4_t lds_read_tr16(const _Float16 *p) {
   return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)p));
 }
 
+// dword 3 of a raw (untyped, unstrided) buffer descriptor on this target
+constexpr int kBufferFlags = 0x00020000;
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// 8 consecutive K or V elements as f16, read through a bounds-checked buffer descriptor
+// (byte offsets: per-lane `voff`, wave-uniform `soff`); out-of-range chunks read as zero.
 template <typename KV_T>
-__device__ __forceinline__ half8_t load_kv_chunk(const KV_T *p);
+__device__ __forceinline__ half8_t load_kv_chunk(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff);
 template <>
-__device__ __forceinline__ half8_t load_kv_chunk<_Float16>(const _Float16 *p) {
-  return *(const half8_t *)p;
+__device__ __forceinline__ half8_t load_kv_chunk<_Float16>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0));
 }
 template <>
-__device__ __forceinline__ half8_t load_kv_chunk<float>(const float *p) {
+__device__ __forceinline__ half8_t load_kv_chunk<float>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+  const float4_t a = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0));
+  const float4_t b = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + 16, soff, 0));
+  half8_t h;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    h[e] = (_Float16)a[e];
+    h[4 + e] = (_Float16)b[e];
+  }
+  return h;
+}
+// 8 consecutive f32 query elements rounded to f16
+__device__ __forceinline__ half8_t load_q_f32(const float *p) {
   const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
   half8_t h;
 #pragma unroll
@@ -126,7 +144,7 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
       half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
       if (row_ok) {
         if (p.q_f16) x = *(const half8_t *)((const _Float16 *)p.q + qoff + 16 * kk);
-        else x = load_kv_chunk<float>((const float *)p.q + qoff + 16 * kk);
+        else x = load_q_f32((const float *)p.q + qoff + 16 * kk);
       }
       qreg[kk] = x;
     }
@@ -164,26 +182,22 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   constexpr bool kDeep = D <= 64;
   half8_t kpre[kDeep ? 2 : 1][CH], vpre[kDeep ? 2 : 1][CH];
   // Chunk cid of an iteration's NG tiles is the 16 bytes at element 8*cid from the first tile's
-  // first row (the tiles are adjacent in the cache), so a fetch is a uniform base plus a per-thread
-  // offset; only an iteration that reaches past the visible keys needs per-chunk bounds checks.
-  auto fetch_tiles = [&](const KV_T *base, int it, half8_t(&pre)[CH]) {
-    const int key_first = (kt_begin + it * NG) * BN;
-    const KV_T *tile = base + (int64_t)key_first * D;
-    if (key_first + NG * BN <= kv_end) {
+  // first row (the tiles are adjacent in the cache), so a fetch is a scalar tile offset plus a
+  // per-thread constant.  The loads go through a buffer descriptor that ends at the last visible
+  // key: rows past it come back as zeros from the bounds check, with no branch and no address
+  // arithmetic, and every step issues the same number of loads, which lets the compiler wait for
+  // exactly the loads a staging step needs and leave the younger ones in flight.
+  const uint32_t kv_bytes = (uint32_t)kv_end * D * sizeof(KV_T);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)kbase, 0, kv_bytes, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)vbase, 0, kv_bytes, kBufferFlags);
+  auto fetch_tiles = [&](__amdgpu_buffer_rsrc_t rsrc, int it, half8_t(&pre)[CH]) {
+    const uint32_t tile_off = (uint32_t)((kt_begin + it * NG) * BN) * (D * sizeof(KV_T));
 #pragma unroll
-      for (int c = 0; c < CH; ++c) pre[c] = load_kv_chunk<KV_T>(tile + (size_t)c * (NT * 8) + threadIdx.x * 8);
-    } else {
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int cid = threadIdx.x + NT * c;
-        half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (key_first + cid / (D / 8) < kv_end) x = load_kv_chunk<KV_T>(tile + (size_t)cid * 8);
-        pre[c] = x;
-      }
-    }
+    for (int c = 0; c < CH; ++c)
+      pre[c] = load_kv_chunk<KV_T>(rsrc, (uint32_t)(threadIdx.x + NT * c) * (8 * sizeof(KV_T)), tile_off);
   };
-  auto fetch_k = [&](int it, auto set_c) { fetch_tiles(kbase, it, kpre[decltype(set_c)::value]); };
-  auto fetch_v = [&](int it, auto set_c) { fetch_tiles(vbase, it, vpre[decltype(set_c)::value]); };
+  auto fetch_k = [&](int it, auto set_c) { fetch_tiles(k_rsrc, it, kpre[decltype(set_c)::value]); };
+  auto fetch_v = [&](int it, auto set_c) { fetch_tiles(v_rsrc, it, vpre[decltype(set_c)::value]); };
   auto stage_k = [&](int buf, auto set_c) {
     constexpr int SET = decltype(set_c)::value;
 #pragma unroll
@@ -350,15 +364,15 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     const bool act = INTERIOR || tile_active(it);
     const bool has_next = INTERIOR || it + 1 < n_it;
     if (act) rescale(t_cur);  // its branch stays out of the phases below
-    if (it + 2 + AHEAD < n_it) fetch_k(it + 2 + AHEAD, FetchSet{});
-    if (it + 1 + AHEAD < n_it) fetch_v(it + 1 + AHEAD, FetchSet{});
+    fetch_k(it + 2 + AHEAD, FetchSet{});  // past the last tile: all zeros, nothing is read
+    fetch_v(it + 1 + AHEAD, FetchSet{});
     // ---- phase A
     if (has_next) qk_tile(it + 1, s_next);  // harmless on a tile the wave cannot see
     if (act) exp_tile(s_cur, t_cur);
     // ---- phase B
     if (act) pv_tile(it);
     if (INTERIOR || tile_active(it + 1)) t_cur = mask_max(it + 1, s_next, interior_c);
-    if (it + 2 < n_it) stage_k(it & 1, StageSet{});
+    if (INTERIOR || it + 2 < n_it) stage_k(it & 1, StageSet{});  // a fill nobody reads is harmless
     if (has_next) stage_v((it + 1) & 1, StageSet{});
     __syncthreads();  // fills are visible; every wave is done with the buffers the next step refills
   };
@@ -396,6 +410,9 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     const int full_keys = min(qt * QPW * 32 + p.q_start + 1, p.cache_len);  // keys every row of the workgroup sees
     n_int = max(0, min(n_it - 1, (full_keys / BN - kt_begin) / NG - 1)) & ~1;
   }
+  // All loads issued so far have landed before the steady state begins: the waits inside the loop
+  // then only ever concern the loads of the loop itself and can leave the youngest in flight.
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   int it = 0;
   for (; it < n_int; it += 2) {
     step(it, s_a, s_b, t_cur, std::true_type{}, std::integral_constant<int, 0>{});
@@ -535,6 +552,12 @@ ARGUS_API int argus_hip_flash_attention_prefill(argus_hip_ctx *ctx, const argus_
     return 0;
   if (((uintptr_t)a->q | (uintptr_t)a->k_cache | (uintptr_t)a->v_cache | (uintptr_t)a->out) & 15)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "flash_attention_prefill: tensors must be 16-byte aligned");
+
+  // K/V tiles are addressed with 32-bit byte offsets from the head's first row
+  const size_t kv_elem = a->kv_dtype == ARGUS_HIP_F16 ? 2 : 4;
+  if (((size_t)a->kv_capacity + 1024) * a->head_dim * kv_elem > 0xffffffffull)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "flash_attention_prefill: one head's cache (%d rows) exceeds 4 GiB",
+                      a->kv_capacity);
 
   PrefillParams p{};
   p.q = a->q;
