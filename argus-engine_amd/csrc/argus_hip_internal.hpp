@@ -109,6 +109,14 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr float kNegInf = -__builtin_huge_valf();
 
+// Pins eight loaded values in registers at this point.  Without it the compiler sinks a load whose
+// value is only used under a lane condition into a branch of its own, and a run of such loads
+// becomes a chain of load-wait-load-wait round trips; pinned together, the eight loads are issued
+// back to back and waited for once.
+__device__ __forceinline__ void loaded8(float (&v)[8]) {
+  asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+}
+
 // x == hi + lo to ~2^-22 relative, both f16.  The value goes through an empty asm so the compiler
 // sees one f32 number, not the expression that made it: otherwise it may round `hi` once straight
 // from a fused product (fma_mix) for one use and twice (f32, then f16) for another, and at a

@@ -131,10 +131,13 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)h * D;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
+      float qv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qv[e] = qp[(4 * kk + j) * 8 + e];  // lanes past the group re-read its last head
+      loaded8(qv);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float qv = qp[(4 * kk + j) * 8 + e];  // unconditional: lanes past the group re-read its last head
-        const float x = (r < G) ? qv * c : 0.0f;
+        const float x = (r < G) ? qv[e] * c : 0.0f;
         _Float16 hi, lo;
         split_f16(x, hi, lo);
         qh[kk][e] = hi;

@@ -204,8 +204,12 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
     const int kk = ra + s * NREP;
     const bool ok = kk < KK && rh < G;
     const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(kvh * G + min(rh, G - 1)) * D + 32 * min(kk, KK - 1) + 8 * j;
+    float qv[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qf[s][e] = ok ? qp[e] * qscale : 0.0f;
+    for (int e = 0; e < 8; ++e) qv[e] = qp[e];  // the address is clamped
+    loaded8(qv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[s][e] = ok ? qv[e] * qscale : 0.0f;
   }
 
   const int foff = field_offset<BITS>(r);
@@ -445,10 +449,14 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       half8_t qh, ql;
+      float qv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qv[e] = qp[32 * kk + e];
+      loaded8(qv);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         _Float16 hi, lo;
-        split_f16((r < G) ? qp[32 * kk + e] * qscale : 0.0f, hi, lo);
+        split_f16((r < G) ? qv[e] * qscale : 0.0f, hi, lo);
         qh[e] = hi;
         ql[e] = lo;
       }
