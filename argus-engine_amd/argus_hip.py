@@ -14,6 +14,7 @@ LIB_PATH = os.environ.get("ARGUS_HIP_LIB") or os.path.join(_HERE, "libargus_hip.
 
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_RUNTIME, ERR_NOMEM = 0, -1, -2, -3, -4
 F32, F16 = 0, 1
+Q4_0, Q4_1, Q8_0 = 2, 3, 4  # block-quantised cache rows (attention_gen)
 HEAD_MAJOR, SEQ_MAJOR = 0, 1
 
 EXPORTED_SYMBOLS = [
@@ -251,15 +252,16 @@ class Context:
     def attention_gen(self, q, k, v, out, num_heads_kv, cache_seq_len, capacity=0,
                       layout=HEAD_MAJOR, scores=None, score_stride=0, kv_index=None, kv_start=0,
                       batch=1, kv_batch_stride=0, index_batch_stride=0, softcap=0.0, scale=0.0,
-                      check=True):
-        """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride]."""
+                      check=True, kv_dtype=None):
+        """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride].
+        kv_dtype: Q4_0 / Q4_1 / Q8_0 for uint8 tensors of blocks (default: from the tensor dtype)."""
         hq, d = q.shape[-2], q.shape[-1]
         a = AttentionGenArgs(
             stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),
             scores_out=_ptr(scores), kv_index=_ptr(kv_index), num_heads_q=hq,
             num_heads_kv=num_heads_kv, head_dim=d, cache_seq_len=cache_seq_len, capacity=capacity,
-            kv_start=kv_start, layout=layout, kv_dtype=_kv_dtype(k), batch=batch,
-            score_stride=score_stride, q_batch_stride=0, out_batch_stride=0,
+            kv_start=kv_start, layout=layout, kv_dtype=_kv_dtype(k) if kv_dtype is None else kv_dtype,
+            batch=batch, score_stride=score_stride, q_batch_stride=0, out_batch_stride=0,
             kv_batch_stride=kv_batch_stride, score_batch_stride=0,
             index_batch_stride=index_batch_stride, softcap=softcap, scale=scale)
         return self._check(lib.argus_hip_attention_gen(self.handle, C.byref(a)), check)

@@ -4,6 +4,8 @@
 
 #include "argus_hip_internal.hpp"
 
+#include <algorithm>
+
 namespace argus_decode {
 
 struct DecodeParams {
@@ -149,8 +151,36 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   }
 }
 
+// Split count of the matrix-core kernels.  The grid is sized against the number of workgroups the
+// device holds at once (`slots`): when the splits fill it in one round every workgroup starts
+// together and streams an equal share, each wave requesting its next tile while it works on the
+// current one; a partial extra round runs thinly occupied (one 32K-token sequence: 2 rounds of
+// 2-tile waves were 10 % slower than 1 round of 4-tile waves).  Cost model, in units of one tile
+// step with the device full: rounds x (tile steps per workgroup + 0.75 for set-up, merge and
+// partial write-out).  Sets p.nsplit and p.chunk (a multiple of tile_rows).
+inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slots) {
+  const int max_splits = std::min((p.len + tile_rows - 1) / tile_rows, kMaxSplits);
+  int nsplit = 1, chunk = (p.len + tile_rows - 1) / tile_rows * tile_rows;
+  float best = 3.0e38f;
+  for (int n = 1; n <= max_splits; ++n) {
+    const int c = ((p.len + n - 1) / n + tile_rows - 1) / tile_rows * tile_rows;
+    const int ns = (p.len + c - 1) / c;
+    const int64_t rounds = ((int64_t)pairs * ns + slots - 1) / slots;
+    const float cost = (float)rounds * ((float)(c / tile_rows) + 0.75f);
+    if (cost < best) {
+      best = cost;
+      nsplit = ns;
+      chunk = c;
+    }
+  }
+  p.nsplit = nsplit;
+  p.chunk = chunk;
+}
+
 // Matrix-core variant (decode_mfma.hip): F16 cache, contiguous slots, no soft-cap.
 bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype);
 int launch_decode_mfma(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hipStream_t stream);
+// Block-quantised caches (decode_blocks.hip): ARGUS_HIP_Q4_0 / Q4_1 / Q8_0, dequantised in registers.
+int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtype, int batch, hipStream_t stream);
 
 }  // namespace argus_decode

@@ -284,35 +284,14 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   constexpr int TW = (D <= 128) ? 2 : 1;
   constexpr int tile_rows = kWaves * 16 * TW;  // one tile per wave
   const int pairs = batch * p.n_heads_kv;
-  // The grid is sized against the number of workgroups the device holds at once: when the splits
-  // fill it in one round every workgroup starts together and streams an equal share, each wave
-  // requesting its next tile while it works on the current one; a partial extra round runs thinly
-  // occupied (one 32K-token sequence: 2 rounds of 2-tile waves were 10 % slower than 1 round of
-  // 4-tile waves).  Cost model, in units of one tile step with the device full: rounds x (tile
-  // steps per workgroup + 0.75 for set-up, merge and partial write-out).
   static int wgs_per_cu = 0;  // per head_dim instantiation; single inference thread
   if (wgs_per_cu == 0) {
     int n = 0;
     ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_mfma_kernel<D, TW, false>, 64 * kWaves, 0));
     wgs_per_cu = std::max(1, n);
   }
-  const int64_t slots = (int64_t)ctx->compute_units * wgs_per_cu;
-  const int max_splits = std::min((p.len + tile_rows - 1) / tile_rows, kMaxSplits);
-  int nsplit = 1, chunk = (p.len + tile_rows - 1) / tile_rows * tile_rows;
-  float best = 3.0e38f;
-  for (int n = 1; n <= max_splits; ++n) {
-    const int c = ((p.len + n - 1) / n + tile_rows - 1) / tile_rows * tile_rows;
-    const int ns = (p.len + c - 1) / c;
-    const int64_t rounds = ((int64_t)pairs * ns + slots - 1) / slots;
-    const float cost = (float)rounds * ((float)(c / tile_rows) + 0.75f);
-    if (cost < best) {
-      best = cost;
-      nsplit = ns;
-      chunk = c;
-    }
-  }
-  p.chunk = chunk;
-  p.nsplit = nsplit;
+  choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu);
+  const int nsplit = p.nsplit;
   p.direct = 0;
   const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
   const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;

@@ -137,18 +137,18 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
 
   // ---- Q as the B operand: lane (query ln, half hl) holds Q[row][16kk + 8hl .. +7] ----------
   half8_t qreg[KK];
-  {
-    const int64_t qoff = (((int64_t)b * p.seq_len + row) * p.n_heads_q + h) * D + 8 * hl;
+  auto load_q = [&]() {
+    // Rows past seq_len re-read the last row (their columns are never stored), so the loads carry
+    // no lane condition and are issued back to back.
+    const int64_t qoff = (((int64_t)b * p.seq_len + min(row, p.seq_len - 1)) * p.n_heads_q + h) * D + 8 * hl;
+    if (p.q_f16) {
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (row_ok) {
-        if (p.q_f16) x = *(const half8_t *)((const _Float16 *)p.q + qoff + 16 * kk);
-        else x = load_q_f32((const float *)p.q + qoff + 16 * kk);
-      }
-      qreg[kk] = x;
+      for (int kk = 0; kk < KK; ++kk) qreg[kk] = *(const half8_t *)((const _Float16 *)p.q + qoff + 16 * kk);
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) qreg[kk] = load_q_f32((const float *)p.q + qoff + 16 * kk);
     }
-  }
+  };
 
   float16_t o_acc[RB];
 #pragma unroll
@@ -381,22 +381,20 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   {
     typedef std::integral_constant<int, 0> Set0;
     typedef std::integral_constant<int, kDeep ? 1 : 0> Set1;
-    if (n_it > 0) {
-      fetch_k(0, Set0{});
-      fetch_v(0, Set0{});
-      if constexpr (kDeep) {  // second register set: all three first tiles in one round trip
-        if (n_it > 1) fetch_k(1, Set1{});
-      }
-      stage_k(0, Set0{});
-      stage_v(0, Set0{});
-      if (n_it > 1) {
-        if constexpr (!kDeep) fetch_k(1, Set0{});
-        stage_k(1, Set1{});
-      }
-    }
+    // Tiles past the last one read as zeros, so nothing here depends on n_it.  The query rows are
+    // requested behind the first tiles and arrive with them.
+    fetch_k(0, Set0{});
+    fetch_v(0, Set0{});
+    if constexpr (kDeep) fetch_k(1, Set1{});  // second register set: all three first tiles in one round trip
+    __builtin_amdgcn_sched_barrier(0);
+    load_q();
+    stage_k(0, Set0{});
+    stage_v(0, Set0{});
+    if constexpr (!kDeep) fetch_k(1, Set0{});
+    stage_k(1, Set1{});
     if constexpr (kDeep) {  // what step 0 stages at its end
-      if (n_it > 2) fetch_k(2, Set1{});
-      if (n_it > 1) fetch_v(1, Set1{});
+      fetch_k(2, Set1{});
+      fetch_v(1, Set1{});
     }
   }
   __syncthreads();

@@ -103,6 +103,53 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
                 gbps_wall=nbytes / wall / 1e9, gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None)
 
 
+def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1):
+    """Decode attention over a block-quantised cache (q4_0 / q8_0 rows of 18- / 34-byte blocks):
+    synthetic blocks (random codes, f16 scales sized for N(0,1)-like values); algorithmic bytes are
+    the attended block rows of K and V plus Q and out."""
+    import torch
+    import argus_hip as A
+    bb = {"q4_0": 18, "q8_0": 34}[fmt]
+    kv_dtype = {"q4_0": A.Q4_0, "q8_0": A.Q8_0}[fmt]
+    row_bytes = d // 32 * bb
+    g = torch.Generator(device="cuda").manual_seed(11)
+
+    def blocks():
+        raw = torch.randint(0, 256, (batch * hkv * L * d // 32, bb), generator=g, device="cuda", dtype=torch.uint8)
+        lo, hi = (0.1, 0.3) if fmt == "q4_0" else (0.005, 0.02)
+        scale = (torch.rand(raw.shape[0], generator=g, device="cuda") * (hi - lo) + lo).half()
+        raw[:, 0:2] = scale.view(torch.uint8).reshape(-1, 2)
+        return raw.reshape(-1)
+
+    ks = [blocks() for _ in range(rotate)]
+    vs = [blocks() for _ in range(rotate)]
+    q = torch.randn((batch, hq, d), generator=g, device="cuda", dtype=torch.float32)
+    out = torch.empty((batch, hq, d), device="cuda", dtype=torch.float32)
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] % rotate
+        state["i"] += 1
+        ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, L, batch=batch, kv_batch_stride=hkv * L * d, kv_dtype=kv_dtype)
+
+    spin_up(step)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ctx.kernel_timing_begin(steps)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    kms = ctx.kernel_timing_end(steps)
+    kernel_ms = sum(kms) / max(len(kms), 1)
+    nbytes = batch * (2 * hkv * L * row_bytes + 2 * hq * d * 4)
+    return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
+                gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None,
+                f16_equivalent_gbps_kernel=decode_bytes(hq, hkv, d, L, batch, 2, False) / (kernel_ms * 1e-3) / 1e9)
+
+
 def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res_cap=128, res_f16=False,
                rotate=8, batch=1):
     """BASELINE config 4: q_tokens = 8064 quantised + 128 residual tokens.  Blocks are synthetic
@@ -229,7 +276,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
-                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "copy_calib"],
+                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1",
+                             "q8_0", "copy_calib"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -261,6 +309,10 @@ def main():
             res = bench_prefill(ctx, args.steps, args.warmup)
         elif w == "prefill_d128":
             res = bench_prefill(ctx, args.steps, args.warmup, hq=32, hkv=8, d=128, s=8192)
+        elif w in ("q4_0", "q8_0"):
+            res = bench_decode_blocks(ctx, w, 32, 8, 128, 32768, 16, args.steps, args.warmup)
+        elif w == "q4_0_b1":
+            res = bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=8)
         elif w == "cfg5":
             res = bench_decode(ctx, 8, 4, 256, 2048, 8, args.steps, args.warmup, capacity=4096, scores=True,
                                softcap=50.0, rotate=4)
@@ -323,6 +375,10 @@ def main():
             "32 caches (sequences) per launch, 365 MB: amortised rate")
         add("cfg4_kivi_q8_x32_caches", bench_kivi(ctx, 8, es, ew, batch=32, rotate=2),
             "32 caches (sequences) per launch, 629 MB: amortised rate")
+        add("cfg3_q4_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew),
+            "--kv-format q4_0 rows attended in-kernel, 604 MB of blocks")
+        add("cfg3_q8_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q8_0", 32, 8, 128, 32768, 16, es, ew),
+            "--kv-format q8_0 rows attended in-kernel, 1141 MB of blocks")
         ex["cfg2_prefill_llama1b_S2048_f16"] = bench_prefill(ctx, es, ew)
         ex["cfg2_prefill_llama1b_S2048_f32io"] = bench_prefill(ctx, es, ew, f16_io=False)
         ex["prefill_llama8b_d128_S8192_f16"] = bench_prefill(ctx, max(5, es // 4), 2, hq=32, hkv=8, d=128, s=8192)

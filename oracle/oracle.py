@@ -402,3 +402,19 @@ def encode_via_descriptor(desc, src):
     if rc != 0:
         raise ValueError("oracle encode_via_descriptor rc=%d" % rc)
     return out
+
+
+def attention_gen_blocks(q, k_raw, v_raw, desc, n_heads_kv, cache_seq_len, capacity, head_major=True,
+                         scores=False, scores_stride=None):
+    """Backend::attention_gen over a block-quantised cache: the Q4_0 arm of the scalar CPU backend
+    (backend/cpu/common.rs:676-850: each K / V row is dequantised, then the F32 algorithm with its
+    guards runs), which is also what the `--kv-format` floor computes after decoding the whole cache
+    (kv/standard_format.rs:538-643).  Restated as exactly that composition: decode_via_descriptor of
+    the raw bytes, then the scalar attention_gen on the F32 cache."""
+    q = np.ascontiguousarray(q, np.float32)
+    d = q.shape[1]
+    rows = n_heads_kv * capacity
+    k = decode_via_descriptor(desc, k_raw, rows * d)
+    v = decode_via_descriptor(desc, v_raw, rows * d)
+    return attention_gen(q, k, v, n_heads_kv, cache_seq_len, capacity, head_major=head_major,
+                         scores=scores, scores_stride=scores_stride, impl="scalar")

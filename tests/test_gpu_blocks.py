@@ -1,0 +1,140 @@
+"""GPU parity: attention_gen over block-quantised caches (q4_0 / q4_1 / q8_0) through the C-ABI,
+against the oracle's restatement of the reference: each row dequantised exactly as
+decode_via_descriptor does, then the scalar F32 attention with its guards
+(backend/cpu/common.rs:676-850; `--kv-format` floor kv/standard_format.rs:538-643)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from blocks_util import random_blocks
+from gpu_util import ctx, dev, host, normal, check_attention_out, check_scores
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = {
+    "q4_0": (O.DESC_Q4_0, "Q4_0"),
+    "q4_1": (O.DESC_Q4_1, "Q4_1"),
+    "q8_0": (O.DESC_Q8_0, "Q8_0"),
+}
+
+
+def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True, kv_start=0, encode=False):
+    import argus_hip as A
+    desc, name = FORMATS[fmt]
+    cap = cap or L
+    rows = hkv * cap
+    if encode:  # real data through the reference's own encoder
+        k_raw = O.encode_via_descriptor(desc, normal((rows, d), seed + 1))
+        v_raw = O.encode_via_descriptor(desc, normal((rows, d), seed + 2))
+    else:
+        k_raw = random_blocks(desc, rows * d // 32, seed + 1)
+        v_raw = random_blocks(desc, rows * d // 32, seed + 2)
+    q = normal((hq, d), seed)
+    out = dev(np.zeros((hq, d), np.float32))
+    sc = dev(np.zeros((hq, L), np.float32)) if scores else None
+    ctx().attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, cap,
+                        layout=A.HEAD_MAJOR if head_major else A.SEQ_MAJOR, scores=sc,
+                        score_stride=L if scores else 0, kv_start=kv_start, kv_dtype=getattr(A, name))
+    # oracle: a window that starts at kv_start is the same cache with its first rows cut off
+    bb = O.desc_block_bytes(desc)
+    row_bytes = d // 32 * bb
+    if kv_start:
+        assert head_major
+        kr = k_raw.reshape(hkv, cap, row_bytes)[:, kv_start:].reshape(-1)
+        vr = v_raw.reshape(hkv, cap, row_bytes)[:, kv_start:].reshape(-1)
+        ref = O.attention_gen_blocks(q, kr, vr, desc, hkv, L, cap - kv_start, scores=scores)
+    else:
+        ref = O.attention_gen_blocks(q, k_raw, v_raw, desc, hkv, L, cap, head_major=head_major, scores=scores)
+    what = "%s Hq%d Hkv%d d%d L%d cap%d %s" % (fmt, hq, hkv, d, L, cap, "HM" if head_major else "SM")
+    if scores:
+        check_attention_out(host(out), ref[0], what)
+        check_scores(host(sc), ref[1], what)
+    else:
+        check_attention_out(host(out), ref, what)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0"])
+@pytest.mark.parametrize("shape", [(14, 2, 64, 1024), (32, 8, 128, 2048), (8, 4, 256, 1024)])
+def test_baseline_shapes(fmt, shape):
+    hq, hkv, d, L = shape
+    run_case(fmt, hq, hkv, d, L)
+
+
+def test_q4_0_blocks_made_by_the_reference_encoder():
+    run_case("q4_0", 32, 8, 128, 4096, encode=True)
+    run_case("q4_0", 14, 2, 64, 1024, encode=True, seed=3)
+
+
+@pytest.mark.parametrize("L", [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 500, 1000])
+def test_ragged_lengths(L):
+    run_case("q4_0", 8, 2, 128, L, cap=1024, seed=L)
+    run_case("q8_0", 4, 4, 64, L, cap=1000 if L <= 1000 else L, seed=L + 1)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0"])
+def test_seq_major_and_window_start(fmt):
+    run_case(fmt, 16, 4, 128, 777, cap=800, head_major=False, seed=11)
+    run_case(fmt, 16, 4, 128, 300, cap=800, kv_start=411, seed=12)
+
+
+def test_group_of_sixteen_and_single_head():
+    run_case("q4_0", 32, 2, 64, 512, seed=21)
+    run_case("q4_0", 1, 1, 128, 512, seed=22)
+
+
+def test_long_row_at_32k_tokens():
+    run_case("q4_0", 32, 8, 128, 32768, scores=True, seed=5)
+
+
+def test_batch_of_sequences():
+    import argus_hip as A
+    desc, _ = FORMATS["q4_0"]
+    b, hq, hkv, d, L, cap = 3, 8, 2, 128, 700, 768
+    raws = [(random_blocks(desc, hkv * cap * d // 32, 30 + i), random_blocks(desc, hkv * cap * d // 32, 40 + i)) for i in range(b)]
+    q = normal((b, hq, d), 9)
+    k = dev(np.stack([r[0] for r in raws]))
+    v = dev(np.stack([r[1] for r in raws]))
+    out = dev(np.zeros((b, hq, d), np.float32))
+    sc = dev(np.zeros((b, hq, L), np.float32))
+    ctx().attention_gen(dev(q), k, v, out, hkv, L, cap, scores=sc, score_stride=L, batch=b,
+                        kv_batch_stride=hkv * cap * d, kv_dtype=A.Q4_0)
+    for i in range(b):
+        ref = O.attention_gen_blocks(q[i], raws[i][0], raws[i][1], desc, hkv, L, cap, scores=True)
+        check_attention_out(host(out)[i], ref[0], "seq %d" % i)
+        check_scores(host(sc)[i], ref[1], "seq %d" % i)
+
+
+def test_nan_query_takes_the_uniform_fallback():
+    # A NaN query makes every logit NaN -> -inf -> uniform weights (common.rs:790-813).
+    import argus_hip as A
+    desc, _ = FORMATS["q4_0"]
+    hq, hkv, d, L = 4, 2, 64, 200
+    k_raw = random_blocks(desc, hkv * L * d // 32, 1)
+    v_raw = random_blocks(desc, hkv * L * d // 32, 2)
+    q = normal((hq, d), 3)
+    q[1, 5] = np.nan
+    out = dev(np.zeros((hq, d), np.float32))
+    sc = dev(np.zeros((hq, L), np.float32))
+    ctx().attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, L, scores=sc, score_stride=L, kv_dtype=A.Q4_0)
+    ref = O.attention_gen_blocks(q, k_raw, v_raw, desc, hkv, L, L, scores=True)
+    got, gsc = host(out), host(sc)
+    np.testing.assert_allclose(gsc[1], 1.0 / L, rtol=1e-6)
+    np.testing.assert_allclose(got[1], ref[0][1], atol=2e-5)
+    for h in (0, 2, 3):
+        check_attention_out(got[h], ref[0][h], "head %d" % h)
+
+
+def test_unsupported_combinations_are_refused():
+    import argus_hip as A
+    desc, _ = FORMATS["q4_0"]
+    hq, hkv, d, L = 4, 2, 64, 64
+    k = dev(random_blocks(desc, hkv * L * d // 32, 1))
+    q = dev(normal((hq, d), 3))
+    out = dev(np.zeros((hq, d), np.float32))
+    c = ctx()
+    assert c.attention_gen(q, k, k, out, hkv, L, L, softcap=30.0, kv_dtype=A.Q4_0, check=False) == A.ERR_UNSUPPORTED
+    idx = dev(np.arange(L, dtype=np.int32))
+    assert c.attention_gen(q, k, k, out, hkv, L, L, kv_index=idx, kv_dtype=A.Q4_0, check=False) == A.ERR_UNSUPPORTED
+    q17 = dev(normal((34, d), 3))
+    out17 = dev(np.zeros((34, d), np.float32))
+    assert c.attention_gen(q17, k, k, out17, 2, L, L, kv_dtype=A.Q4_0, check=False) == A.ERR_UNSUPPORTED

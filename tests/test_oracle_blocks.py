@@ -1,0 +1,53 @@
+"""The oracle's attention over block-quantised caches (the Q4_0 arm of the scalar CPU backend,
+backend/cpu/common.rs:676-850) is pinned here by an independent route: the blocks are unpacked with
+a few lines of numpy written from the format definition (quant.rs BlockQ4_0 / BlockQ4_1 / BlockQ8_0:
+x = d*(n-8), d*n+m, d*c; element i in the low nibble of byte i, element 16+i in the high nibble)
+and attended with the float64 textbook softmax attention."""
+import numpy as np
+import pytest
+
+import oracle as O
+import textbook as T
+from blocks_util import random_blocks as blocks
+
+
+def unpack(desc, raw, n_elems):
+    bb = O.desc_block_bytes(desc)
+    blk = np.asarray(raw, np.uint8).reshape(-1, bb)
+    d = blk[:, 0:2].copy().view(np.float16).astype(np.float64)
+    if desc == O.DESC_Q8_0:
+        x = d * blk[:, 2:].view(np.int8).astype(np.float64)
+    else:
+        hdr = 4 if desc == O.DESC_Q4_1 else 2
+        codes = blk[:, hdr:]
+        n = np.concatenate([codes & 15, codes >> 4], axis=1).astype(np.float64)
+        if desc == O.DESC_Q4_1:
+            x = d * n + blk[:, 2:4].copy().view(np.float16).astype(np.float64)
+        else:
+            x = d * (n - 8.0)
+    return x.reshape(-1)[:n_elems]
+
+
+@pytest.mark.parametrize("desc", [O.DESC_Q4_0, O.DESC_Q4_1, O.DESC_Q8_0])
+@pytest.mark.parametrize("head_major", [True, False])
+def test_against_numpy_unpack_and_textbook_attention(desc, head_major):
+    hq, hkv, d, L, cap = 8, 2, 64, 300, 320
+    n = hkv * cap * d
+    k_raw, v_raw = blocks(desc, n // 32, 1), blocks(desc, n // 32, 2)
+    q = np.random.default_rng(3).standard_normal((hq, d)).astype(np.float32)
+    out, sc = O.attention_gen_blocks(q, k_raw, v_raw, desc, hkv, L, cap, head_major=head_major, scores=True)
+    shape = (hkv, cap, d) if head_major else (cap, hkv, d)
+    k = unpack(desc, k_raw, n).reshape(shape)
+    v = unpack(desc, v_raw, n).reshape(shape)
+    if not head_major:
+        k, v = k.transpose(1, 0, 2), v.transpose(1, 0, 2)
+    ref_out, ref_p = T.decode_attention(q, k, v, hkv, L)
+    assert np.abs(out - ref_out).max() < 1e-5
+    assert np.abs(sc - ref_p).max() < 1e-6
+    np.testing.assert_allclose(sc.sum(-1), 1.0, rtol=1e-5)
+
+
+def test_q4_0_unpack_matches_the_descriptor_decode_bit_for_bit():
+    raw = blocks(O.DESC_Q4_0, 64, 5)
+    got = O.decode_via_descriptor(O.DESC_Q4_0, raw, 64 * 32)
+    assert np.array_equal(got, unpack(O.DESC_Q4_0, raw, 64 * 32).astype(np.float32))
