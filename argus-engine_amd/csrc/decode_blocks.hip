@@ -44,11 +44,26 @@ struct BlockFmt {
   static constexpr int CW = (FMT == kFmtQ8_0) ? 2 : 1;              // code dwords per lane piece
 };
 
-// Element (within its block) held by slot s of the piece a lane with code index x loads.
+// Element (within its block) held by slot s of the piece a lane with code index x loads
+// (q4: the slots follow the order in which the shifts below bring the nibbles out).
 template <int FMT>
 __host__ __device__ constexpr int slot_elem(int x, int s) {
-  return (FMT == kFmtQ8_0) ? 8 * x + s : (s < 4 ? 4 * x + s : 16 + 4 * x + (s - 4));
+  if (FMT == kFmtQ8_0) return 8 * x + s;
+  const int within = (s & 3) == 1 ? 2 : ((s & 3) == 2 ? 1 : (s & 3));  // 0, 2, 1, 3
+  return (s < 4 ? 0 : 16) + 4 * x + within;
 }
+
+// How the operands carry a code.  q4: the nibble n sits in mantissa bits 4..7 (where the high
+// nibble of a byte already is) under the exponent of 64, i.e. the half is exactly 64 + n, with no
+// arithmetic at all; the bias (and q4_0's zero point 8) is taken out where it is cheap: from the
+// block dot product as (bias + zero) * sum(Q), folded into the accumulator the MFMA starts from,
+// and from the values as one fma whose addend -64 d is exact.  q8: the int8 c is made exact by a
+// packed subtract (bias 0).
+template <int FMT>
+struct Codec {
+  static constexpr float kBias = (FMT == kFmtQ8_0) ? 0.0f : 64.0f;  // operand = kBias + code
+  static constexpr float kZero = (FMT == kFmtQ4_0) ? 8.0f : 0.0f;   // value = d * (code - kZero) (+ m)
+};
 
 // What one lane holds of one block before it is dequantised.
 template <int FMT>
@@ -70,6 +85,65 @@ __device__ __forceinline__ RawPiece<FMT> load_piece(const uint8_t *base, uint32_
   return p;
 }
 
+// A whole block as one lane loads it when head_dim is 128: the K rows of a tile are read one block
+// per lane (lane group j takes block j of row r: 16 or 32 contiguous code bytes), which touches
+// each cache line of the tile once per request instead of once per 4-byte piece, and the lane
+// groups then trade dwords (block_to_pieces).
+template <int FMT>
+struct RawBlock {
+  uint32_t code[4 * BlockFmt<FMT>::CW];
+  uint32_t hdr;
+};
+typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+
+template <int FMT>
+__device__ __forceinline__ RawBlock<FMT> load_block(const uint8_t *base, uint32_t blk) {
+  using F = BlockFmt<FMT>;
+  RawBlock<FMT> b;
+  if constexpr (FMT == kFmtQ4_1) b.hdr = *(const uint32_t *)(base + blk);
+  else b.hdr = *(const uint16_t *)(base + blk);
+#pragma unroll
+  for (int w = 0; w < F::CW; ++w) {
+    const u32x4_a2 c = *(const u32x4_a2 *)(base + (blk + (uint32_t)F::HDR + 16u * (uint32_t)w));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) b.code[4 * w + i] = c[i];
+  }
+  return b;
+}
+
+// 4 x 4 transpose across the four lane groups (lanes 16 apart): lane group j ends up with what lane
+// groups 0..3 held in v[j].  v_permlane16_swap trades v[0], v[2] of the odd groups with v[1], v[3]
+// of the even ones, v_permlane32_swap does the same between the halves of the wave.
+__device__ __forceinline__ void transpose_lane_groups(uint32_t (&v)[4]) {
+  auto a = __builtin_amdgcn_permlane16_swap(v[0], v[1], false, false);
+  auto b = __builtin_amdgcn_permlane16_swap(v[2], v[3], false, false);
+  auto c = __builtin_amdgcn_permlane32_swap(a[0], b[0], false, false);
+  auto d = __builtin_amdgcn_permlane32_swap(a[1], b[1], false, false);
+  v[0] = c[0]; v[2] = c[1]; v[1] = d[0]; v[3] = d[1];
+}
+
+// Lane group j holds block j of its row; afterwards piece[kk] is the lane's piece (code index j)
+// of block kk, with that block's header.
+template <int FMT>
+__device__ __forceinline__ void block_to_pieces(const RawBlock<FMT> &b, RawPiece<FMT> (&piece)[4]) {
+  constexpr int CW = BlockFmt<FMT>::CW;
+#pragma unroll
+  for (int w = 0; w < CW; ++w) {
+    // piece dword w of code index x is block dword CW * x + w
+    uint32_t v[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] = b.code[CW * x + w];
+    transpose_lane_groups(v);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) piece[kk].code[w] = v[kk];
+  }
+  // headers: all-gather over the lane groups with the same two trades
+  auto p = __builtin_amdgcn_permlane16_swap(b.hdr, b.hdr, false, false);       // (even group's, odd group's)
+  auto lo = __builtin_amdgcn_permlane32_swap(p[0], p[0], false, false);         // (group 0's, group 2's)
+  auto hi = __builtin_amdgcn_permlane32_swap(p[1], p[1], false, false);         // (group 1's, group 3's)
+  piece[0].hdr = lo[0]; piece[2].hdr = lo[1]; piece[1].hdr = hi[0]; piece[3].hdr = hi[1];
+}
+
 // Bytes b0 b1 b2 b3 of `bytes` (each < 256) -> halves {1024 + b0, 1024 + b1} and {1024 + b2, 1024 + b3}:
 // 0x64 in the high byte of a half is the exponent of 1024, whose mantissa unit is 1.
 __device__ __forceinline__ half2_t bytes_lo(uint32_t bytes) {
@@ -78,8 +152,16 @@ __device__ __forceinline__ half2_t bytes_lo(uint32_t bytes) {
 __device__ __forceinline__ half2_t bytes_hi(uint32_t bytes) {
   return __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, bytes, 0x04030402u));
 }
+// Two nibbles of a code word, 16 bits apart and already at bits 4..7 / 20..23 -> {64 + n, 64 + n'}.
+// One v_and_or_b32 (spelled out: this target's three-operand form takes no literal, and the
+// compiler otherwise emits the AND and the OR separately).
+__device__ __forceinline__ half2_t nibbles(uint32_t word, uint32_t mask, uint32_t exponent) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(word), "v"(mask), "v"(exponent));
+  return __builtin_bit_cast(half2_t, r);
+}
 
-// The 8 codes of a piece as exact f16 integers: n - 8 (q4_0), n (q4_1), c (q8_0).
+// The 8 codes of a piece as exact f16 numbers Codec::kBias + code.
 template <int FMT>
 __device__ __forceinline__ void piece_codes(const RawPiece<FMT> &p, half2_t (&v)[4]) {
   if constexpr (FMT == kFmtQ8_0) {
@@ -92,13 +174,13 @@ __device__ __forceinline__ void piece_codes(const RawPiece<FMT> &p, half2_t (&v)
       v[2 * w + 1] = bytes_hi(u) + off;
     }
   } else {
-    const uint32_t lo = p.code[0] & 0x0f0f0f0fu, hi = (p.code[0] >> 4) & 0x0f0f0f0fu;
-    const _Float16 o = (FMT == kFmtQ4_0) ? (_Float16)-1032.0f : (_Float16)-1024.0f;  // 1024 (and the zero point 8)
-    const half2_t off = {o, o};
-    v[0] = bytes_lo(lo) + off;
-    v[1] = bytes_hi(lo) + off;
-    v[2] = bytes_lo(hi) + off;
-    v[3] = bytes_hi(hi) + off;
+    const uint32_t w = p.code[0];
+    uint32_t mask = 0x00f000f0u, exponent = 0x54005400u;
+    asm("" : "+v"(mask), "+v"(exponent));  // keep both in vector registers
+    v[0] = nibbles(w << 4, mask, exponent);  // low nibbles of bytes 0, 2
+    v[1] = nibbles(w >> 4, mask, exponent);  // low nibbles of bytes 1, 3
+    v[2] = nibbles(w, mask, exponent);       // high nibbles of bytes 0, 2
+    v[3] = nibbles(w >> 8, mask, exponent);  // high nibbles of bytes 1, 3
   }
 }
 
@@ -109,25 +191,22 @@ __device__ __forceinline__ half8_t code_operand(const RawPiece<FMT> &p) {
   return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
 }
 
-// The 8 values of a piece, rounded once to f16: d * code (+ m).
+// The 8 values of a piece without zero point and minimum, d * code, rounded once to f16.
 template <int FMT>
-__device__ __forceinline__ half8_t dequant_piece(const RawPiece<FMT> &p) {
+__device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p) {
   const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u));  // {d, d}
   half2_t v[4];
   piece_codes<FMT>(p, v);
-  if constexpr (FMT == kFmtQ4_1) {
-    const half2_t mm = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x03020302u));  // {m, m}
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = __builtin_elementwise_fma(v[i], dd, mm);
-  } else {
+  if constexpr (FMT == kFmtQ8_0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = v[i] * dd;
+  } else {
+    const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_elementwise_fma(v[i], dd, nb);
   }
   return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
 }
-
-__device__ __forceinline__ float hdr_scale(uint32_t hdr) { return (float)__builtin_bit_cast(half2_t, hdr)[0]; }
-__device__ __forceinline__ float hdr_min(uint32_t hdr) { return (float)__builtin_bit_cast(half2_t, hdr)[1]; }
 
 // One element of a block as f32 (rare paths only).
 template <int FMT>
@@ -177,6 +256,7 @@ template <int FMT, int D, int TW>
 __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
+  using CD = Codec<FMT>;
   constexpr int KK = SH::KK, VSEG = SH::VSEG, NACC = SH::NACC;
   constexpr int TILE = 16 * TW;  // tokens per wave iteration
   constexpr float kLn2 = 0.6931471805599453f;
@@ -200,8 +280,15 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg) vblk[sg] = (4 * sg + r / 4) % KK;
 
-  RawPiece<FMT> kraw[TW][KK];
-  RawPiece<FMT> vraw[TW][VSEG][4];
+  constexpr bool kBlockLoads = KK == 4;  // head_dim 128: one block per lane, traded between lane groups
+  RawPiece<FMT> kraw[TW][kBlockLoads ? 1 : KK];
+  RawBlock<FMT> kblk[TW];
+  // ... and for the 4-bit formats the V rows too: lane (j, r) takes block r/4 of token 4j + r%4, and
+  // the four lanes of a quad trade dwords through a wave-private strip of LDS (16 bytes per lane,
+  // plus 16 bytes after every 16 lanes so that the four lane groups read different banks).
+  constexpr bool kStageV = kBlockLoads && FMT != kFmtQ8_0;
+  RawPiece<FMT> vraw[TW][VSEG][kStageV ? 1 : 4];
+  RawBlock<FMT> vblk_raw[TW];
   // Rows past the chunk re-read its last row (they are masked below), so every request is
   // unconditional and a tile may be asked for before it is known to exist.
   const int last = t_end - 1;
@@ -209,19 +296,29 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + r, last), row_bytes);
+      if constexpr (kBlockLoads) {
+        kblk[tw] = load_block<FMT>(kb, off + (uint32_t)(j * F::BB));
+      } else {
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) kraw[tw][kk] = load_piece<FMT>(kb, off + (uint32_t)(kk * F::BB), (uint32_t)j);
+        for (int kk = 0; kk < KK; ++kk) kraw[tw][kk] = load_piece<FMT>(kb, off + (uint32_t)(kk * F::BB), (uint32_t)j);
+      }
     }
   };
   auto load_v = [&](int base) {
 #pragma unroll
-    for (int tw = 0; tw < TW; ++tw)
+    for (int tw = 0; tw < TW; ++tw) {
+      if constexpr (kStageV) {
+        const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + (r & 3), last), row_bytes);
+        vblk_raw[tw] = load_block<FMT>(vb, off + (uint32_t)((r >> 2) * F::BB));
+      } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + e, last), row_bytes);
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + e, last), row_bytes);
 #pragma unroll
-        for (int sg = 0; sg < VSEG; ++sg) vraw[tw][sg][e] = load_piece<FMT>(vb, off + (uint32_t)(vblk[sg] * F::BB), (uint32_t)(r & 3));
+          for (int sg = 0; sg < VSEG; ++sg) vraw[tw][sg][e] = load_piece<FMT>(vb, off + (uint32_t)(vblk[sg] * F::BB), (uint32_t)(r & 3));
+        }
       }
+    }
   };
   const int base0 = t_begin + __builtin_amdgcn_readfirstlane(wave) * TILE;
   load_k(base0);
@@ -230,7 +327,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 
   // ---- Q operand: lane (j, h = r), block kk: the elements slot_elem(j, 0..7), log2 domain, hi + lo
   half8_t qh[KK], ql[KK];
-  float qsum[KK];  // q4_1 only: sum of the scaled query over block kk, for the m term
+  float qsum[KK];  // sum of the scaled query over block kk: bias / zero-point and minimum terms
   {
     const float c = p.scale * 1.4426950408889634f;
     const int h = kvh * G + min(r, G - 1);
@@ -266,6 +363,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
   float4_t o_acc[NACC];
 #pragma unroll
   for (int a = 0; a < NACC; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  // sum over tokens of p * d (q4_0: times -8 it is the zero-point term of the lane's channels) or
+  // of p * m (q4_1: the minimum term), per V piece; one more MFMA column each
+  constexpr bool kHdrTerm = FMT != kFmtQ8_0;
+  float4_t h_acc[VSEG];
+#pragma unroll
+  for (int sg = 0; sg < VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
@@ -274,39 +377,62 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       s[tw] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      RawPiece<FMT> kpc[KK];
+      if constexpr (kBlockLoads) {
+        block_to_pieces<FMT>(kblk[tw], kpc);
+      } else {
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        const half8_t ka = code_operand<FMT>(kraw[tw][kk]);
-        float4_t dot = {0.0f, 0.0f, 0.0f, 0.0f};
-        dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qh[kk], dot, 0, 0, 0);
-        dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, ql[kk], dot, 0, 0, 0);
-        const int d_own = __builtin_bit_cast(int, hdr_scale(kraw[tw][kk].hdr));
+        for (int kk = 0; kk < KK; ++kk) kpc[kk] = kraw[tw][kk];
+      }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float d_tok = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(hdr_src[i], d_own));
-          s[tw][i] = fmaf(d_tok, dot[i], s[tw][i]);
+      for (int kp = 0; kp < KK / 2; ++kp) {
+        float4_t dot[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int kk = 2 * kp + u;
+          const half8_t ka = code_operand<FMT>(kpc[kk]);
+          // sum of (code - zero) * q = sum of operand * q - (bias + zero) * sum of q
+          const float c0 = -(CD::kBias + CD::kZero) * qsum[kk];
+          dot[u] = float4_t{c0, c0, c0, c0};
+          dot[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qh[kk], dot[u], 0, 0, 0);
+          dot[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, ql[kk], dot[u], 0, 0, 0);
         }
         if constexpr (FMT == kFmtQ4_1) {
-          const int m_own = __builtin_bit_cast(int, hdr_min(kraw[tw][kk].hdr));
+          // the header word already holds (d, m): one exchange per token and block
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const half2_t dm = __builtin_bit_cast(half2_t, __builtin_amdgcn_ds_bpermute(hdr_src[i], (int)kpc[2 * kp + u].hdr));
+              s[tw][i] = fmaf((float)dm[0], dot[u][i], fmaf((float)dm[1], qsum[2 * kp + u], s[tw][i]));
+            }
+        } else {
+          // scales of two blocks travel together
+          const int d_pair = (int)__builtin_amdgcn_perm(kpc[2 * kp + 1].hdr, kpc[2 * kp].hdr, 0x05040100u);
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float m_tok = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(hdr_src[i], m_own));
-            s[tw][i] = fmaf(m_tok, qsum[kk], s[tw][i]);
+            const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_ds_bpermute(hdr_src[i], d_pair));
+            s[tw][i] = fmaf((float)dd[0], dot[0][i], fmaf((float)dd[1], dot[1][i], s[tw][i]));
           }
         }
       }
     }
     load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
     const bool full = base + TILE <= t_end;
+    if (!full) {  // uniform: only the chunk's last tile has rows to mask
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (base + 16 * tw + 4 * j + i >= t_end) s[tw][i] = kNegInf;
+    }
     float mt = kNegInf;
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float sv = fmaxf(s[tw][i], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
-        if (!full && base + 16 * tw + 4 * j + i >= t_end) sv = kNegInf;
-        s[tw][i] = sv;
-        mt = fmaxf(mt, sv);
+        s[tw][i] = fmaxf(s[tw][i], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
+        mt = fmaxf(mt, s[tw][i]);
       }
     if (p.scores && r < G) {
       // Logits in natural units; the combine pass rewrites them as probabilities.
@@ -350,6 +476,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
       for (int a = 0; a < NACC; ++a)
 #pragma unroll
         for (int i = 0; i < 4; ++i) o_acc[a][i] *= al[i];
+      if constexpr (kHdrTerm) {
+#pragma unroll
+        for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) h_acc[sg][i] *= al[i];
+      }
     }
 
     // ---- O += P . V -----------------------------------------------------------------------------
@@ -357,9 +489,38 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
       for (int sg = 0; sg < VSEG; ++sg) {
+        RawPiece<FMT> vpc[4];  // the lane's piece of tokens 4j .. 4j+3
+        if constexpr (kStageV) {
+          __shared__ uint32_t v_strip[kWaves][TW][64 * 4 + 4 * 4];
+          uint32_t *strip = v_strip[wave][tw];
+          typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+          *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{vblk_raw[tw].code[0], vblk_raw[tw].code[1], vblk_raw[tw].code[2], vblk_raw[tw].code[3]};
+          // token 4j + e was loaded by lane 16j + 4(r/4) + e; this lane wants dword r%4 of it
+          const uint32_t *src = strip + 68 * j + 16 * (r >> 2) + (r & 3);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) vpc[e].code[0] = src[4 * e];
+          // header of token 4j + e: lane e of the quad has it
+          const int own_hdr = (int)vblk_raw[tw].hdr;
+          vpc[0].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0x00, 0xf, 0xf, false);
+          vpc[1].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0x55, 0xf, 0xf, false);
+          vpc[2].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0xaa, 0xf, 0xf, false);
+          vpc[3].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0xff, 0xf, 0xf, false);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) vpc[e] = vraw[tw][sg][e];
+        }
         half8_t vrow[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) vrow[e] = dequant_piece<FMT>(vraw[tw][sg][e]);
+        for (int e = 0; e < 4; ++e) vrow[e] = scaled_codes<FMT>(vpc[e]);
+        if constexpr (kHdrTerm) {
+          // d (q4_0: low halves of the headers) or m (q4_1: high halves) of the lane's four tokens
+          constexpr uint32_t sel = (FMT == kFmtQ4_1) ? 0x07060302u : 0x05040100u;
+          const uint32_t h01 = __builtin_amdgcn_perm(vpc[1].hdr, vpc[0].hdr, sel);
+          const uint32_t h23 = __builtin_amdgcn_perm(vpc[3].hdr, vpc[2].hdr, sel);
+          typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+          const half4_t hv = __builtin_bit_cast(half4_t, u32x2_t{h01, h23});
+          h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+        }
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
           const half4_t bv = {vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
@@ -367,6 +528,16 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         }
       }
     load_v(base + kWaves * TILE);
+  }
+
+  if constexpr (kHdrTerm) {
+    constexpr float kTerm = (FMT == kFmtQ4_0) ? -CD::kZero : 1.0f;
+#pragma unroll
+    for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o_acc[sg * 8 + c][i] = fmaf(kTerm, h_acc[sg][i], o_acc[sg * 8 + c][i]);
   }
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------

@@ -42,7 +42,7 @@ using Status = Result<Unit>;
 inline Status OkStatus() { return Status::Ok(Unit{}); }
 
 // DType subset of engine/src/buffer.rs:25-47.
-enum class DType { F32 = ARGUS_HIP_F32, F16 = ARGUS_HIP_F16, Q4_0 = 100 };
+enum class DType { F32 = ARGUS_HIP_F32, F16 = ARGUS_HIP_F16, Q4_0 = ARGUS_HIP_Q4_0 };
 
 // A tensor is a shape over a lent buffer (engine/src/tensor.rs:8-58); `device` tells whether the
 // pointer is a device pointer of this backend (a `Buffer` of another backend has none).
@@ -318,9 +318,10 @@ inline Status HipBackend::attention_gen(const Tensor &q, const Tensor &k_cache, 
                                         size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
                                         float *scores_out, size_t scores_len) {
   // The reference falls back to its CPU companion for non-device buffers and Q4_0 KV
-  // (cuda_pc.rs:1716-1729); this mirror has no CPU companion, so it reports the case.
-  if (!q.device || !k_cache.device || !v_cache.device || !out.device || k_cache.dtype == DType::Q4_0)
-    return Status::Err("attention_gen: not a device F32/F16 call; route to the CPU companion");
+  // (cuda_pc.rs:1716-1729); this mirror has no CPU companion, so it reports the former.  Q4_0
+  // caches are attended on the device (BlockQ4_0 rows, common.rs:676-850).
+  if (!q.device || !k_cache.device || !v_cache.device || !out.device)
+    return Status::Err("attention_gen: not a device call; route to the CPU companion");
   const std::vector<size_t> &kd = k_cache.dims;
   // Layout rule of x86.rs:195-198.
   const bool head_major = kd.size() >= 3 && kd[1] == num_heads_kv && kd[1] != kd[2];

@@ -75,5 +75,31 @@ def main():
          q4_0_decoded=O.decode_via_descriptor(O.DESC_Q4_0, O.encode_via_descriptor(O.DESC_Q4_0, x), x.size))
 
 
+def blocks():
+    """attention_gen over q4_0 / q8_0 block rows (own generator, so the fixtures above keep their bytes)."""
+    rng = np.random.default_rng(20240922)
+    hq, hkv, d, L, cap = 8, 2, 64, 80, 96
+    q = rng.standard_normal((hq, d)).astype(np.float32)
+    arrays = {"q": q, "dims": np.array([hq, hkv, d, L, cap])}
+    # q4_0: N(0,1) rows through the reference-shaped encoder
+    kq = O.encode_via_descriptor(O.DESC_Q4_0, rng.standard_normal(hkv * cap * d).astype(np.float32))
+    vq = O.encode_via_descriptor(O.DESC_Q4_0, rng.standard_normal(hkv * cap * d).astype(np.float32))
+    out, sc = O.attention_gen_blocks(q, kq, vq, O.DESC_Q4_0, hkv, L, cap, scores=True)
+    arrays.update(k_q4_0=kq, v_q4_0=vq, out_q4_0=out, scores_q4_0=sc)
+    # q8_0: random codes, scales sized for unit-variance values (the reference has no q8_0 encoder)
+    def q8(n_blocks):
+        raw = rng.integers(0, 256, size=(n_blocks, 34), dtype=np.uint8)
+        raw[:, 0:2] = rng.uniform(0.005, 0.02, n_blocks).astype(np.float16).view(np.uint8).reshape(n_blocks, 2)
+        return raw.reshape(-1)
+    k8, v8 = q8(hkv * cap * d // 32), q8(hkv * cap * d // 32)
+    out, sc = O.attention_gen_blocks(q, k8, v8, O.DESC_Q8_0, hkv, L, cap, scores=True)
+    arrays.update(k_q8_0=k8, v_q8_0=v8, out_q8_0=out, scores_q8_0=sc)
+    save("blocks", **arrays)
+
+
 if __name__ == "__main__":
-    main()
+    if len(sys.argv) > 1 and sys.argv[1] == "blocks":
+        blocks()  # python tests/golden/make_golden.py blocks: only this fixture
+    else:
+        main()
+        blocks()

@@ -24,6 +24,10 @@ int oracle_prefill_attention(const float *q, const void *k, const void *v, float
                              int cache_len, int d, int capacity, int batch, int kv_dtype, int window, int n_threads);
 int oracle_score_fused_reduce(const float *scores, float *imp, float *himp, float decay_factor, int n_layers, int hq,
                               int hkv, int len, int64_t stride, int max_seq);
+int oracle_decode_via_descriptor(int block_elems, int bits, int scale_layout, int packing, const uint8_t *src, float *dst,
+                                 int64_t n_elems);
+int oracle_encode_via_descriptor(int block_elems, int bits, int scale_layout, int packing, const float *src, uint8_t *dst,
+                                 int64_t n_elems);
 void oracle_kv_scatter(const float *k_src, const float *v_src, void *k_dst, void *v_dst, int kv_heads, int head_dim,
                        int capacity, int write_pos_start, int seq_len, int dst_f16);
 }
@@ -135,7 +139,29 @@ static void test_attention_gen(HipBackend &be) {
     host_q.device = false;
     CHECK(!be.attention_gen(host_q, tk, tv, tout, hq, hkv, d, len, nullptr, 0).ok(), "host tensor is refused");
   }
-  printf("[attention_gen] unit shape f32/f16 + host score slice ok\n");
+  {
+    // Q4_0 cache (BlockQ4_0 rows, common.rs:676-850): blocks made by the q4_0 encoder, reference =
+    // the same blocks decoded to F32 and attended by the scalar oracle.
+    std::vector<uint8_t> kq(kf.size() / 32 * 18), vq(kq.size());
+    CHECK(oracle_encode_via_descriptor(32, 4, 1, 1, kf.data(), kq.data(), kf.size()) == 0, "encode K");
+    CHECK(oracle_encode_via_descriptor(32, 4, 1, 1, vf.data(), vq.data(), vf.size()) == 0, "encode V");
+    std::vector<float> kd(kf.size()), vd(vf.size());
+    oracle_decode_via_descriptor(32, 4, 1, 1, kq.data(), kd.data(), kd.size());
+    oracle_decode_via_descriptor(32, 4, 1, 1, vq.data(), vd.data(), vd.size());
+    DevBuf dq(&be, q.size() * 4, q.data()), dk(&be, kq.size(), kq.data()), dv(&be, vq.size(), vq.data()), dout(&be, q.size() * 4);
+    Tensor tq{dq.p, DType::F32, {(size_t)hq, (size_t)d}}, tout{dout.p, DType::F32, {(size_t)hq, (size_t)d}};
+    Tensor tk{dk.p, DType::Q4_0, {1, (size_t)hkv, (size_t)cap, (size_t)d}}, tv = tk;
+    tv.ptr = dv.p;
+    std::vector<float> sc(hq * len), ref(hq * d), ref_sc(hq * len), got(hq * d);
+    CHECK(be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, sc.data(), sc.size()).ok(), "attention_gen q4_0: %s", be.last_error().c_str());
+    be.read_buffer(got.data(), dout.p, got.size() * 4);
+    oracle_attention_gen_scalar(q.data(), kd.data(), vd.data(), ref.data(), hq, hkv, d, len, cap, 1, 0, ref_sc.data(), len, 0.0f, nullptr);
+    CHECK(max_abs_diff(got, ref) < 1e-3f, "attention_gen q4_0 out diff %g", max_abs_diff(got, ref));
+    float worst = 0;
+    for (size_t i = 0; i < sc.size(); ++i) worst = fmaxf(worst, fabsf(sc[i] - ref_sc[i]) / ref_sc[i]);
+    CHECK(worst < 1e-4f, "q4_0 scores rel diff %g", worst);
+  }
+  printf("[attention_gen] unit shape f32/f16/q4_0 + host score slice ok\n");
 }
 
 static void test_accumulator_binding(HipBackend &be) {
