@@ -265,7 +265,7 @@ def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
 # HBM bytes per launch of the primary workload's kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs
 # scaled by what the same counters read for a plain 1 GiB copy (x2.000 and x1.000); the runs and
 # their commands are summarised in profiles/decode_mfma_cfg3_L32768_b16_hbm_traffic.md.
-DECODE_TRAFFIC_BYTES = 2_191_763_046
+DECODE_TRAFFIC_BYTES = 2_153_496_471
 
 
 def main():
