@@ -12,13 +12,16 @@
 //        O^T = V^T . P^T   (A = V^T from LDS, B = P^T taken straight from the S^T accumulators)
 //    so a lane owns one query column: the softmax runs over in-lane registers plus one
 //    cross-half shuffle, the O rescale is a per-lane scalar, and P never goes through LDS.
-//  * One wave = 32 query rows of one Q head.  A workgroup's 4 waves are HPW heads of one GQA group
-//    times 4/HPW consecutive 32-row blocks; they share each K/V tile staged once in LDS (K row
-//    major, V transposed while being written), so GQA multiplies neither HBM nor LDS-fill traffic.
-//  * The next K/V tile is fetched into registers while the current one is being consumed.
+//  * One wave = 32 query rows of one Q head.  Four waves -- HPW heads of one GQA group times 4/HPW
+//    consecutive 32-row blocks -- share each K/V tile, staged once in LDS (both row major; the V^T
+//    operand comes out of a transposing LDS read), so GQA multiplies neither HBM nor LDS-fill
+//    traffic.  A workgroup is one such quartet, or two of them (KV groups) on alternate key tiles
+//    of the same query block when the grid alone would leave one wave per SIMD.
+//  * Tiles are fetched into registers ahead of the step that stages them, through bounds-checked
+//    buffer loads; the logits MFMAs of tile t+1 overlap the exponentials of tile t.
 //  * blockIdx is laid out so that consecutive workgroups hit different KV heads (one XCD / L2 per
-//    KV head when there are 8 of them) and long (late) query tiles are issued before short ones,
-//    pairing a long and a short tile on each compute unit.
+//    KV head when there are 8 of them); a workgroup takes query tiles n-1-j then j, so all carry
+//    the same number of key tiles.
 #include "argus_hip_internal.hpp"
 
 #include <cstdlib>
@@ -500,13 +503,19 @@ int launch_ng(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream, size_t l
 
 template <int D, int HPW, typename KV_T>
 int launch(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
-  // KV groups split the serial chain of key tiles of a query block over 4*NG waves.  Two groups
-  // (8 waves, <= 256 VGPRs each) measured best; four groups need a 128-VGPR cap that spills.
+  // Two waves per SIMD are needed to overlap anything.  When the grid alone provides them -- two
+  // 4-wave workgroups per compute unit -- the workgroups run independently and measure 4-8 % faster
+  // (S >= 4096 at Hq32/Hkv8).  Smaller grids get them from two KV groups inside an 8-wave workgroup:
+  // the groups take alternate key tiles of the same query block and merge at the end (BASELINE
+  // config 2: 32.3 us against 33.9 us).  Four groups would need a 128-VGPR cap that spills.
   const size_t tile_bytes = (size_t)PrefillTile<D>::HALFS * sizeof(_Float16);
   const size_t lds_limit = ctx->props.sharedMemPerBlock;
-  static const bool one_group = getenv("ARGUS_PREFILL_NG1") != nullptr;
   if constexpr (D <= 128) {
-    if (!one_group && 2 * 2 * tile_bytes <= lds_limit) return launch_ng<D, HPW, 2, KV_T>(ctx, p, stream, 2 * 2 * tile_bytes);
+    constexpr int QPW = 4 / HPW;
+    const int64_t n_qtiles = (p.seq_len + 32 * QPW - 1) / (32 * QPW);
+    const int64_t wgs = (int64_t)p.batch * p.n_heads_kv * (p.group / HPW) * ((n_qtiles + 1) / 2);
+    const bool grid_fills = wgs >= 2 * (int64_t)ctx->compute_units;
+    if (!grid_fills && 2 * 2 * tile_bytes <= lds_limit) return launch_ng<D, HPW, 2, KV_T>(ctx, p, stream, 2 * 2 * tile_bytes);
   }
   if (2 * tile_bytes > lds_limit)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: %zu bytes of LDS needed, %zu available", 2 * tile_bytes, lds_limit);

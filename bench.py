@@ -248,7 +248,7 @@ def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
     oracle.attention_gen(q, k, v, hkv, L, L, impl="avx2", n_threads=cores)  # warm-up
     times = []
     t_start = time.perf_counter()
-    while len(times) < 20 or (time.perf_counter() - t_start < budget_s and len(times) < 400):
+    while len(times) < 20 or (time.perf_counter() - t_start < budget_s and len(times) < 8000):
         t0 = time.perf_counter()
         oracle.attention_gen(q, k, v, hkv, L, L, impl="avx2", n_threads=cores)
         times.append(time.perf_counter() - t0)

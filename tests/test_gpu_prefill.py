@@ -97,6 +97,19 @@ def test_config2_llama1b_shape_all_f16():
     check_attention_out(got32, ref)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_grid_that_fills_the_device_with_four_wave_workgroups(d):
+    # Two sequences of the config-2 shape give 512 workgroups: the launcher then runs one KV group
+    # per workgroup (two independent workgroups per compute unit) instead of two groups in one.
+    b, s, hq, hkv = 2, 2048, 32, 8
+    q = f16(normal((b, s, hq, d), 7))
+    k = f16(normal((b, hkv, s, d), 8))
+    v = f16(normal((b, hkv, s, d), 9))
+    rc, got = run_prefill(q, k, v, hkv, s, s)
+    assert rc == 1
+    check_attention_out(got, O.prefill_attention(q.astype(np.float32), k, v, hkv, s, s))
+
+
 def test_batched_prefill_with_capacity_and_offset():
     b, s, hq, hkv, d, cap, csl = 3, 150, 8, 2, 128, 400, 333
     q = normal((b, s, hq, d), 1)
