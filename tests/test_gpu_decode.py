@@ -180,6 +180,35 @@ def test_batched_sequences_match_looped_calls():
         check_scores(sc[i], p, "seq %d" % i)
 
 
+@pytest.mark.parametrize("hq,hkv,d,L", [(32, 8, 128, 4096), (14, 2, 64, 1024), (16, 1, 64, 3000), (3, 3, 128, 777),
+                                       (32, 4, 256, 8192), (24, 6, 256, 9000), (7, 1, 128, 20000)])
+def test_calls_without_scores_alternating_lengths(hq, hkv, d, L):
+    # Calls of different lengths (so different split counts) alternate on one context and share its
+    # partial workspace: state left over from the previous call would show as a wrong output.
+    cap = L + 5
+    q = normal((hq, d), 1 + L)
+    k = f16(normal((hkv, cap, d), 2 + L))
+    v = f16(normal((hkv, cap, d), 3 + L))
+    lengths = [L, 64 + L // 3, L, 100]
+    refs = {n: O.attention_gen(q, k, v, hkv, n, cap) for n in set(lengths)}
+    for rep in range(3):
+        for n in lengths:
+            check_attention_out(run_decode(q, k, v, hkv, n, cap), refs[n], "len %d rep %d" % (n, rep))
+
+
+def test_calls_without_scores_batch_and_fallback():
+    b, hq, hkv, d, L, cap = 6, 16, 4, 128, 2000, 2048
+    q = normal((b, hq, d), 5)
+    k = f16(normal((b, hkv, cap, d), 6))
+    v = f16(normal((b, hkv, cap, d), 7))
+    k[2, 1] = np.nan  # every logit of that KV head's four query heads is NaN: uniform weights
+    k[4, 3, 17, 0] = np.nan
+    for rep in range(2):
+        got = run_decode(q, k, v, hkv, L, cap, batch=b, kv_batch_stride=hkv * cap * d)
+        for i in range(b):
+            check_attention_out(got[i], O.attention_gen(q[i], k[i], v[i], hkv, L, cap), "seq %d rep %d" % (i, rep))
+
+
 def test_config1_qwen_shape():
     # BASELINE config 1: Hq14 Hkv2 d64 L1024, f32 N(0,1) -> F16 KV, scale 1/8.
     hq, hkv, d, L = 14, 2, 64, 1024
