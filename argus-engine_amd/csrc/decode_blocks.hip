@@ -8,9 +8,12 @@
 // q4_0: x = d * (n - 8), q4_1: x = d * n + m, n = 4-bit code, element i in the low nibble of code
 // byte i, element 16 + i in the high nibble; q8_0: x = d * c, c = int8.
 //
-// Same data flow as decode_mfma.hip (nothing goes through LDS memory).  A lane turns the 4 (q4) or
-// 8 (q8) code bytes it loaded into 8 f16 values: v_perm puts each code under the exponent of 1024
-// and a packed subtract leaves the exact integer.
+// Same data flow as decode_mfma.hip.  Rows are requested one whole block per lane (contiguous 16 or
+// 32 code bytes, so a request touches each cache line once) and the lanes then trade dwords
+// (v_permlane swaps for K, a wave-private LDS strip for 4-bit V rows) until each holds the 4 (q4) or
+// 8 (q8) code bytes of its MFMA operand, which it turns into 8 f16 values: q8 bytes go under the
+// exponent of 1024 with v_perm and a packed subtract leaves the exact integer; q4 nibbles are
+// masked into the mantissa of 64 + n.
 //   S^T[token][head] = sum over blocks kk of d_kk(token) * (C_kk . Q_kk^T)
 //       v_mfma_f32_16x16x32_f16 per 32-element block with A = the integer codes n - 8 (q4_0), n
 //       (q4_1) or c (q8_0) -- lane (j, r) = token r, code bytes 4j..4j+3 of block kk, i.e. elements
@@ -85,10 +88,9 @@ __device__ __forceinline__ RawPiece<FMT> load_piece(const uint8_t *base, uint32_
   return p;
 }
 
-// A whole block as one lane loads it when head_dim is 128: the K rows of a tile are read one block
-// per lane (lane group j takes block j of row r: 16 or 32 contiguous code bytes), which touches
-// each cache line of the tile once per request instead of once per 4-byte piece, and the lane
-// groups then trade dwords (block_to_pieces).
+// A whole block as one lane loads it: the rows of a tile are read one block per lane (16 or 32
+// contiguous code bytes), which touches each cache line of the tile once per request instead of
+// once per 4-byte piece, and the lanes then trade dwords (block_to_pieces, the V strip).
 template <int FMT>
 struct RawBlock {
   uint32_t code[4 * BlockFmt<FMT>::CW];
@@ -280,42 +282,56 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg) vblk[sg] = (4 * sg + r / 4) % KK;
 
-  constexpr bool kBlockLoads = KK == 4;  // head_dim 128: one block per lane, traded between lane groups
-  RawPiece<FMT> kraw[TW][kBlockLoads ? 1 : KK];
-  RawBlock<FMT> kblk[TW];
-  // ... and for the 4-bit formats the V rows too: lane (j, r) takes block r/4 of token 4j + r%4, and
-  // the four lanes of a quad trade dwords through a wave-private strip of LDS (16 bytes per lane,
-  // plus 16 bytes after every 16 lanes so that the four lane groups read different banks).
-  constexpr bool kStageV = kBlockLoads && FMT != kFmtQ8_0;
+  // K rows are read one whole block per lane and traded between the lane groups (load_block,
+  // block_to_pieces).  A wave-wide request covers 16 rows x 4 blocks: one 16-token tile at
+  // head_dim 128, half of one at 256 (two requests per tile), both tiles of an iteration at 64
+  // (lane group j takes block j % 2 of tile j / 2).
+  static_assert(D != 64 || TW == 2, "head_dim 64 pairs the two tiles of an iteration in one request");
+  constexpr int KQ = (D == 64) ? 1 : KK / 4;        // requests per tile (head_dim 64: per iteration)
+  constexpr int KL = (D == 64) ? 1 : TW * KQ;
+  RawBlock<FMT> kblk[KL];
+  // ... and for the 4-bit formats the V rows too: lane (j, r) takes block r/4 (of the request's four)
+  // of token 4j + r%4, and the lanes trade dwords through a wave-private strip of LDS (16 bytes per
+  // lane, plus 16 bytes after every 16 lanes so that the four lane groups read different banks).
+  // head_dim 64: lanes r < 8 take tile 0, the others tile 1.  q8_0 V rows are read in 8-byte pieces.
+  constexpr bool kStageV = FMT != kFmtQ8_0;
+  constexpr int VL = (D == 64) ? 1 : TW * VSEG;
   RawPiece<FMT> vraw[TW][VSEG][kStageV ? 1 : 4];
-  RawBlock<FMT> vblk_raw[TW];
+  RawBlock<FMT> vblk_raw[kStageV ? VL : 1];
   // Rows past the chunk re-read its last row (they are masked below), so every request is
   // unconditional and a tile may be asked for before it is known to exist.
   const int last = t_end - 1;
   auto load_k = [&](int base) {
+    if constexpr (D == 64) {
+      const uint32_t off = __umul24((uint32_t)min(base + 16 * (j >> 1) + r, last), row_bytes);
+      kblk[0] = load_block<FMT>(kb, off + (uint32_t)((j & 1) * F::BB));
+    } else {
 #pragma unroll
-    for (int tw = 0; tw < TW; ++tw) {
-      const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + r, last), row_bytes);
-      if constexpr (kBlockLoads) {
-        kblk[tw] = load_block<FMT>(kb, off + (uint32_t)(j * F::BB));
-      } else {
+      for (int tw = 0; tw < TW; ++tw) {
+        const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + r, last), row_bytes);
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) kraw[tw][kk] = load_piece<FMT>(kb, off + (uint32_t)(kk * F::BB), (uint32_t)j);
+        for (int u = 0; u < KQ; ++u) kblk[tw * KQ + u] = load_block<FMT>(kb, off + (uint32_t)((4 * u + j) * F::BB));
       }
     }
   };
   auto load_v = [&](int base) {
+    if constexpr (kStageV && D == 64) {
+      const uint32_t off = __umul24((uint32_t)min(base + 16 * (r >> 3) + 4 * j + (r & 3), last), row_bytes);
+      vblk_raw[0] = load_block<FMT>(vb, off + (uint32_t)(((r >> 2) & 1) * F::BB));
+    } else {
 #pragma unroll
-    for (int tw = 0; tw < TW; ++tw) {
-      if constexpr (kStageV) {
-        const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + (r & 3), last), row_bytes);
-        vblk_raw[tw] = load_block<FMT>(vb, off + (uint32_t)((r >> 2) * F::BB));
-      } else {
+      for (int tw = 0; tw < TW; ++tw) {
+        if constexpr (kStageV) {
+          const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + (r & 3), last), row_bytes);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + e, last), row_bytes);
+          for (int sg = 0; sg < VSEG; ++sg) vblk_raw[tw * VSEG + sg] = load_block<FMT>(vb, off + (uint32_t)((4 * sg + (r >> 2)) * F::BB));
+        } else {
 #pragma unroll
-          for (int sg = 0; sg < VSEG; ++sg) vraw[tw][sg][e] = load_piece<FMT>(vb, off + (uint32_t)(vblk[sg] * F::BB), (uint32_t)(r & 3));
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + e, last), row_bytes);
+#pragma unroll
+            for (int sg = 0; sg < VSEG; ++sg) vraw[tw][sg][e] = load_piece<FMT>(vb, off + (uint32_t)(vblk[sg] * F::BB), (uint32_t)(r & 3));
+          }
         }
       }
     }
@@ -374,15 +390,23 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
   for (int base = base0; base < t_end; base += kWaves * TILE) {
     // ---- logits ---------------------------------------------------------------------------------
     float4_t s[TW];
+    RawPiece<FMT> both[4];  // head_dim 64: lane group g held block g % 2 of tile g / 2
+    if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       s[tw] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
       RawPiece<FMT> kpc[KK];
-      if constexpr (kBlockLoads) {
-        block_to_pieces<FMT>(kblk[tw], kpc);
+      if constexpr (D == 64) {
+        kpc[0] = both[2 * tw];
+        kpc[1] = both[2 * tw + 1];
       } else {
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) kpc[kk] = kraw[tw][kk];
+        for (int u = 0; u < KQ; ++u) {
+          RawPiece<FMT> four[4];
+          block_to_pieces<FMT>(kblk[tw * KQ + u], four);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) kpc[4 * u + x] = four[x];
+        }
       }
 #pragma unroll
       for (int kp = 0; kp < KK / 2; ++kp) {
@@ -417,6 +441,10 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         }
       }
     }
+    // The requests stay behind the logits: when the scheduler was free to move them up between the
+    // last block's MFMAs, the q4_1 head_dim 256 build returned wrong logits for the iteration's last
+    // tile (register data flow of that build read correct; cause not identified).
+    __builtin_amdgcn_sched_barrier(0);
     load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
     const bool full = base + TILE <= t_end;
     if (!full) {  // uniform: only the chunk's last tile has rows to mask
@@ -491,16 +519,25 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
       for (int sg = 0; sg < VSEG; ++sg) {
         RawPiece<FMT> vpc[4];  // the lane's piece of tokens 4j .. 4j+3
         if constexpr (kStageV) {
-          __shared__ uint32_t v_strip[kWaves][TW][64 * 4 + 4 * 4];
-          uint32_t *strip = v_strip[wave][tw];
           typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-          *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{vblk_raw[tw].code[0], vblk_raw[tw].code[1], vblk_raw[tw].code[2], vblk_raw[tw].code[3]};
-          // token 4j + e was loaded by lane 16j + 4(r/4) + e; this lane wants dword r%4 of it
-          const uint32_t *src = strip + 68 * j + 16 * (r >> 2) + (r & 3);
+          __shared__ uint32_t v_strip[kWaves][VL][64 * 4 + 4 * 4];
+          constexpr bool kShared = D == 64;  // one request serves both tiles
+          const RawBlock<FMT> &mine = vblk_raw[kShared ? 0 : tw * VSEG + sg];
+          uint32_t *strip = v_strip[wave][kShared ? 0 : tw * VSEG + sg];
+          if (!kShared || tw == 0)
+            *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{mine.code[0], mine.code[1], mine.code[2], mine.code[3]};
+          // token 4j + e was loaded by lane 16j + 4(r/4) + e (head_dim 64: 16j + 8 tw + 4(r/4 % 2) + e);
+          // this lane wants dword r%4 of it
+          const int quad = kShared ? 2 * tw + ((r >> 2) & 1) : (r >> 2);
+          const uint32_t *src = strip + 68 * j + 16 * quad + (r & 3);
 #pragma unroll
           for (int e = 0; e < 4; ++e) vpc[e].code[0] = src[4 * e];
-          // header of token 4j + e: lane e of the quad has it
-          const int own_hdr = (int)vblk_raw[tw].hdr;
+          // header of token 4j + e: lane e of that quad has it (head_dim 64: the quad may sit 8 lanes away)
+          int own_hdr = (int)mine.hdr;
+          if constexpr (kShared) {
+            const int other = __builtin_amdgcn_update_dpp(0, own_hdr, 0x128, 0xf, 0xf, false);  // row_ror:8
+            own_hdr = ((r >> 3) == tw) ? own_hdr : other;
+          }
           vpc[0].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0x00, 0xf, 0xf, false);
           vpc[1].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0x55, 0xf, 0xf, false);
           vpc[2].hdr = (uint32_t)__builtin_amdgcn_update_dpp(0, own_hdr, 0xaa, 0xf, 0xf, false);
@@ -586,7 +623,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 
 template <int FMT, int D>
 int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
-  constexpr int TW = 2;
+  constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
   constexpr int tile_rows = kWaves * 16 * TW;
   static int wgs_per_cu = 0;  // per instantiation; single inference thread
   if (wgs_per_cu == 0) {

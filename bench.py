@@ -379,6 +379,10 @@ def main():
             "--kv-format q4_0 rows attended in-kernel, 604 MB of blocks")
         add("cfg3_q8_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q8_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q8_0 rows attended in-kernel, 1141 MB of blocks")
+        add("qwen_d64_q4_0_blocks_L32768_b64", bench_decode_blocks(ctx, "q4_0", 14, 2, 64, 32768, 64, es, ew),
+            "head_dim 64 (Hq14 Hkv2), 302 MB of q4_0 blocks")
+        add("gemma_d256_q4_0_blocks_L32768_b8", bench_decode_blocks(ctx, "q4_0", 16, 8, 256, 32768, 8, es, ew),
+            "head_dim 256 (Hq16 Hkv8), 604 MB of q4_0 blocks")
         ex["cfg2_prefill_llama1b_S2048_f16"] = bench_prefill(ctx, es, ew)
         ex["cfg2_prefill_llama1b_S2048_f32io"] = bench_prefill(ctx, es, ew, f16_io=False)
         ex["prefill_llama8b_d128_S8192_f16"] = bench_prefill(ctx, max(5, es // 4), 2, hq=32, hkv=8, d=128, s=8192)

@@ -86,6 +86,21 @@ def test_long_row_at_32k_tokens():
     run_case("q4_0", 32, 8, 128, 32768, scores=True, seed=5)
 
 
+@pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_1", 8, 4, 256, 20000), ("q4_0", 14, 2, 64, 20000), ("q8_0", 8, 2, 256, 20000),
+                                            ("q4_1", 14, 2, 64, 33000), ("q8_0", 4, 4, 64, 17001), ("q4_0", 16, 2, 256, 9999)])
+def test_several_tiles_per_wave_at_every_head_dim(fmt, hq, hkv, d, L):
+    # Long rows give every wave more than one tile, so the tile requested ahead of the one being
+    # worked on is the one consumed next (head_dim 64 pairs two tiles per request, 256 splits one over two).
+    run_case(fmt, hq, hkv, d, L, cap=L + 3, seed=L % 97)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0"])
+@pytest.mark.parametrize("d", [64, 256])
+def test_ragged_lengths_at_head_dim_64_and_256(fmt, d):
+    for L in (1, 7, 16, 17, 31, 32, 33, 47, 48, 49, 64, 65, 100, 129, 333):
+        run_case(fmt, 8, 2, d, L, cap=400, seed=L + d)
+
+
 def test_batch_of_sequences():
     import argus_hip as A
     desc, _ = FORMATS["q4_0"]
