@@ -210,6 +210,34 @@ __device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p) {
   return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
 }
 
+// Half a piece (head_dim 64): the element held by slot s of the half `upper` of code index x, and
+// its 4 values d * code.  q4: `upper` selects the high nibbles, brought down by a per-lane shift so
+// that both halves run the same instructions; q8: the piece's one code dword is already the half.
+template <int FMT>
+__host__ __device__ constexpr int half_slot_elem(int x, int upper, int s) {
+  if (FMT == kFmtQ8_0) return 8 * x + 4 * upper + s;
+  return 16 * upper + 4 * x + (s == 1 ? 2 : (s == 2 ? 1 : s));  // 0, 2, 1, 3
+}
+template <int FMT>
+__device__ __forceinline__ half4_t scaled_half(const RawPiece<FMT> &p, uint32_t upper) {
+  const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u));  // {d, d}
+  half2_t v[2];
+  if constexpr (FMT == kFmtQ8_0) {
+    const half2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    const uint32_t u = p.code[0] ^ 0x80808080u;
+    v[0] = (bytes_lo(u) + off) * dd;
+    v[1] = (bytes_hi(u) + off) * dd;
+  } else {
+    const uint32_t w = p.code[0] >> (4u * upper);
+    uint32_t mask = 0x00f000f0u, exponent = 0x54005400u;
+    asm("" : "+v"(mask), "+v"(exponent));
+    const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
+    v[0] = __builtin_elementwise_fma(nibbles(w << 4, mask, exponent), dd, nb);  // bytes 0, 2
+    v[1] = __builtin_elementwise_fma(nibbles(w >> 4, mask, exponent), dd, nb);  // bytes 1, 3
+  }
+  return half4_t{v[0][0], v[0][1], v[1][0], v[1][1]};
+}
+
 // One element of a block as f32 (rare paths only).
 template <int FMT>
 __device__ float block_elem(const uint8_t *blk, int e) {
@@ -249,8 +277,12 @@ constexpr int kWaves = 4;
 template <int D>
 struct BlockShape {
   static constexpr int KK = D / 32;                       // blocks per row
-  static constexpr int VSEG = (D + 127) / 128;            // V pieces per lane per row (8 channels each)
-  static constexpr int NACC = 8 * VSEG;                   // O accumulators (float4 each)
+  static constexpr int VSEG = (D + 127) / 128;            // V pieces per lane per row
+  // Channels a lane takes from a V piece: all 8, or at head_dim 64 (where 8 lanes would cover the
+  // row and the other 8 repeat them) half a piece: lanes r < 8 the low nibbles / first code dword,
+  // lanes r >= 8 the high nibbles / second dword.
+  static constexpr int VCH = (D == 64) ? 4 : 8;
+  static constexpr int NACC = VCH * VSEG;                 // O accumulators (float4 each)
   static constexpr int MAXH = (D == 256) ? 8 : 16;        // query heads per KV head (bounds the merge LDS)
 };
 
@@ -259,7 +291,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
   using CD = Codec<FMT>;
-  constexpr int KK = SH::KK, VSEG = SH::VSEG, NACC = SH::NACC;
+  constexpr int KK = SH::KK, VSEG = SH::VSEG, NACC = SH::NACC, VCH = SH::VCH;
   constexpr int TILE = 16 * TW;  // tokens per wave iteration
   constexpr float kLn2 = 0.6931471805599453f;
 
@@ -330,7 +362,15 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
           for (int e = 0; e < 4; ++e) {
             const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + e, last), row_bytes);
 #pragma unroll
-            for (int sg = 0; sg < VSEG; ++sg) vraw[tw][sg][e] = load_piece<FMT>(vb, off + (uint32_t)(vblk[sg] * F::BB), (uint32_t)(r & 3));
+            for (int sg = 0; sg < VSEG; ++sg) {
+              if constexpr (D == 64) {  // q8_0: the lane's half of the piece is one dword
+                const uint32_t blk = off + (uint32_t)(vblk[sg] * F::BB);
+                vraw[tw][sg][e].hdr = *(const uint16_t *)(vb + blk);
+                vraw[tw][sg][e].code[0] = *(const u32_a2 *)(vb + (blk + (uint32_t)F::HDR + 4u * (uint32_t)(2 * (r & 3) + (r >> 3))));
+              } else {
+                vraw[tw][sg][e] = load_piece<FMT>(vb, off + (uint32_t)(vblk[sg] * F::BB), (uint32_t)(r & 3));
+              }
+            }
           }
         }
       }
@@ -546,9 +586,13 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
           for (int e = 0; e < 4; ++e) vpc[e] = vraw[tw][sg][e];
         }
-        half8_t vrow[4];
+        typedef _Float16 vrow_t __attribute__((ext_vector_type(VCH)));
+        vrow_t vrow[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) vrow[e] = scaled_codes<FMT>(vpc[e]);
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (D == 64) vrow[e] = scaled_half<FMT>(vpc[e], (uint32_t)(r >> 3));
+          else vrow[e] = scaled_codes<FMT>(vpc[e]);
+        }
         if constexpr (kHdrTerm) {
           // d (q4_0: low halves of the headers) or m (q4_1: high halves) of the lane's four tokens
           constexpr uint32_t sel = (FMT == kFmtQ4_1) ? 0x07060302u : 0x05040100u;
@@ -559,9 +603,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
           h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
         }
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
+        for (int c = 0; c < VCH; ++c) {
           const half4_t bv = {vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
-          o_acc[sg * 8 + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * 8 + c], 0, 0, 0);
+          o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * VCH + c], 0, 0, 0);
         }
       }
     load_v(base + kWaves * TILE);
@@ -572,9 +616,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
     for (int sg = 0; sg < VSEG; ++sg)
 #pragma unroll
-      for (int c = 0; c < 8; ++c)
+      for (int c = 0; c < VCH; ++c)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o_acc[sg * 8 + c][i] = fmaf(kTerm, h_acc[sg][i], o_acc[sg * 8 + c][i]);
+        for (int i = 0; i < 4; ++i) o_acc[sg * VCH + c][i] = fmaf(kTerm, h_acc[sg][i], o_acc[sg * VCH + c][i]);
   }
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
@@ -586,15 +630,15 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     lds_m[wave][r] = m_run;
     lds_l[wave][r] = l_run;
   }
-  if (r < 4 * KK || VSEG > 1) {  // head_dim 64: lanes 8..15 hold copies
 #pragma unroll
-    for (int sg = 0; sg < VSEG; ++sg)
+  for (int sg = 0; sg < VSEG; ++sg)
 #pragma unroll
-      for (int c = 0; c < 8; ++c)
+    for (int c = 0; c < VCH; ++c) {
+      const int ch = 32 * vblk[sg] + ((D == 64) ? half_slot_elem<FMT>(r & 3, r >> 3, c) : slot_elem<FMT>(r & 3, c));
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][32 * vblk[sg] + slot_elem<FMT>(r & 3, c)] = o_acc[sg * 8 + c][i];
-  }
+      for (int i = 0; i < 4; ++i)
+        if (4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][ch] = o_acc[sg * VCH + c][i];
+    }
   __syncthreads();
 
   for (int idx = threadIdx.x; idx < G * D; idx += 64 * kWaves) {
