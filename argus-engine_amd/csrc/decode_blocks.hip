@@ -286,14 +286,15 @@ struct BlockShape {
   static constexpr int MAXH = (D == 256) ? 8 : 16;        // query heads per KV head (bounds the merge LDS)
 };
 
-template <int FMT, int D, int TW>
+template <int FMT, int D, int TW, bool SOFTCAP>
 __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
   using CD = Codec<FMT>;
   constexpr int KK = SH::KK, VSEG = SH::VSEG, NACC = SH::NACC, VCH = SH::VCH;
   constexpr int TILE = 16 * TW;  // tokens per wave iteration
-  constexpr float kLn2 = 0.6931471805599453f;
+  constexpr float kLn2 = 0.6931471805599453f, kLog2e = 1.4426950408889634f;
+  const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
 
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -486,6 +487,17 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     // tile (register data flow of that build read correct; cause not identified).
     __builtin_amdgcn_sched_barrier(0);
     load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
+    if constexpr (SOFTCAP) {
+      // cap * tanh(logit / cap) on the natural-unit logit (flash_attn_f32_f16.cl:563-565), back to log2 units
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float sv = s[tw][i];
+          const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * kLog2e;
+          s[tw][i] = (sv != sv) ? kNegInf : capped;
+        }
+    }
     const bool full = base + TILE <= t_end;
     if (!full) {  // uniform: only the chunk's last tile has rows to mask
 #pragma unroll
@@ -672,7 +684,7 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   static int wgs_per_cu = 0;  // per instantiation; single inference thread
   if (wgs_per_cu == 0) {
     int n = 0;
-    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_blocks_kernel<FMT, D, TW>, 64 * kWaves, 0));
+    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_blocks_kernel<FMT, D, TW, false>, 64 * kWaves, 0));
     wgs_per_cu = std::max(1, n);
   }
   choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu);
@@ -685,7 +697,8 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   {
     KernelTimer timer(ctx, stream);
-    hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW>), dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
+    if (p.softcap > 0.0f) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true>), dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
+    else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false>), dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<BlockFallback<FMT>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -705,9 +718,9 @@ int launch_blocks_dim(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hip
 }  // namespace
 
 int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtype, int batch, hipStream_t stream) {
-  if (p.kv_index || p.softcap > 0.0f)
+  if (p.kv_index)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED,
-                      "attention_gen: block-quantised caches take no index list or soft-cap; decode them with "
+                      "attention_gen: block-quantised caches take no index list; decode them with "
                       "argus_hip_kv_decode_descriptor and attend the F16 copy");
   if (p.group > ((D == 256) ? 8 : 16))
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: %d query heads per KV head on a block-quantised cache", p.group);

@@ -18,7 +18,7 @@ FORMATS = {
 }
 
 
-def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True, kv_start=0, encode=False):
+def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True, kv_start=0, encode=False, softcap=0.0, q_gain=1.0):
     import argus_hip as A
     desc, name = FORMATS[fmt]
     cap = cap or L
@@ -29,12 +29,12 @@ def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True,
     else:
         k_raw = random_blocks(desc, rows * d // 32, seed + 1)
         v_raw = random_blocks(desc, rows * d // 32, seed + 2)
-    q = normal((hq, d), seed)
+    q = normal((hq, d), seed) * np.float32(q_gain)
     out = dev(np.zeros((hq, d), np.float32))
     sc = dev(np.zeros((hq, L), np.float32)) if scores else None
     ctx().attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, cap,
                         layout=A.HEAD_MAJOR if head_major else A.SEQ_MAJOR, scores=sc,
-                        score_stride=L if scores else 0, kv_start=kv_start, kv_dtype=getattr(A, name))
+                        score_stride=L if scores else 0, kv_start=kv_start, kv_dtype=getattr(A, name), softcap=softcap)
     # oracle: a window that starts at kv_start is the same cache with its first rows cut off
     bb = O.desc_block_bytes(desc)
     row_bytes = d // 32 * bb
@@ -42,9 +42,9 @@ def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True,
         assert head_major
         kr = k_raw.reshape(hkv, cap, row_bytes)[:, kv_start:].reshape(-1)
         vr = v_raw.reshape(hkv, cap, row_bytes)[:, kv_start:].reshape(-1)
-        ref = O.attention_gen_blocks(q, kr, vr, desc, hkv, L, cap - kv_start, scores=scores)
+        ref = O.attention_gen_blocks(q, kr, vr, desc, hkv, L, cap - kv_start, scores=scores, softcap=softcap)
     else:
-        ref = O.attention_gen_blocks(q, k_raw, v_raw, desc, hkv, L, cap, head_major=head_major, scores=scores)
+        ref = O.attention_gen_blocks(q, k_raw, v_raw, desc, hkv, L, cap, head_major=head_major, scores=scores, softcap=softcap)
     what = "%s Hq%d Hkv%d d%d L%d cap%d %s" % (fmt, hq, hkv, d, L, cap, "HM" if head_major else "SM")
     if scores:
         check_attention_out(host(out), ref[0], what)
@@ -101,6 +101,13 @@ def test_ragged_lengths_at_head_dim_64_and_256(fmt, d):
         run_case(fmt, 8, 2, d, L, cap=400, seed=L + d)
 
 
+@pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_0", 16, 8, 256, 2048), ("q8_0", 8, 4, 256, 1000), ("q4_1", 32, 8, 128, 1500), ("q4_0", 14, 2, 64, 777)])
+def test_soft_cap_on_block_caches(fmt, hq, hkv, d, L):
+    # Gemma-2 style logit soft-cap (cap * tanh(logit / cap)) with queries large enough that the cap bites.
+    run_case(fmt, hq, hkv, d, L, cap=L + 8, seed=L % 89, softcap=50.0, q_gain=4.0)
+    run_case(fmt, hq, hkv, d, L, cap=L + 8, seed=L % 89 + 1, softcap=3.0)
+
+
 def test_batch_of_sequences():
     import argus_hip as A
     desc, _ = FORMATS["q4_0"]
@@ -147,7 +154,6 @@ def test_unsupported_combinations_are_refused():
     q = dev(normal((hq, d), 3))
     out = dev(np.zeros((hq, d), np.float32))
     c = ctx()
-    assert c.attention_gen(q, k, k, out, hkv, L, L, softcap=30.0, kv_dtype=A.Q4_0, check=False) == A.ERR_UNSUPPORTED
     idx = dev(np.arange(L, dtype=np.int32))
     assert c.attention_gen(q, k, k, out, hkv, L, L, kv_index=idx, kv_dtype=A.Q4_0, check=False) == A.ERR_UNSUPPORTED
     q17 = dev(normal((34, d), 3))
