@@ -1,4 +1,4 @@
-// KIVI fused dequant + decode attention on the matrix cores (Q2 / Q4 / Q8, head_dim 64 / 128).
+// KIVI fused dequant + decode attention on the matrix cores (Q2 / Q4 / Q8, head_dim 64 / 128 / 256).
 //
 // Same arithmetic as kivi_attn.hip (dequant `code*d + m`, crates/techniques/kivi/src/kivi_attn.cu:
 // 213-218, block layouts kivi_attn.cu:256-262 / 357-361), reorganised so the per-code work is a
@@ -155,14 +155,28 @@ __device__ __forceinline__ void load_row8(const _Float16 *p, float (&o)[8]) {
   for (int e = 0; e < 8; ++e) o[e] = (float)a[e];
 }
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): slice indices must be constants
+// (they select DPP shifts).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 constexpr float kLn2 = 0.6931471805599453f;
 // Power of two on the f16 operands that carry block scales: keeps the low halves of the hi + lo
 // splits and small p*d products out of the f16 subnormal range.
 constexpr float kOpScale = 64.0f;
 constexpr float kCodeUnit = 16777216.0f;  // a raw code field n is the half n * 2^-24
 
+// Query heads per KV head the kernel takes (bounds the merge area).
+constexpr int kMaxGroup = 8;
+
 template <int BITS, int D, int GT>
-__global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) {
+__global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(const KiviParams kp) {
   constexpr int BB = 4 + 32 * BITS / 8;  // block bytes
   constexpr int KK = D / 32;             // 32-channel slices == V blocks per token
   constexpr int TILE_BYTES = D * BB;     // one K tile == one V tile
@@ -174,7 +188,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
   constexpr int VPAD = 16;
   constexpr int V8_VEC = 8 * KK * BB / 16;  // 16-byte vectors per 8 tokens
   constexpr int WAVE_BYTES = 2 * TILE_BYTES + 4 * VPAD;
-  constexpr int MERGE_BYTES = 4 * 16 * (D + 4) * 4 + 4 * 16 * KK * 4 + 2 * 4 * 16 * 4;
+  constexpr int MERGE_BYTES = 4 * kMaxGroup * (D + 4) * 4 + 4 * kMaxGroup * KK * 4 + 2 * 4 * 16 * 4;
   constexpr int SMEM = (4 * WAVE_BYTES > MERGE_BYTES) ? 4 * WAVE_BYTES : MERGE_BYTES;
   constexpr int NREP = 16 / GT;               // lanes of a row that share one head
   constexpr int NS = (KK + NREP - 1) / NREP;  // slices each lane prepares
@@ -361,12 +375,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
       s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bl, s[0], 0, 0, 0);
       s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bl, s[1], 0, 0, 0);
     };
-    qk_slice(std::integral_constant<int, 0>{});
-    qk_slice(std::integral_constant<int, 1>{});
-    if constexpr (KK > 2) {
-      qk_slice(std::integral_constant<int, 2>{});
-      qk_slice(std::integral_constant<int, 3>{});
-    }
+    static_for<KK>(qk_slice);
     // undo the field position and the operand units
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -409,12 +418,7 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
       o_acc[2 * cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b0, o_acc[2 * cb], 0, 0, 0);
       o_acc[2 * cb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b1, o_acc[2 * cb + 1], 0, 0, 0);
     };
-    pv_block(std::integral_constant<int, 0>{});
-    pv_block(std::integral_constant<int, 1>{});
-    if constexpr (KK > 2) {
-      pv_block(std::integral_constant<int, 2>{});
-      pv_block(std::integral_constant<int, 3>{});
-    }
+    static_for<KK>(pv_block);
     // zero-point term: column n = cb holds sum_t p[h][t] m[t][cb]
     u32x4_t mw = {0u, 0u, 0u, 0u};
     if (r < KK) {
@@ -499,22 +503,24 @@ __global__ __launch_bounds__(256, 3) void kivi_mfma_kernel(const KiviParams kp) 
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
   __syncthreads();  // every wave is done with its tile region
-  float(*lds_acc)[16][D + 4] = (float(*)[16][D + 4]) smem;
-  float(*lds_mt)[16][KK] = (float(*)[16][KK])(smem + 4 * 16 * (D + 4) * 4);
-  float(*lds_m)[16] = (float(*)[16])(smem + 4 * 16 * (D + 4) * 4 + 4 * 16 * KK * 4);
+  float(*lds_acc)[kMaxGroup][D + 4] = (float(*)[kMaxGroup][D + 4]) smem;
+  float(*lds_mt)[kMaxGroup][KK] = (float(*)[kMaxGroup][KK])(smem + 4 * kMaxGroup * (D + 4) * 4);
+  float(*lds_m)[16] = (float(*)[16])(smem + 4 * kMaxGroup * (D + 4) * 4 + 4 * kMaxGroup * KK * 4);
   float(*lds_l)[16] = lds_m + 4;
   if (j == 0) {
     lds_m[wave][r] = m_run;
     lds_l[wave][r] = l_run;
   }
+  if (4 * j < kMaxGroup) {  // accumulator rows 4j + i are heads; only the first kMaxGroup can be real
 #pragma unroll
-  for (int cb = 0; cb < KK; ++cb)
+    for (int cb = 0; cb < KK; ++cb)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *(float2 *)&lds_acc[wave][4 * j + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
-  if (r < KK) {
+      for (int i = 0; i < 4; ++i)
+        *(float2 *)&lds_acc[wave][4 * j + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
+    if (r < KK) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
+      for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
+    }
   }
   __syncthreads();
 
@@ -579,15 +585,19 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
 
 template <int BITS>
 int launch_dim(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
-  return kp.head_dim == 64 ? launch<BITS, 64>(ctx, kp, batch, stream) : launch<BITS, 128>(ctx, kp, batch, stream);
+  switch (kp.head_dim) {
+    case 64: return launch<BITS, 64>(ctx, kp, batch, stream);
+    case 128: return launch<BITS, 128>(ctx, kp, batch, stream);
+    default: return launch<BITS, 256>(ctx, kp, batch, stream);
+  }
 }
 
 }  // namespace
 
 bool kivi_mfma_supported(const KiviParams &kp) {
   const DecodeParams &p = kp.d;
-  if (kp.head_dim != 64 && kp.head_dim != 128) return false;
-  if (p.group > 8 || p.softcap > 0.0f) return false;
+  if (kp.head_dim != 64 && kp.head_dim != 128 && kp.head_dim != 256) return false;
+  if (p.group > kMaxGroup || p.softcap > 0.0f) return false;
   // tiles are copied as 16-byte vectors
   if ((((uintptr_t)kp.qk | (uintptr_t)kp.qv) & 15) || (kp.qk_bs & 15) || (kp.qv_bs & 15)) return false;
   // residual rows are read as 16-byte vectors
