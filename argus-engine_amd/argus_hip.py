@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("ARGUS_HIP_LIB") or os.path.join(_HERE, "libargus_hip.
 
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_RUNTIME, ERR_NOMEM = 0, -1, -2, -3, -4
 F32, F16 = 0, 1
-Q4_0, Q4_1, Q8_0 = 2, 3, 4  # block-quantised cache rows (attention_gen)
+Q4_0, Q4_1, Q8_0, Q2_0 = 2, 3, 4, 5  # block-quantised cache rows (attention_gen)
 HEAD_MAJOR, SEQ_MAJOR = 0, 1
 
 EXPORTED_SYMBOLS = [
@@ -254,7 +254,7 @@ class Context:
                       batch=1, kv_batch_stride=0, index_batch_stride=0, softcap=0.0, scale=0.0,
                       check=True, kv_dtype=None):
         """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride].
-        kv_dtype: Q4_0 / Q4_1 / Q8_0 for uint8 tensors of blocks (default: from the tensor dtype)."""
+        kv_dtype: Q4_0 / Q4_1 / Q8_0 / Q2_0 for uint8 tensors of blocks (default: from the tensor dtype)."""
         hq, d = q.shape[-2], q.shape[-1]
         a = AttentionGenArgs(
             stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),

@@ -363,7 +363,8 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
   if (a->batch > 1 && p.kv_bs == 0)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: batch > 1 needs kv_batch_stride");
   // The kernels move K/V rows and output rows as 16-byte vectors.
-  const bool blocks = a->kv_dtype == ARGUS_HIP_Q4_0 || a->kv_dtype == ARGUS_HIP_Q4_1 || a->kv_dtype == ARGUS_HIP_Q8_0;
+  const bool blocks = a->kv_dtype == ARGUS_HIP_Q4_0 || a->kv_dtype == ARGUS_HIP_Q4_1 || a->kv_dtype == ARGUS_HIP_Q8_0 ||
+                      a->kv_dtype == ARGUS_HIP_Q2_0;
   const int64_t kv_vec = blocks ? 32 : (a->kv_dtype == ARGUS_HIP_F16 ? 8 : 4);
   if (((uintptr_t)a->k_cache | (uintptr_t)a->v_cache | (uintptr_t)a->out) & 15)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: k/v/out must be 16-byte aligned");

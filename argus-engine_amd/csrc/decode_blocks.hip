@@ -1,4 +1,4 @@
-// Split-KV flash-decode over block-quantised caches (q4_0, q4_1, q8_0), dequantised in registers.
+// Split-KV flash-decode over block-quantised caches (q4_0, q4_1, q8_0, q2_0), dequantised in registers.
 //
 // The Q4_0 arm of Backend::attention_gen (engine/src/backend/cpu/common.rs:676-850: dequantise each
 // K / V row, then the F32 algorithm with its NaN and uniform-weights guards) and the in-kernel form
@@ -6,7 +6,8 @@
 // (engine/src/kv/standard_format.rs:538-643).  Blocks are the descriptor formats of
 // engine/src/format/dtype_layout.rs:102-166 with 32 elements: [f16 d][f16 m?][codes];
 // q4_0: x = d * (n - 8), q4_1: x = d * n + m, n = 4-bit code, element i in the low nibble of code
-// byte i, element 16 + i in the high nibble; q8_0: x = d * c, c = int8.
+// byte i, element 16 + i in the high nibble; q8_0: x = d * c, c = int8; q2_0: [f16 d][f16 m][8 code
+// bytes], x = d * n + m, element 4i + k in bits 2k, 2k+1 of code byte i (dtype_layout.rs:146-166).
 //
 // Same data flow as decode_mfma.hip.  Rows are requested one whole block per lane (contiguous 16 or
 // 32 code bytes, so a request touches each cache line once) and the lanes then trade dwords
@@ -38,13 +39,16 @@ namespace {
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32_a2 __attribute__((aligned(2)));  // code words sit at 2-byte boundaries (18- and 34-byte blocks)
 
-enum { kFmtQ4_0 = 0, kFmtQ4_1 = 1, kFmtQ8_0 = 2 };
+enum { kFmtQ4_0 = 0, kFmtQ4_1 = 1, kFmtQ8_0 = 2, kFmtQ2_0 = 3 };
 
 template <int FMT>
 struct BlockFmt {
-  static constexpr int HDR = (FMT == kFmtQ4_1) ? 4 : 2;             // header bytes
-  static constexpr int BB = HDR + ((FMT == kFmtQ8_0) ? 32 : 16);    // block bytes
-  static constexpr int CW = (FMT == kFmtQ8_0) ? 2 : 1;              // code dwords per lane piece
+  static constexpr bool kHasMin = FMT == kFmtQ4_1 || FMT == kFmtQ2_0;  // header is (d, m)
+  static constexpr int HDR = kHasMin ? 4 : 2;                                          // header bytes
+  static constexpr int CODE_DW = (FMT == kFmtQ8_0) ? 8 : ((FMT == kFmtQ2_0) ? 2 : 4);  // code dwords per block
+  static constexpr int BB = HDR + 4 * CODE_DW;                                         // block bytes
+  // code dwords per lane piece (q2_0: the piece is one 16-bit half of its dword)
+  static constexpr int CW = (FMT == kFmtQ8_0) ? 2 : 1;
 };
 
 // Element (within its block) held by slot s of the piece a lane with code index x loads
@@ -52,6 +56,7 @@ struct BlockFmt {
 template <int FMT>
 __host__ __device__ constexpr int slot_elem(int x, int s) {
   if (FMT == kFmtQ8_0) return 8 * x + s;
+  if (FMT == kFmtQ2_0) return 8 * x + (s >> 1) + 4 * (s & 1);  // slot 2f + h: field f of byte 2x + h
   const int within = (s & 3) == 1 ? 2 : ((s & 3) == 2 ? 1 : (s & 3));  // 0, 2, 1, 3
   return (s < 4 ? 0 : 16) + 4 * x + within;
 }
@@ -62,10 +67,16 @@ __host__ __device__ constexpr int slot_elem(int x, int s) {
 // block dot product as (bias + zero) * sum(Q), folded into the accumulator the MFMA starts from,
 // and from the values as one fma whose addend -64 d is exact.  q8: the int8 c is made exact by a
 // packed subtract (bias 0).
+// q2_0 (x = d * n + m, four 2-bit codes per byte, element 4i + k in bits 2k.. of byte i) works the
+// same way with two positions: fields 0 and 1 are shifted up by 4, so every code sits at bits 4..5
+// (under the exponent of 64) or bits 6..7 (under the exponent of 16) and the bias depends on the slot.
 template <int FMT>
 struct Codec {
-  static constexpr float kBias = (FMT == kFmtQ8_0) ? 0.0f : 64.0f;  // operand = kBias + code
+  static constexpr float kBias = (FMT == kFmtQ8_0) ? 0.0f : 64.0f;  // operand = kBias + code (q2_0: slot_bias)
   static constexpr float kZero = (FMT == kFmtQ4_0) ? 8.0f : 0.0f;   // value = d * (code - kZero) (+ m)
+  static __host__ __device__ constexpr float slot_bias(int s) {
+    return (FMT == kFmtQ2_0) ? (((s >> 1) & 1) ? 16.0f : 64.0f) : kBias;
+  }
 };
 
 // What one lane holds of one block before it is dequantised.
@@ -81,7 +92,7 @@ template <int FMT>
 __device__ __forceinline__ RawPiece<FMT> load_piece(const uint8_t *base, uint32_t blk, uint32_t x) {
   using F = BlockFmt<FMT>;
   RawPiece<FMT> p;
-  if constexpr (FMT == kFmtQ4_1) p.hdr = *(const uint32_t *)(base + blk);
+  if constexpr (F::kHasMin) p.hdr = *(const uint32_t *)(base + blk);
   else p.hdr = *(const uint16_t *)(base + blk);
 #pragma unroll
   for (int w = 0; w < F::CW; ++w) p.code[w] = *(const u32_a2 *)(base + (blk + (uint32_t)F::HDR + 4u * ((uint32_t)F::CW * x + (uint32_t)w)));
@@ -93,7 +104,7 @@ __device__ __forceinline__ RawPiece<FMT> load_piece(const uint8_t *base, uint32_
 // once per 4-byte piece, and the lanes then trade dwords (block_to_pieces, the V strip).
 template <int FMT>
 struct RawBlock {
-  uint32_t code[4 * BlockFmt<FMT>::CW];
+  uint32_t code[BlockFmt<FMT>::CODE_DW];
   uint32_t hdr;
 };
 typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
@@ -102,13 +113,20 @@ template <int FMT>
 __device__ __forceinline__ RawBlock<FMT> load_block(const uint8_t *base, uint32_t blk) {
   using F = BlockFmt<FMT>;
   RawBlock<FMT> b;
-  if constexpr (FMT == kFmtQ4_1) b.hdr = *(const uint32_t *)(base + blk);
+  if constexpr (F::kHasMin) b.hdr = *(const uint32_t *)(base + blk);
   else b.hdr = *(const uint16_t *)(base + blk);
+  if constexpr (FMT == kFmtQ2_0) {
+    typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+    const u32x2_a4 c = *(const u32x2_a4 *)(base + (blk + (uint32_t)F::HDR));
+    b.code[0] = c[0];
+    b.code[1] = c[1];
+  } else {
 #pragma unroll
-  for (int w = 0; w < F::CW; ++w) {
-    const u32x4_a2 c = *(const u32x4_a2 *)(base + (blk + (uint32_t)F::HDR + 16u * (uint32_t)w));
+    for (int w = 0; w < F::CW; ++w) {
+      const u32x4_a2 c = *(const u32x4_a2 *)(base + (blk + (uint32_t)F::HDR + 16u * (uint32_t)w));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) b.code[4 * w + i] = c[i];
+      for (int i = 0; i < 4; ++i) b.code[4 * w + i] = c[i];
+    }
   }
   return b;
 }
@@ -134,7 +152,10 @@ __device__ __forceinline__ void block_to_pieces(const RawBlock<FMT> &b, RawPiece
     // piece dword w of code index x is block dword CW * x + w
     uint32_t v[4];
 #pragma unroll
-    for (int x = 0; x < 4; ++x) v[x] = b.code[CW * x + w];
+    for (int x = 0; x < 4; ++x) {
+      if constexpr (FMT == kFmtQ2_0) v[x] = b.code[x >> 1];  // the dword that holds half x
+      else v[x] = b.code[CW * x + w];
+    }
     transpose_lane_groups(v);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) piece[kk].code[w] = v[kk];
@@ -163,10 +184,25 @@ __device__ __forceinline__ half2_t nibbles(uint32_t word, uint32_t mask, uint32_
   return __builtin_bit_cast(half2_t, r);
 }
 
-// The 8 codes of a piece as exact f16 numbers Codec::kBias + code.
+// v_perm selectors that spread one 16-bit half of a dword as [byte, 0, next byte, 0] (q2_0 pieces),
+// and one byte as [byte, 0, byte, 0] (q2_0 half pieces).
+__device__ __forceinline__ uint32_t q2_half_selector(int half) { return half ? 0x0c030c02u : 0x0c010c00u; }
+__device__ __forceinline__ uint32_t q2_byte_selector(int byte) { return 0x0c000c00u | (uint32_t)byte | ((uint32_t)byte << 16); }
+
+// The 8 codes of a piece as exact f16 numbers Codec::slot_bias + code.  `sel` (q2_0 only): the
+// lane's q2_half_selector.
 template <int FMT>
-__device__ __forceinline__ void piece_codes(const RawPiece<FMT> &p, half2_t (&v)[4]) {
-  if constexpr (FMT == kFmtQ8_0) {
+__device__ __forceinline__ void piece_codes(const RawPiece<FMT> &p, half2_t (&v)[4], uint32_t sel) {
+  if constexpr (FMT == kFmtQ2_0) {
+    const uint32_t w = __builtin_amdgcn_perm(0u, p.code[0], sel);  // [byte 2x, 0, byte 2x+1, 0]
+    const uint32_t w4 = w << 4;
+    uint32_t mask_a = 0x00300030u, exp_a = 0x54005400u, mask_b = 0x00c000c0u, exp_b = 0x4c004c00u;
+    asm("" : "+v"(mask_a), "+v"(exp_a), "+v"(mask_b), "+v"(exp_b));
+    v[0] = nibbles(w4, mask_a, exp_a);  // field 0 -> bits 4..5: 64 + n
+    v[1] = nibbles(w4, mask_b, exp_b);  // field 1 -> bits 6..7: 16 + n
+    v[2] = nibbles(w, mask_a, exp_a);   // field 2
+    v[3] = nibbles(w, mask_b, exp_b);   // field 3
+  } else if constexpr (FMT == kFmtQ8_0) {
     // int8 c -> byte c + 128 -> 1024 + 128 + c
     const half2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
 #pragma unroll
@@ -187,21 +223,26 @@ __device__ __forceinline__ void piece_codes(const RawPiece<FMT> &p, half2_t (&v)
 }
 
 template <int FMT>
-__device__ __forceinline__ half8_t code_operand(const RawPiece<FMT> &p) {
+__device__ __forceinline__ half8_t code_operand(const RawPiece<FMT> &p, uint32_t sel) {
   half2_t v[4];
-  piece_codes<FMT>(p, v);
+  piece_codes<FMT>(p, v, sel);
   return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
 }
 
 // The 8 values of a piece without zero point and minimum, d * code, rounded once to f16.
 template <int FMT>
-__device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p) {
+__device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p, uint32_t sel) {
   const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u));  // {d, d}
   half2_t v[4];
-  piece_codes<FMT>(p, v);
+  piece_codes<FMT>(p, v, sel);
   if constexpr (FMT == kFmtQ8_0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = v[i] * dd;
+  } else if constexpr (FMT == kFmtQ2_0) {
+    const half2_t nb_a = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
+    const half2_t nb_b = dd * half2_t{(_Float16)-16.0f, (_Float16)-16.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_elementwise_fma(v[i], dd, (i & 1) ? nb_b : nb_a);
   } else {
     const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
 #pragma unroll
@@ -212,17 +253,25 @@ __device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p) {
 
 // Half a piece (head_dim 64): the element held by slot s of the half `upper` of code index x, and
 // its 4 values d * code.  q4: `upper` selects the high nibbles, brought down by a per-lane shift so
-// that both halves run the same instructions; q8: the piece's one code dword is already the half.
+// that both halves run the same instructions; q8: the piece's one code dword is already the half;
+// q2_0: `sel` is the lane's q2_byte_selector (the half is one byte: four fields).
 template <int FMT>
 __host__ __device__ constexpr int half_slot_elem(int x, int upper, int s) {
-  if (FMT == kFmtQ8_0) return 8 * x + 4 * upper + s;
+  if (FMT == kFmtQ8_0 || FMT == kFmtQ2_0) return 8 * x + 4 * upper + s;
   return 16 * upper + 4 * x + (s == 1 ? 2 : (s == 2 ? 1 : s));  // 0, 2, 1, 3
 }
 template <int FMT>
-__device__ __forceinline__ half4_t scaled_half(const RawPiece<FMT> &p, uint32_t upper) {
+__device__ __forceinline__ half4_t scaled_half(const RawPiece<FMT> &p, uint32_t upper, uint32_t sel) {
   const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u));  // {d, d}
   half2_t v[2];
-  if constexpr (FMT == kFmtQ8_0) {
+  if constexpr (FMT == kFmtQ2_0) {
+    const uint32_t w = __builtin_amdgcn_perm(0u, p.code[0], sel);  // [byte, 0, byte, 0]
+    uint32_t mask = 0x00c00030u, exponent = 0x4c005400u;           // low half: bits 4..5 (64 + n), high half: bits 6..7 (16 + n)
+    asm("" : "+v"(mask), "+v"(exponent));
+    const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-16.0f};  // exact
+    v[0] = __builtin_elementwise_fma(nibbles(w << 4, mask, exponent), dd, nb);  // fields 0, 1
+    v[1] = __builtin_elementwise_fma(nibbles(w, mask, exponent), dd, nb);       // fields 2, 3
+  } else if constexpr (FMT == kFmtQ8_0) {
     const half2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
     const uint32_t u = p.code[0] ^ 0x80808080u;
     v[0] = (bytes_lo(u) + off) * dd;
@@ -244,6 +293,8 @@ __device__ float block_elem(const uint8_t *blk, int e) {
   using F = BlockFmt<FMT>;
   const float d = (float)*(const _Float16 *)blk;
   if constexpr (FMT == kFmtQ8_0) return d * (float)(int8_t)blk[F::HDR + e];
+  if constexpr (FMT == kFmtQ2_0)
+    return d * (float)((blk[F::HDR + (e >> 2)] >> (2 * (e & 3))) & 3) + (float)*(const _Float16 *)(blk + 2);
   const int byte = blk[F::HDR + (e & 15)];
   const int n = e < 16 ? (byte & 15) : (byte >> 4);
   if constexpr (FMT == kFmtQ4_0) return d * (float)(n - 8);
@@ -384,7 +435,8 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 
   // ---- Q operand: lane (j, h = r), block kk: the elements slot_elem(j, 0..7), log2 domain, hi + lo
   half8_t qh[KK], ql[KK];
-  float qsum[KK];  // sum of the scaled query over block kk: bias / zero-point and minimum terms
+  float qsum[KK];   // sum of the scaled query over block kk: the minimum term
+  float qinit[KK];  // what a block's MFMA accumulator starts from: -sum over the block of (slot bias + zero point) * q
   {
     const float c = p.scale * 1.4426950408889634f;
     const int h = kvh * G + min(r, G - 1);
@@ -395,11 +447,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
       for (int s = 0; s < 8; ++s) qv[s] = qp[32 * kk + slot_elem<FMT>(j, s)];  // lanes past the group re-read its last head
       loaded8(qv);
-      float part = 0.0f;
+      float part = 0.0f, biased = 0.0f;
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
         const float x = (r < G) ? qv[s] * c : 0.0f;
         part += x;
+        if constexpr (FMT == kFmtQ2_0) biased = fmaf(CD::slot_bias(s), x, biased);
         _Float16 hi, lo;
         split_f16(x, hi, lo);
         qh[kk][s] = hi;
@@ -409,11 +462,22 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
       part += __shfl_xor(part, 16, 64);
       part += __shfl_xor(part, 32, 64);
       qsum[kk] = part;
+      if constexpr (FMT == kFmtQ2_0) {
+        biased += __shfl_xor(biased, 16, 64);
+        biased += __shfl_xor(biased, 32, 64);
+        qinit[kk] = -biased;
+      } else {
+        qinit[kk] = -(CD::kBias + CD::kZero) * part;
+      }
     }
   }
   // Result lane (j, h) of a logits MFMA holds tokens 4j..4j+3; their block headers were loaded by
   // lanes 16j + (4j + i) (token = lane % 16).
   int hdr_src[4];
+  // q2_0: which 16-bit half of a code dword is this lane's piece (K: code index j; V: code index r % 4),
+  // and for head_dim 64 which byte of the dword is its half piece
+  const uint32_t k_sel = q2_half_selector(j & 1), v_sel = q2_half_selector(r & 1);
+  const uint32_t v_half_sel = q2_byte_selector(2 * (r & 1) + (r >> 3));
 #pragma unroll
   for (int i = 0; i < 4; ++i) hdr_src[i] = 4 * (20 * j + i);  // ds_bpermute byte address
 
@@ -455,14 +519,14 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const int kk = 2 * kp + u;
-          const half8_t ka = code_operand<FMT>(kpc[kk]);
-          // sum of (code - zero) * q = sum of operand * q - (bias + zero) * sum of q
-          const float c0 = -(CD::kBias + CD::kZero) * qsum[kk];
+          const half8_t ka = code_operand<FMT>(kpc[kk], k_sel);
+          // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q
+          const float c0 = qinit[kk];
           dot[u] = float4_t{c0, c0, c0, c0};
           dot[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qh[kk], dot[u], 0, 0, 0);
           dot[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, ql[kk], dot[u], 0, 0, 0);
         }
-        if constexpr (FMT == kFmtQ4_1) {
+        if constexpr (F::kHasMin) {
           // the header word already holds (d, m): one exchange per token and block
 #pragma unroll
           for (int u = 0; u < 2; ++u)
@@ -576,12 +640,14 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
           constexpr bool kShared = D == 64;  // one request serves both tiles
           const RawBlock<FMT> &mine = vblk_raw[kShared ? 0 : tw * VSEG + sg];
           uint32_t *strip = v_strip[wave][kShared ? 0 : tw * VSEG + sg];
-          if (!kShared || tw == 0)
-            *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{mine.code[0], mine.code[1], mine.code[2], mine.code[3]};
+          if (!kShared || tw == 0) {
+            if constexpr (FMT == kFmtQ2_0) *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{mine.code[0], mine.code[1], 0u, 0u};
+            else *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{mine.code[0], mine.code[1], mine.code[2], mine.code[3]};
+          }
           // token 4j + e was loaded by lane 16j + 4(r/4) + e (head_dim 64: 16j + 8 tw + 4(r/4 % 2) + e);
           // this lane wants dword r%4 of it
           const int quad = kShared ? 2 * tw + ((r >> 2) & 1) : (r >> 2);
-          const uint32_t *src = strip + 68 * j + 16 * quad + (r & 3);
+          const uint32_t *src = strip + 68 * j + 16 * quad + ((FMT == kFmtQ2_0) ? ((r & 3) >> 1) : (r & 3));  // q2_0: the dword with half r%4
 #pragma unroll
           for (int e = 0; e < 4; ++e) vpc[e].code[0] = src[4 * e];
           // header of token 4j + e: lane e of that quad has it (head_dim 64: the quad may sit 8 lanes away)
@@ -602,12 +668,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         vrow_t vrow[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if constexpr (D == 64) vrow[e] = scaled_half<FMT>(vpc[e], (uint32_t)(r >> 3));
-          else vrow[e] = scaled_codes<FMT>(vpc[e]);
+          if constexpr (D == 64) vrow[e] = scaled_half<FMT>(vpc[e], (uint32_t)(r >> 3), v_half_sel);
+          else vrow[e] = scaled_codes<FMT>(vpc[e], v_sel);
         }
         if constexpr (kHdrTerm) {
-          // d (q4_0: low halves of the headers) or m (q4_1: high halves) of the lane's four tokens
-          constexpr uint32_t sel = (FMT == kFmtQ4_1) ? 0x07060302u : 0x05040100u;
+          // d (q4_0: low halves of the headers) or m (q4_1, q2_0: high halves) of the lane's four tokens
+          constexpr uint32_t sel = F::kHasMin ? 0x07060302u : 0x05040100u;
           const uint32_t h01 = __builtin_amdgcn_perm(vpc[1].hdr, vpc[0].hdr, sel);
           const uint32_t h23 = __builtin_amdgcn_perm(vpc[3].hdr, vpc[2].hdr, sel);
           typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
@@ -732,6 +798,7 @@ int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtyp
   switch (kv_dtype) {
     case ARGUS_HIP_Q4_0: return launch_blocks_dim<kFmtQ4_0>(ctx, p, D, batch, stream);
     case ARGUS_HIP_Q4_1: return launch_blocks_dim<kFmtQ4_1>(ctx, p, D, batch, stream);
+    case ARGUS_HIP_Q2_0: return launch_blocks_dim<kFmtQ2_0>(ctx, p, D, batch, stream);
     default: return launch_blocks_dim<kFmtQ8_0>(ctx, p, D, batch, stream);
   }
 }

@@ -104,21 +104,23 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
 
 
 def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1):
-    """Decode attention over a block-quantised cache (q4_0 / q8_0 rows of 18- / 34-byte blocks):
+    """Decode attention over a block-quantised cache (q4_0 / q8_0 / q2_0 rows of 18- / 34- / 12-byte blocks):
     synthetic blocks (random codes, f16 scales sized for N(0,1)-like values); algorithmic bytes are
     the attended block rows of K and V plus Q and out."""
     import torch
     import argus_hip as A
-    bb = {"q4_0": 18, "q8_0": 34}[fmt]
-    kv_dtype = {"q4_0": A.Q4_0, "q8_0": A.Q8_0}[fmt]
+    bb = {"q4_0": 18, "q8_0": 34, "q2_0": 12}[fmt]
+    kv_dtype = {"q4_0": A.Q4_0, "q8_0": A.Q8_0, "q2_0": A.Q2_0}[fmt]
     row_bytes = d // 32 * bb
     g = torch.Generator(device="cuda").manual_seed(11)
 
     def blocks():
         raw = torch.randint(0, 256, (batch * hkv * L * d // 32, bb), generator=g, device="cuda", dtype=torch.uint8)
-        lo, hi = (0.1, 0.3) if fmt == "q4_0" else (0.005, 0.02)
+        lo, hi = {"q4_0": (0.1, 0.3), "q8_0": (0.005, 0.02), "q2_0": (0.8, 1.6)}[fmt]
         scale = (torch.rand(raw.shape[0], generator=g, device="cuda") * (hi - lo) + lo).half()
         raw[:, 0:2] = scale.view(torch.uint8).reshape(-1, 2)
+        if fmt == "q2_0":  # [f16 d][f16 m]: minimum at -1.5 d
+            raw[:, 2:4] = (scale.float() * -1.5).half().view(torch.uint8).reshape(-1, 2)
         return raw.reshape(-1)
 
     ks = [blocks() for _ in range(rotate)]
@@ -379,6 +381,8 @@ def main():
             "--kv-format q4_0 rows attended in-kernel, 604 MB of blocks")
         add("cfg3_q8_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q8_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q8_0 rows attended in-kernel, 1141 MB of blocks")
+        add("cfg3_q2_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q2_0", 32, 8, 128, 32768, 16, es, ew),
+            "--kv-format q2_0 rows attended in-kernel, 403 MB of blocks")
         add("qwen_d64_q4_0_blocks_L32768_b64", bench_decode_blocks(ctx, "q4_0", 14, 2, 64, 32768, 64, es, ew),
             "head_dim 64 (Hq14 Hkv2), 302 MB of q4_0 blocks")
         add("gemma_d256_q4_0_blocks_L32768_b8", bench_decode_blocks(ctx, "q4_0", 16, 8, 256, 32768, 8, es, ew),

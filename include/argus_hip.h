@@ -35,12 +35,14 @@ extern "C" {
 #define ARGUS_HIP_F32 0
 #define ARGUS_HIP_F16 1
 /* Block-quantised cache rows, 32 elements per block (DType::Q4_0 of the reference,
- * engine/src/backend/cpu/common.rs:676-690, and the `--kv-format` descriptors q4_0 / q4_1 / q8_0,
- * engine/src/format/dtype_layout.rs:102-166): [f16 d][16 nibble bytes] = 18 bytes,
- * [f16 d][f16 m][16 nibble bytes] = 20 bytes, [f16 d][32 int8] = 34 bytes.  attention_gen only. */
+ * engine/src/backend/cpu/common.rs:676-690, and the `--kv-format` descriptors q4_0 / q4_1 / q8_0 /
+ * q2_0, engine/src/format/dtype_layout.rs:102-166): [f16 d][16 nibble bytes] = 18 bytes,
+ * [f16 d][f16 m][16 nibble bytes] = 20 bytes, [f16 d][32 int8] = 34 bytes,
+ * [f16 d][f16 m][8 bytes of four 2-bit codes] = 12 bytes.  attention_gen only. */
 #define ARGUS_HIP_Q4_0 2
 #define ARGUS_HIP_Q4_1 3
 #define ARGUS_HIP_Q8_0 4
+#define ARGUS_HIP_Q2_0 5
 
 /* KVLayout, engine/src/kv/kv_cache_ops.rs:18-21. */
 #define ARGUS_HIP_HEAD_MAJOR 0 /* [batch, kv_heads, capacity, head_dim] */
@@ -107,7 +109,7 @@ int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream);
  *   softcap                : cap*tanh(s/cap) after scaling
  *                            (engine/kernels/flash_attn_f32_f16.cl:563-565; host passes 0);
  *   scale                  : 0 selects 1/sqrt(head_dim) (x86.rs:192).
- * Block-quantised caches (kv_dtype ARGUS_HIP_Q4_0 / Q4_1 / Q8_0): the Q4_0 arm of the reference
+ * Block-quantised caches (kv_dtype ARGUS_HIP_Q4_0 / Q4_1 / Q8_0 / Q2_0): the Q4_0 arm of the reference
  * (common.rs:676-850, rows dequantised on the fly) and the in-kernel form of the `--kv-format`
  * attention whose reference floor decodes the whole cache to F32 first
  * (engine/src/kv/standard_format.rs:538-643).  Rows are head_dim/32 blocks; capacity, kv_start and
@@ -129,7 +131,7 @@ typedef struct argus_hip_attention_gen_args {
   int32_t capacity;      /* HeadMajor rows per head; ignored for SeqMajor */
   int32_t kv_start;
   int32_t layout;        /* ARGUS_HIP_HEAD_MAJOR / ARGUS_HIP_SEQ_MAJOR */
-  int32_t kv_dtype;      /* ARGUS_HIP_F16 / ARGUS_HIP_F32 / ARGUS_HIP_Q4_0 / ARGUS_HIP_Q4_1 / ARGUS_HIP_Q8_0 */
+  int32_t kv_dtype;      /* ARGUS_HIP_F16 / ARGUS_HIP_F32 / ARGUS_HIP_Q4_0 / _Q4_1 / _Q8_0 / _Q2_0 */
   int32_t batch;         /* >= 1 */
   int32_t score_stride;  /* floats per head row of scores_out, >= cache_seq_len */
   int64_t q_batch_stride;     /* elements; 0 = num_heads_q*head_dim */

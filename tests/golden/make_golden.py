@@ -76,7 +76,7 @@ def main():
 
 
 def blocks():
-    """attention_gen over q4_0 / q8_0 block rows (own generator, so the fixtures above keep their bytes)."""
+    """attention_gen over q4_0 / q8_0 / q2_0 block rows (own generator, so the fixtures above keep their bytes)."""
     rng = np.random.default_rng(20240922)
     hq, hkv, d, L, cap = 8, 2, 64, 80, 96
     q = rng.standard_normal((hq, d)).astype(np.float32)
@@ -94,6 +94,11 @@ def blocks():
     k8, v8 = q8(hkv * cap * d // 32), q8(hkv * cap * d // 32)
     out, sc = O.attention_gen_blocks(q, k8, v8, O.DESC_Q8_0, hkv, L, cap, scores=True)
     arrays.update(k_q8_0=k8, v_q8_0=v8, out_q8_0=out, scores_q8_0=sc)
+    # q2_0: N(0,1) rows through the reference-shaped asymmetric 2-bit encoder (drawn last: the arrays above keep their bytes)
+    k2 = O.encode_via_descriptor(O.DESC_Q2_0, rng.standard_normal(hkv * cap * d).astype(np.float32))
+    v2 = O.encode_via_descriptor(O.DESC_Q2_0, rng.standard_normal(hkv * cap * d).astype(np.float32))
+    out, sc = O.attention_gen_blocks(q, k2, v2, O.DESC_Q2_0, hkv, L, cap, scores=True)
+    arrays.update(k_q2_0=k2, v_q2_0=v2, out_q2_0=out, scores_q2_0=sc)
     save("blocks", **arrays)
 
 

@@ -152,7 +152,7 @@ def test_gpu_reduce_pfa_descriptor_match_fixtures():
 def test_oracle_block_attention_reproduces_fixture():
     f = load("blocks")
     hq, hkv, d, L, cap = [int(x) for x in f["dims"]]
-    for fmt, desc in (("q4_0", O.DESC_Q4_0), ("q8_0", O.DESC_Q8_0)):
+    for fmt, desc in (("q4_0", O.DESC_Q4_0), ("q8_0", O.DESC_Q8_0), ("q2_0", O.DESC_Q2_0)):
         out, sc = O.attention_gen_blocks(f["q"], f["k_" + fmt], f["v_" + fmt], desc, hkv, L, cap, scores=True)
         assert bits_equal(out, f["out_" + fmt]) and bits_equal(sc, f["scores_" + fmt])
 
@@ -163,7 +163,7 @@ def test_gpu_block_attention_matches_fixture():
     from gpu_util import ctx, dev, host, check_attention_out, check_scores
     f = load("blocks")
     hq, hkv, d, L, cap = [int(x) for x in f["dims"]]
-    for fmt, code in (("q4_0", A.Q4_0), ("q8_0", A.Q8_0)):
+    for fmt, code in (("q4_0", A.Q4_0), ("q8_0", A.Q8_0), ("q2_0", A.Q2_0)):
         out = dev(np.zeros((hq, d), np.float32))
         sc = dev(np.zeros((hq, L), np.float32))
         ctx().attention_gen(dev(f["q"]), dev(f["k_" + fmt]), dev(f["v_" + fmt]), out, hkv, L, cap, scores=sc,

@@ -15,6 +15,7 @@ FORMATS = {
     "q4_0": (O.DESC_Q4_0, "Q4_0"),
     "q4_1": (O.DESC_Q4_1, "Q4_1"),
     "q8_0": (O.DESC_Q8_0, "Q8_0"),
+    "q2_0": (O.DESC_Q2_0, "Q2_0"),
 }
 
 
@@ -53,16 +54,19 @@ def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True,
         check_attention_out(host(out), ref, what)
 
 
-@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0"])
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
 @pytest.mark.parametrize("shape", [(14, 2, 64, 1024), (32, 8, 128, 2048), (8, 4, 256, 1024)])
 def test_baseline_shapes(fmt, shape):
     hq, hkv, d, L = shape
     run_case(fmt, hq, hkv, d, L)
 
 
-def test_q4_0_blocks_made_by_the_reference_encoder():
+def test_blocks_made_by_the_reference_encoder():
+    # encode_via_descriptor writes q4_0 and q2_0 (dtype_layout.rs:302-440)
     run_case("q4_0", 32, 8, 128, 4096, encode=True)
     run_case("q4_0", 14, 2, 64, 1024, encode=True, seed=3)
+    run_case("q2_0", 32, 8, 128, 4096, encode=True, seed=4)
+    run_case("q2_0", 14, 2, 64, 1024, encode=True, seed=5)
 
 
 @pytest.mark.parametrize("L", [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 500, 1000])
@@ -71,7 +75,7 @@ def test_ragged_lengths(L):
     run_case("q8_0", 4, 4, 64, L, cap=1000 if L <= 1000 else L, seed=L + 1)
 
 
-@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0"])
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
 def test_seq_major_and_window_start(fmt):
     run_case(fmt, 16, 4, 128, 777, cap=800, head_major=False, seed=11)
     run_case(fmt, 16, 4, 128, 300, cap=800, kv_start=411, seed=12)
@@ -87,21 +91,23 @@ def test_long_row_at_32k_tokens():
 
 
 @pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_1", 8, 4, 256, 20000), ("q4_0", 14, 2, 64, 20000), ("q8_0", 8, 2, 256, 20000),
-                                            ("q4_1", 14, 2, 64, 33000), ("q8_0", 4, 4, 64, 17001), ("q4_0", 16, 2, 256, 9999)])
+                                            ("q4_1", 14, 2, 64, 33000), ("q8_0", 4, 4, 64, 17001), ("q4_0", 16, 2, 256, 9999),
+                                            ("q2_0", 14, 2, 64, 20000), ("q2_0", 32, 8, 128, 20000), ("q2_0", 16, 8, 256, 9999)])
 def test_several_tiles_per_wave_at_every_head_dim(fmt, hq, hkv, d, L):
     # Long rows give every wave more than one tile, so the tile requested ahead of the one being
     # worked on is the one consumed next (head_dim 64 pairs two tiles per request, 256 splits one over two).
     run_case(fmt, hq, hkv, d, L, cap=L + 3, seed=L % 97)
 
 
-@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0"])
-@pytest.mark.parametrize("d", [64, 256])
-def test_ragged_lengths_at_head_dim_64_and_256(fmt, d):
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_ragged_lengths_at_every_head_dim(fmt, d):
     for L in (1, 7, 16, 17, 31, 32, 33, 47, 48, 49, 64, 65, 100, 129, 333):
         run_case(fmt, 8, 2, d, L, cap=400, seed=L + d)
 
 
-@pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_0", 16, 8, 256, 2048), ("q8_0", 8, 4, 256, 1000), ("q4_1", 32, 8, 128, 1500), ("q4_0", 14, 2, 64, 777)])
+@pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_0", 16, 8, 256, 2048), ("q8_0", 8, 4, 256, 1000), ("q4_1", 32, 8, 128, 1500), ("q4_0", 14, 2, 64, 777),
+                                            ("q2_0", 32, 8, 128, 900)])
 def test_soft_cap_on_block_caches(fmt, hq, hkv, d, L):
     # Gemma-2 style logit soft-cap (cap * tanh(logit / cap)) with queries large enough that the cap bites.
     run_case(fmt, hq, hkv, d, L, cap=L + 8, seed=L % 89, softcap=50.0, q_gain=4.0)

@@ -1,8 +1,9 @@
 """The oracle's attention over block-quantised caches (the Q4_0 arm of the scalar CPU backend,
 backend/cpu/common.rs:676-850) is pinned here by an independent route: the blocks are unpacked with
 a few lines of numpy written from the format definition (quant.rs BlockQ4_0 / BlockQ4_1 / BlockQ8_0:
-x = d*(n-8), d*n+m, d*c; element i in the low nibble of byte i, element 16+i in the high nibble)
-and attended with the float64 textbook softmax attention."""
+x = d*(n-8), d*n+m, d*c; element i in the low nibble of byte i, element 16+i in the high nibble;
+BlockQ2_0: x = d*n+m, element 4i+k in bits 2k, 2k+1 of byte i) and attended with the float64
+textbook softmax attention."""
 import numpy as np
 import pytest
 
@@ -17,6 +18,10 @@ def unpack(desc, raw, n_elems):
     d = blk[:, 0:2].copy().view(np.float16).astype(np.float64)
     if desc == O.DESC_Q8_0:
         x = d * blk[:, 2:].view(np.int8).astype(np.float64)
+    elif desc == O.DESC_Q2_0:
+        codes = blk[:, 4:]
+        n = np.stack([(codes >> (2 * k)) & 3 for k in range(4)], axis=2).reshape(len(blk), 32).astype(np.float64)
+        x = d * n + blk[:, 2:4].copy().view(np.float16).astype(np.float64)
     else:
         hdr = 4 if desc == O.DESC_Q4_1 else 2
         codes = blk[:, hdr:]
@@ -28,7 +33,7 @@ def unpack(desc, raw, n_elems):
     return x.reshape(-1)[:n_elems]
 
 
-@pytest.mark.parametrize("desc", [O.DESC_Q4_0, O.DESC_Q4_1, O.DESC_Q8_0])
+@pytest.mark.parametrize("desc", [O.DESC_Q4_0, O.DESC_Q4_1, O.DESC_Q8_0, O.DESC_Q2_0])
 @pytest.mark.parametrize("head_major", [True, False])
 def test_against_numpy_unpack_and_textbook_attention(desc, head_major):
     hq, hkv, d, L, cap = 8, 2, 64, 300, 320
