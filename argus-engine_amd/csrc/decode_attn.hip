@@ -345,6 +345,7 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
   p.group = a->num_heads_q / a->num_heads_kv;
   p.len = a->cache_seq_len;
   p.kv_start = a->kv_index ? 0 : a->kv_start;
+  p.slot_bound = a->capacity;
   p.score_stride = a->score_stride;
   if (a->layout == ARGUS_HIP_HEAD_MAJOR) {
     p.row_stride = D;

@@ -308,11 +308,14 @@ struct BlockFallback {
     using F = BlockFmt<FMT>;
     const int kvh = h / p.group;
     const uint8_t *vb = (const uint8_t *)p.v + ((int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride) / 32 * F::BB;
+    const int32_t *idx = p.kv_index ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
     const float u = 1.0f / (float)p.len;
     for (int c = threadIdx.x; c < D; c += blockDim.x) {
       float acc = 0.0f;
-      for (int t = 0; t < p.len; ++t)
-        acc += u * block_elem<FMT>(vb + ((int64_t)(p.kv_start + t) * p.row_stride / 32 + c / 32) * F::BB, c % 32);
+      for (int t = 0; t < p.len; ++t) {
+        const int64_t slot = idx ? idx[t] : (p.kv_start + t);
+        acc += u * block_elem<FMT>(vb + (slot * p.row_stride / 32 + c / 32) * F::BB, c % 32);
+      }
       p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = acc;
     }
     if (p.scores) {
@@ -337,7 +340,7 @@ struct BlockShape {
   static constexpr int MAXH = (D == 256) ? 8 : 16;        // query heads per KV head (bounds the merge LDS)
 };
 
-template <int FMT, int D, int TW, bool SOFTCAP>
+template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED>
 __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
@@ -385,14 +388,47 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
   // Rows past the chunk re-read its last row (they are masked below), so every request is
   // unconditional and a tile may be asked for before it is known to exist.
   const int last = t_end - 1;
+  // Token -> cache row.  With an index list (INDEXED) the rows of the tile after next are read from
+  // the list while the next tile's blocks are requested: the K rows right behind the K requests and
+  // the V rows right behind the V requests, so that neither request waits on a load younger than
+  // the data it is about to use.
+  constexpr int NKR = (D == 64) ? 1 : TW;                               // K rows a lane addresses per iteration
+  constexpr int NVR = kStageV ? ((D == 64) ? 1 : TW) : 4 * TW;          // V rows
+  const int32_t *idx = INDEXED ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
+  int k_row[INDEXED ? NKR : 1], v_row[INDEXED ? NVR : 1];
+  auto k_tok = [&](int base, int i) { return min((D == 64) ? base + 16 * (j >> 1) + r : base + 16 * i + r, last); };
+  auto v_tok = [&](int base, int i) {
+    if constexpr (!kStageV) return min(base + 16 * (i >> 2) + 4 * j + (i & 3), last);
+    else return min((D == 64) ? base + 16 * (r >> 3) + 4 * j + (r & 3) : base + 16 * i + 4 * j + (r & 3), last);
+  };
+  auto load_idx_k = [&](int base) {
+    if constexpr (INDEXED) {
+#pragma unroll
+      for (int i = 0; i < NKR; ++i) k_row[i] = idx[k_tok(base, i)];
+    }
+  };
+  auto load_idx_v = [&](int base) {
+    if constexpr (INDEXED) {
+#pragma unroll
+      for (int i = 0; i < NVR; ++i) v_row[i] = idx[v_tok(base, i)];
+    }
+  };
+  auto k_rowof = [&](int base, int i) -> uint32_t {
+    if constexpr (INDEXED) return (uint32_t)k_row[i];
+    else return (uint32_t)k_tok(base, i);
+  };
+  auto v_rowof = [&](int base, int i) -> uint32_t {
+    if constexpr (INDEXED) return (uint32_t)v_row[i];
+    else return (uint32_t)v_tok(base, i);
+  };
   auto load_k = [&](int base) {
     if constexpr (D == 64) {
-      const uint32_t off = __umul24((uint32_t)min(base + 16 * (j >> 1) + r, last), row_bytes);
+      const uint32_t off = __umul24(k_rowof(base, 0), row_bytes);
       kblk[0] = load_block<FMT>(kb, off + (uint32_t)((j & 1) * F::BB));
     } else {
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
-        const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + r, last), row_bytes);
+        const uint32_t off = __umul24(k_rowof(base, tw), row_bytes);
 #pragma unroll
         for (int u = 0; u < KQ; ++u) kblk[tw * KQ + u] = load_block<FMT>(kb, off + (uint32_t)((4 * u + j) * F::BB));
       }
@@ -400,19 +436,19 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
   };
   auto load_v = [&](int base) {
     if constexpr (kStageV && D == 64) {
-      const uint32_t off = __umul24((uint32_t)min(base + 16 * (r >> 3) + 4 * j + (r & 3), last), row_bytes);
+      const uint32_t off = __umul24(v_rowof(base, 0), row_bytes);
       vblk_raw[0] = load_block<FMT>(vb, off + (uint32_t)(((r >> 2) & 1) * F::BB));
     } else {
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
         if constexpr (kStageV) {
-          const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + (r & 3), last), row_bytes);
+          const uint32_t off = __umul24(v_rowof(base, tw), row_bytes);
 #pragma unroll
           for (int sg = 0; sg < VSEG; ++sg) vblk_raw[tw * VSEG + sg] = load_block<FMT>(vb, off + (uint32_t)((4 * sg + (r >> 2)) * F::BB));
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const uint32_t off = __umul24((uint32_t)min(base + 16 * tw + 4 * j + e, last), row_bytes);
+            const uint32_t off = __umul24(v_rowof(base, 4 * tw + e), row_bytes);
 #pragma unroll
             for (int sg = 0; sg < VSEG; ++sg) {
               if constexpr (D == 64) {  // q8_0: the lane's half of the piece is one dword
@@ -429,8 +465,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     }
   };
   const int base0 = t_begin + __builtin_amdgcn_readfirstlane(wave) * TILE;
+  load_idx_k(base0);
+  load_idx_v(base0);
   load_k(base0);
+  load_idx_k(base0 + kWaves * TILE);
   load_v(base0);
+  load_idx_v(base0 + kWaves * TILE);
   __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the query's
 
   // ---- Q operand: lane (j, h = r), block kk: the elements slot_elem(j, 0..7), log2 domain, hi + lo
@@ -551,6 +591,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     // tile (register data flow of that build read correct; cause not identified).
     __builtin_amdgcn_sched_barrier(0);
     load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
+    load_idx_k(base + 2 * kWaves * TILE);
     if constexpr (SOFTCAP) {
       // cap * tanh(logit / cap) on the natural-unit logit (flash_attn_f32_f16.cl:563-565), back to log2 units
 #pragma unroll
@@ -687,6 +728,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         }
       }
     load_v(base + kWaves * TILE);
+    load_idx_v(base + 2 * kWaves * TILE);
   }
 
   if constexpr (kHdrTerm) {
@@ -750,7 +792,7 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   static int wgs_per_cu = 0;  // per instantiation; single inference thread
   if (wgs_per_cu == 0) {
     int n = 0;
-    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_blocks_kernel<FMT, D, TW, false>, 64 * kWaves, 0));
+    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_blocks_kernel<FMT, D, TW, false, false>, 64 * kWaves, 0));
     wgs_per_cu = std::max(1, n);
   }
   choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu);
@@ -763,8 +805,12 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   {
     KernelTimer timer(ctx, stream);
-    if (p.softcap > 0.0f) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true>), dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
-    else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false>), dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
+    const dim3 grid(p.nsplit, p.n_heads_kv, batch), block(64 * kWaves);
+    const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
+    if (cap && indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, true>), grid, block, 0, stream, p);
+    else if (cap) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, false>), grid, block, 0, stream, p);
+    else if (indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, false>), grid, block, 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<BlockFallback<FMT>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -784,16 +830,13 @@ int launch_blocks_dim(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hip
 }  // namespace
 
 int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtype, int batch, hipStream_t stream) {
-  if (p.kv_index)
-    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED,
-                      "attention_gen: block-quantised caches take no index list; decode them with "
-                      "argus_hip_kv_decode_descriptor and attend the F16 copy");
   if (p.group > ((D == 256) ? 8 : 16))
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: %d query heads per KV head on a block-quantised cache", p.group);
   if ((p.row_stride % 32) || (p.head_stride % 32) || (p.kv_bs % 32))
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: block-quantised cache strides must be whole 32-element blocks");
   // rows are addressed as (row index, 24 bits) x (row bytes, 24 bits) -> 32-bit byte offset
-  if (p.len >= (1 << 24) || p.row_stride / 32 * 34 >= (1 << 24) || (int64_t)p.len * (p.row_stride / 32 * 34) > 0xffffffffll)
+  const int64_t rows = p.kv_index ? p.slot_bound : p.len;  // an index list may name any slot of the cache
+  if (rows >= (1 << 24) || p.row_stride / 32 * 34 >= (1 << 24) || rows * (p.row_stride / 32 * 34) > 0xffffffffll)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: block-quantised head slab beyond 4 GiB");
   switch (kv_dtype) {
     case ARGUS_HIP_Q4_0: return launch_blocks_dim<kFmtQ4_0>(ctx, p, D, batch, stream);

@@ -25,6 +25,7 @@ struct DecodeParams {
   int64_t q_bs, out_bs, kv_bs, score_bs, index_bs;
   float scale, softcap;
   int32_t direct;  // nsplit == 1 and no scores: first pass writes `out` itself
+  int32_t slot_bound;  // slots an index list may name (the cache capacity)
 };
 
 // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1); the argument is clamped where

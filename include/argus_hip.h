@@ -113,9 +113,9 @@ int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream);
  * (common.rs:676-850, rows dequantised on the fly) and the in-kernel form of the `--kv-format`
  * attention whose reference floor decodes the whole cache to F32 first
  * (engine/src/kv/standard_format.rs:538-643).  Rows are head_dim/32 blocks; capacity, kv_start and
- * the strides stay in elements (multiples of 32).  softcap applies as for F16 caches.  No kv_index
- * (ARGUS_HIP_ERR_UNSUPPORTED: decode with argus_hip_kv_decode_descriptor and attend the F16 copy);
- * up to 16 query heads per KV head (8 at head_dim 256). */
+ * the strides stay in elements (multiples of 32).  softcap and kv_index apply as for F16 caches;
+ * up to 16 query heads per KV head (8 at head_dim 256), else ARGUS_HIP_ERR_UNSUPPORTED (decode with
+ * argus_hip_kv_decode_descriptor and attend the F16 copy). */
 typedef struct argus_hip_attention_gen_args {
   void *stream;
   const float *q;       /* [batch, num_heads_q, head_dim] F32 */

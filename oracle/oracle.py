@@ -405,7 +405,7 @@ def encode_via_descriptor(desc, src):
 
 
 def attention_gen_blocks(q, k_raw, v_raw, desc, n_heads_kv, cache_seq_len, capacity, head_major=True,
-                         scores=False, scores_stride=None, softcap=0.0):
+                         scores=False, scores_stride=None, softcap=0.0, kv_index=None):
     """Backend::attention_gen over a block-quantised cache: the Q4_0 arm of the scalar CPU backend
     (backend/cpu/common.rs:676-850: each K / V row is dequantised, then the F32 algorithm with its
     guards runs), which is also what the `--kv-format` floor computes after decoding the whole cache
@@ -417,4 +417,4 @@ def attention_gen_blocks(q, k_raw, v_raw, desc, n_heads_kv, cache_seq_len, capac
     k = decode_via_descriptor(desc, k_raw, rows * d)
     v = decode_via_descriptor(desc, v_raw, rows * d)
     return attention_gen(q, k, v, n_heads_kv, cache_seq_len, capacity, head_major=head_major,
-                         scores=scores, scores_stride=scores_stride, impl="scalar", softcap=softcap)
+                         scores=scores, scores_stride=scores_stride, impl="scalar", softcap=softcap, kv_index=kv_index)
