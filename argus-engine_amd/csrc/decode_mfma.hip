@@ -66,7 +66,7 @@ struct VPiece<4> { using type = half4_t; };
 // less data per microsecond: 27.4 us against 26.4 us on one 32K-token sequence.)
 constexpr int kWaves = 4;
 
-template <int D, int TW, bool SOFTCAP>
+template <int D, int TW, bool SOFTCAP, bool INDEXED>
 __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodeParams p) {
   using SH = MfmaShape<D>;
   constexpr int KK = SH::KK, VC = SH::VC, VSEG = SH::VSEG, NACC = SH::NACC;
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
   // compiler then waits for exactly the ones it needs) and a tile may be requested before it is
   // known to exist.  Offsets: a per-lane constant plus the wave-uniform first row of the tile.
   const int64_t rs = p.row_stride;
-  const uint32_t slab_bytes = (uint32_t)((int64_t)(p.kv_start + t_end) * rs * 2);
+  const uint32_t slab_bytes = (uint32_t)((int64_t)(INDEXED ? p.slot_bound : p.kv_start + t_end) * rs * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)kb, 0, slab_bytes, kBufferFlags);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)vb, 0, slab_bytes, kBufferFlags);
   const uint32_t k_lane = (uint32_t)(((int64_t)(p.kv_start + r) * rs + 8 * j) * 2);
@@ -99,13 +99,34 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
   const uint32_t row_bytes = (uint32_t)(rs * 2);
   half8_t kr[TW][KK];
   vpiece_t vr[TW][VSEG][4];
+  // With an index list (INDEXED: token t lives in slot kv_index[t]) the slots of the tile after next
+  // are read from the list right behind the requests for the next tile, K slots behind the K
+  // requests and V slots behind the V requests, so neither request waits on a load younger than
+  // the data about to be used.  Tokens past the chunk re-read its last slot and are masked below.
+  const int32_t *idx = INDEXED ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
+  const int last = t_end - 1;
+  int k_slot[INDEXED ? TW : 1], v_slot[INDEXED ? 4 * TW : 1];
+  auto load_idx_k = [&](int base) {
+    if constexpr (INDEXED) {
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) k_slot[tw] = idx[min(base + 16 * tw + r, last)];
+    }
+  };
+  auto load_idx_v = [&](int base) {
+    if constexpr (INDEXED) {
+#pragma unroll
+      for (int i = 0; i < 4 * TW; ++i) v_slot[i] = idx[min(base + 16 * (i >> 2) + 4 * j + (i & 3), last)];
+    }
+  };
   auto load_k = [&](int base) {  // TW tiles of 16 tokens starting at token `base`
     const uint32_t tile = (uint32_t)base * row_bytes;
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-        kr[tw][kk] = buffer_load_stream<half8_t>(k_rsrc, k_lane + 16 * tw * row_bytes + 64 * kk, tile);
+      for (int kk = 0; kk < KK; ++kk) {
+        if constexpr (INDEXED) kr[tw][kk] = buffer_load_stream<half8_t>(k_rsrc, __umul24((uint32_t)k_slot[tw], row_bytes) + 16 * j + 64 * kk, 0u);
+        else kr[tw][kk] = buffer_load_stream<half8_t>(k_rsrc, k_lane + 16 * tw * row_bytes + 64 * kk, tile);
+      }
   };
   auto load_v = [&](int base) {
     const uint32_t tile = (uint32_t)base * row_bytes;
@@ -114,13 +135,21 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
 #pragma unroll
       for (int e = 0; e < 4; ++e)
 #pragma unroll
-        for (int sg = 0; sg < VSEG; ++sg)
-          vr[tw][sg][e] = buffer_load_stream<vpiece_t>(v_rsrc, v_lane + (16 * tw + e) * row_bytes + 32 * VC * sg, tile);
+        for (int sg = 0; sg < VSEG; ++sg) {
+          if constexpr (INDEXED)
+            vr[tw][sg][e] = buffer_load_stream<vpiece_t>(v_rsrc, __umul24((uint32_t)v_slot[4 * tw + e], row_bytes) + 2 * VC * r + 32 * VC * sg, 0u);
+          else
+            vr[tw][sg][e] = buffer_load_stream<vpiece_t>(v_rsrc, v_lane + (16 * tw + e) * row_bytes + 32 * VC * sg, tile);
+        }
   };
   // The first tile is requested before the query is prepared, so both arrive together.
   const int base0 = t_begin + __builtin_amdgcn_readfirstlane(wave) * TILE;
+  load_idx_k(base0);
+  load_idx_v(base0);
   load_k(base0);
+  load_idx_k(base0 + kWaves * TILE);
   load_v(base0);
+  load_idx_v(base0 + kWaves * TILE);
   __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the query's
 
   // ---- Q operand: lane (j, h = r) holds chunk 4kk + j of head h, scaled to the log2 domain ------
@@ -165,6 +194,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     }
     // The K registers are free again: request the wave's next tile (past the chunk: zeros, no traffic).
     load_k(base + kWaves * TILE);
+    load_idx_k(base + 2 * kWaves * TILE);
     const bool full = base + TILE <= t_end;
     float mt = kNegInf;
 #pragma unroll
@@ -235,6 +265,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
           o_acc[sg * VC + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * VC + c], 0, 0, 0);
         }
     load_v(base + kWaves * TILE);
+    load_idx_v(base + 2 * kWaves * TILE);
   }
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
@@ -287,7 +318,7 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   static int wgs_per_cu = 0;  // per head_dim instantiation; single inference thread
   if (wgs_per_cu == 0) {
     int n = 0;
-    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_mfma_kernel<D, TW, false>, 64 * kWaves, 0));
+    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves, 0));
     wgs_per_cu = std::max(1, n);
   }
   choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu);
@@ -301,8 +332,12 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   {
     KernelTimer timer(ctx, stream);
-    if (p.softcap > 0.0f) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true>), dim3(nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
-    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false>), dim3(nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), 0, stream, p);
+    const dim3 grid(nsplit, p.n_heads_kv, batch), block(64 * kWaves);
+    const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
+    if (cap && indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, true>), grid, block, 0, stream, p);
+    else if (cap) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, false>), grid, block, 0, stream, p);
+    else if (indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, false>), grid, block, 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -313,9 +348,12 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
 }  // namespace
 
 bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
-  if (kv_dtype != ARGUS_HIP_F16 || p.kv_index || p.len < 64) return false;
-  // rows are addressed with 32-bit byte offsets from the head's first row, a few tiles past the end
-  if (((int64_t)p.kv_start + p.len + 1024) * p.row_stride * 2 > 0x7fffffffll) return false;
+  if (kv_dtype != ARGUS_HIP_F16 || p.len < 64) return false;
+  // rows are addressed with 32-bit byte offsets from the head's first row, a few tiles past the end;
+  // an index list may name any slot of the cache (slot x row bytes is a 24-bit multiply)
+  const int64_t rows = p.kv_index ? p.slot_bound : (int64_t)p.kv_start + p.len;
+  if ((rows + 1024) * p.row_stride * 2 > 0x7fffffffll) return false;
+  if (p.kv_index && (rows >= (1 << 24) || p.row_stride * 2 >= (1 << 24))) return false;
   if (D == 64 || D == 128) return p.group <= 16;
   // head_dim 256: one 64-row tile per workgroup costs more set-up (Q split over 256 channels) than it
   // saves; measured against the vector-ALU kernel it only pays for long rows and wider groups

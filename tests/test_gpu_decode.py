@@ -209,6 +209,35 @@ def test_calls_without_scores_batch_and_fallback():
             check_attention_out(got[i], O.attention_gen(q[i], k[i], v[i], hkv, L, cap), "seq %d rep %d" % (i, rep))
 
 
+@pytest.mark.parametrize("hq,hkv,d,L,cap", [(32, 8, 128, 3000, 8192), (14, 2, 64, 1000, 1024), (8, 2, 128, 20000, 40000),
+                                           (32, 4, 256, 9000, 12000), (5, 1, 64, 77, 300)])
+def test_index_list_on_the_matrix_core_path(hq, hkv, d, L, cap):
+    # Post-eviction addressing on F16 caches: token t lives in slot kv_index[t] (shuffled here), the
+    # result is the attention over the gathered rows; with scores, without, and with a soft-cap.
+    q = normal((hq, d), L)
+    k = f16(normal((hkv, cap, d), L + 1))
+    v = f16(normal((hkv, cap, d), L + 2))
+    idx = np.random.default_rng(L).choice(cap, L, replace=False).astype(np.int32)
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, kv_index=dev(idx))
+    ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, kv_index=idx)
+    check_attention_out(got, ref, "indexed")
+    check_scores(sc, p, "indexed")
+    check_attention_out(run_decode(q, k, v, hkv, L, cap, kv_index=dev(idx)), ref, "indexed, no scores")
+    got = run_decode(q * 3.0, k, v, hkv, L, cap, kv_index=dev(idx), softcap=8.0)
+    check_attention_out(got, O.attention_gen(q * 3.0, k, v, hkv, L, cap, kv_index=idx, softcap=8.0), "indexed + soft-cap")
+
+
+def test_index_list_per_sequence_in_a_batch():
+    b, hq, hkv, d, L, cap = 4, 16, 4, 128, 1500, 2048
+    q = normal((b, hq, d), 1)
+    k = f16(normal((b, hkv, cap, d), 2))
+    v = f16(normal((b, hkv, cap, d), 3))
+    idx = np.stack([np.random.default_rng(10 + i).choice(cap, L, replace=False) for i in range(b)]).astype(np.int32)
+    got = run_decode(q, k, v, hkv, L, cap, batch=b, kv_batch_stride=hkv * cap * d, kv_index=dev(idx), index_batch_stride=L)
+    for i in range(b):
+        check_attention_out(got[i], O.attention_gen(q[i], k[i], v[i], hkv, L, cap, kv_index=idx[i]), "seq %d" % i)
+
+
 def test_config1_qwen_shape():
     # BASELINE config 1: Hq14 Hkv2 d64 L1024, f32 N(0,1) -> F16 KV, scale 1/8.
     hq, hkv, d, L = 14, 2, 64, 1024
