@@ -175,7 +175,7 @@ constexpr float kCodeUnit = 16777216.0f;  // a raw code field n is the half n * 
 // Query heads per KV head the kernel takes (bounds the merge area).
 constexpr int kMaxGroup = 8;
 
-template <int BITS, int D, int GT>
+template <int BITS, int D, int GT, bool SOFTCAP>
 __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(const KiviParams kp) {
   constexpr int BB = 4 + 32 * BITS / 8;  // block bytes
   constexpr int KK = D / 32;             // 32-channel slices == V blocks per token
@@ -238,12 +238,19 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 
   // Online-softmax step for one unit.  In: s[w][i] = logit (log2 units) of token 8j + 2i + w for
   // head r.  Out: pa[e] = probability of token 8j + e relative to the running maximum.
+  const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
   auto softmax_step = [&](float4_t(&s)[2], int tok0, int n_valid) -> half8_t {
     float mt = kNegInf;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
+        if constexpr (SOFTCAP) {
+          // cap * tanh(logit / cap) on the natural-unit logit, back to log2 units; NaN stays NaN
+          const float sv = s[w][i];
+          const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * 1.4426950408889634f;
+          s[w][i] = (sv != sv) ? sv : capped;
+        }
         if (8 * j + 2 * i + w >= n_valid) s[w][i] = kNegInf;
         mt = fmaxf(mt, s[w][i]);  // a NaN logit propagates (the reference kernels have no guard)
       }
@@ -554,8 +561,8 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   // the occupancy the unit loop needs to hide its LDS and HBM latency.
   static const int wgs_per_cu = [] {
     int n4 = 0, n8 = 0;
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n4, kivi_mfma_kernel<BITS, D, 4>, 256, 0);
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n8, kivi_mfma_kernel<BITS, D, 8>, 256, 0);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n4, kivi_mfma_kernel<BITS, D, 4, false>, 256, 0);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n8, kivi_mfma_kernel<BITS, D, 8, false>, 256, 0);
     return std::max(1, std::min(n4, n8));
   }();
   const int slots = ctx->compute_units * wgs_per_cu;
@@ -574,8 +581,11 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   const dim3 grid(nsplit, p.n_heads_kv, batch);
   {
     KernelTimer timer(ctx, stream);
-    if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4>), grid, dim3(256), 0, stream, kp);
-    else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8>), grid, dim3(256), 0, stream, kp);
+    const bool cap = p.softcap > 0.0f;
+    if (p.group <= 4 && cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, true>), grid, dim3(256), 0, stream, kp);
+    else if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, false>), grid, dim3(256), 0, stream, kp);
+    else if (cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, true>), grid, dim3(256), 0, stream, kp);
+    else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false>), grid, dim3(256), 0, stream, kp);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<NoFallback, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
@@ -597,7 +607,7 @@ int launch_dim(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream
 bool kivi_mfma_supported(const KiviParams &kp) {
   const DecodeParams &p = kp.d;
   if (kp.head_dim != 64 && kp.head_dim != 128 && kp.head_dim != 256) return false;
-  if (p.group > kMaxGroup || p.softcap > 0.0f) return false;
+  if (p.group > kMaxGroup) return false;
   // tiles are copied as 16-byte vectors
   if ((((uintptr_t)kp.qk | (uintptr_t)kp.qv) & 15) || (kp.qk_bs & 15) || (kp.qv_bs & 15)) return false;
   // residual rows are read as 16-byte vectors

@@ -109,6 +109,26 @@ def test_kivi_attention_vs_oracle(bits, hq, hkv, d, R, n):
     check_attention_out(out, r64)
 
 
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("hq,hkv,d,R,n", [(8, 4, 256, 128, 900), (32, 8, 128, 128, 700), (14, 2, 64, 32, 333)])
+def test_kivi_soft_cap(bits, hq, hkv, d, R, n):
+    # The logit soft-cap (cap * tanh(logit / cap)) has no counterpart in the reference's KIVI kernels;
+    # it is checked against the float64 textbook attention over the dequantised view, with queries
+    # large enough that the cap bites.
+    rng = np.random.default_rng(bits * 100 + n)
+    k = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    q = (3.0 * rng.standard_normal((hq, d))).astype(np.float32)
+    c = O.kivi_build(k, v, R, bits)
+    scale = 1.0 / np.sqrt(d)
+    ak, av = O.kivi_assemble_view(c)
+    for cap in (50.0, 4.0):
+        out, sc = run_kivi(q, c, scale, scores="dev", softcap=cap)
+        r64, p64 = T.decode_attention(q, ak.transpose(1, 0, 2), av.transpose(1, 0, 2), hkv, n, softcap=cap, scale=scale)
+        check_attention_out(out, r64, "cap %g" % cap)
+        check_scores(sc, p64, "cap %g" % cap)
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 def test_config4_llama8b_kivi(bits):
     # BASELINE config 4: Hq32 Hkv8 d128, 8192 appended tokens, res_cap 128 -> q_tokens 8064 +
