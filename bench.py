@@ -238,6 +238,83 @@ def bench_prefill(ctx, steps, warmup, hq=32, hkv=8, d=64, s=2048, batch=1, f16_i
                 tflops_wall=round(flops / wall / 1e12, 1))
 
 
+def bench_aux(ctx, steps, warmup):
+    """The data-movement kernels either side of the attention calls, each at a size of the BASELINE
+    configurations: microseconds per call (torch events on the current stream, `steps` calls back to
+    back) and the rate on the bytes the call has to move."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(3)
+    res = {}
+
+    def timed(name, fn, nbytes, note):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / steps
+        res[name] = {"us_per_call": round(us, 2), "bytes": nbytes, "gbps": round(nbytes / us / 1e3, 1),
+                     "hbm_frac": round(nbytes / us / 1e3 / 8000.0, 4), "note": note}
+
+    # (a-4) H2O score reduce: 32 layers x 32 heads of probabilities over 32768 positions
+    nl, hq, hkv, L = 32, 32, 8, 32768
+    scores = torch.rand((nl, hq, L), generator=g, device="cuda")
+    imp = torch.zeros(L, device="cuda")
+    himp = torch.zeros(hkv * L, device="cuda")
+    lf = torch.zeros(nl * L, device="cuda")
+    spin_up(lambda: ctx.score_reduce(scores, imp, himp, 0.9, nl, hq, hkv, L, L, L))
+    timed("score_reduce_L32768_32x32", lambda: ctx.score_reduce(scores, imp, himp, 0.9, nl, hq, hkv, L, L, L),
+          scores.numel() * 4 + 2 * (imp.numel() + himp.numel()) * 4, "fused importance + per-KV-head importance")
+    timed("score_reduce_per_layer_L32768_32x32", lambda: ctx.score_reduce_per_layer(scores, lf, 0.9, nl, hq, hkv, L, L, L),
+          scores.numel() * 4 + 2 * lf.numel() * 4, "per-layer importance")
+    del scores
+
+    # (f-1) KV scatter of a 2048-token prefill chunk, F32 rows -> F16 HeadMajor cache
+    hkv, d, cap, sl = 8, 128, 32768, 2048
+    ks = torch.randn((sl, hkv, d), generator=g, device="cuda")
+    vs = torch.randn((sl, hkv, d), generator=g, device="cuda")
+    kd = torch.zeros((hkv, cap, d), device="cuda", dtype=torch.float16)
+    vd = torch.zeros_like(kd)
+    timed("kv_scatter_f32_to_f16_2048_tokens", lambda: ctx.kv_scatter(ks, vs, kd, vd, hkv, d, cap, 100, seq_len=sl),
+          2 * sl * hkv * d * (4 + 2), "K and V rows of one layer")
+    k1, v1 = ks[:1].contiguous(), vs[:1].contiguous()
+    timed("kv_scatter_f32_to_f16_1_token", lambda: ctx.kv_scatter(k1, v1, kd, vd, hkv, d, cap, 100),
+          2 * hkv * d * 6, "decode step: launch latency")
+
+    # (f-4) descriptor codec over one layer's cache of 32768 tokens (8 KV heads x 128)
+    import oracle as O
+    n = 32768 * hkv * d
+    x = torch.randn(n, generator=g, device="cuda")
+    for name, desc, bb in (("q4_0", O.DESC_Q4_0, 18), ("q2_0", O.DESC_Q2_0, 12)):
+        blocks = torch.zeros(n // 32 * bb, dtype=torch.uint8, device="cuda")
+        f16 = torch.zeros(n, dtype=torch.float16, device="cuda")
+        timed("kv_encode_descriptor_%s_32768_tokens" % name, lambda: ctx.kv_encode_descriptor(desc, x, blocks, n),
+              n * 4 + blocks.numel(), "F32 rows -> blocks")
+        timed("kv_decode_descriptor_%s_to_f16_32768_tokens" % name, lambda: ctx.kv_decode_descriptor(desc, blocks, f16, n),
+              blocks.numel() + n * 2, "blocks -> F16 rows (the floor's decode pass)")
+
+    # (f-2) KIVI flush of a full 128-token residual, and the F16 view of one flush (config-4 shape)
+    R, hkv, d = 128, 8, 128
+    for bits in (2, 4, 8):
+        bb = 4 + 32 * bits // 8
+        res_k = torch.randn((hkv, R, d), generator=g, device="cuda")
+        res_v = torch.randn((hkv, R, d), generator=g, device="cuda")
+        nblk = hkv * R * d // 32
+        qk = torch.zeros(nblk * bb, dtype=torch.uint8, device="cuda")
+        qv = torch.zeros(nblk * bb, dtype=torch.uint8, device="cuda")
+        timed("kivi_flush_q%d_128_tokens" % bits, lambda: ctx.quant_flush(res_k, res_v, qk, qv, hkv, R, d, R, 0, 0, bits),
+              2 * hkv * R * d * 4 + 2 * nblk * bb, "quantise K and V residuals (launch latency: 1 MB)")
+        view = torch.zeros((R + 2, hkv, d), device="cuda", dtype=torch.float16)
+        timed("kivi_dequant_flush_q%d_key_128_tokens" % bits,
+              lambda: ctx.quant_dequant_flush(qk, view, hkv, d, R // 32, 0, 0, bits, True),
+              nblk * bb + hkv * R * d * 2, "blocks -> F16 view rows")
+    return res
+
+
 def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
     """Restated CpuBackendAVX2::attention_gen on one sequence of the primary workload."""
     import numpy as np
@@ -279,7 +356,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
                     choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1",
-                             "q8_0", "copy_calib"],
+                             "q8_0", "copy_calib", "aux"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -305,6 +382,8 @@ def main():
                 dst.copy_(src)
             torch.cuda.synchronize()
             res = {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}
+        elif w == "aux":
+            res = bench_aux(ctx, args.steps, args.warmup)
         elif w == "decode_b1":
             res = bench_decode(ctx, 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=4)
         elif w == "prefill":
