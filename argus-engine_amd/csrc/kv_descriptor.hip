@@ -6,8 +6,11 @@
 // KVLayoutDesc { block_elems, bits, scale_layout, packing } (argus-extension-api lib.rs:1111-1159).
 // Results are bit-identical to the CPU functions: products of a small integer and an f16 scale are
 // exact in f32, the encoders use the same correctly rounded divide / reciprocal / round-half-away.
-// One thread per block; blocks are only 2-byte aligned (18 / 34 bytes), so they are read and written
-// as 16-bit units.
+// Blocks are only 2-byte aligned (12 / 18 / 20 / 34 bytes), so they are read and written as 16-bit
+// units.  32-element blocks (every named format) take four threads per block, eight elements each:
+// a thread then stores or loads 16 or 32 contiguous bytes of the row and the wave's accesses are
+// dense (one thread per block wrote 2-byte elements 64 bytes apart: 0.5 TB/s).  Other block sizes
+// keep the one-thread-per-block kernels.
 #include "argus_hip_internal.hpp"
 
 namespace {
@@ -66,6 +69,54 @@ __global__ __launch_bounds__(256) void desc_decode_kernel(const DescParams p, co
   }
 }
 
+typedef uint32_t u32_a2 __attribute__((aligned(2)));  // dword reads at 2-byte boundaries
+
+// 32-element blocks, four threads per block: thread q decodes elements 8q .. 8q+7.
+template <typename OUT_T>
+__global__ __launch_bounds__(256) void desc_decode32_kernel(const DescParams p, const uint16_t *src, OUT_T *dst) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t bi = gid >> 2;
+  const int q = (int)(gid & 3);
+  if (bi >= p.n_blocks) return;
+  const uint16_t *blk = src + bi * (p.block_bytes / 2);
+  const float scale = half_bits_to_float(blk[0]);
+  const bool has_min = p.scale_layout == kScaleF16Min;
+  const float mn = has_min ? half_bits_to_float(blk[1]) : 0.0f;
+  const uint16_t *qw = blk + (has_min ? 2 : 1);
+  float r[8];
+  if (p.packing == kNibble) {
+    // element i < 16: low nibble of byte i; element 16 + i: high nibble of byte i
+    const int zp = 1 << (p.bits - 1), sh = (q >> 1) * 4;
+    const u32_a2 *cw = (const u32_a2 *)(qw + 4 * (q & 1));  // the thread's 8 code bytes as two dwords
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t w = cw[k];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int code = (int)((w >> (8 * e + sh)) & 0x0fu);
+        r[4 * k + e] = has_min ? __fadd_rn(__fmul_rn((float)code, scale), mn) : __fmul_rn((float)(code - zp), scale);
+      }
+    }
+  } else if (p.packing == kByte) {
+    const u32_a2 *cw = (const u32_a2 *)(qw + 4 * q);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t w = cw[k];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[4 * k + e] = __fmul_rn((float)(int)(int8_t)((w >> (8 * e)) & 0xffu), scale);
+    }
+  } else {
+    const uint32_t w = qw[q];  // bytes 2q, 2q+1: elements 8q .. 8q+7, two bits each
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = __fadd_rn(__fmul_rn((float)((w >> (2 * e)) & 3u), scale), mn);
+  }
+  typedef OUT_T out8_t __attribute__((ext_vector_type(8)));
+  out8_t o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = store_cast<OUT_T>(r[e]);
+  *(out8_t *)(dst + bi * 32 + 8 * q) = o;
+}
+
 __device__ __forceinline__ uint16_t float_to_half_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
 
 __global__ __launch_bounds__(256) void desc_encode_kernel(const DescParams p, const float *src, uint16_t *dst) {
@@ -121,6 +172,78 @@ __global__ __launch_bounds__(256) void desc_encode_kernel(const DescParams p, co
   }
 }
 
+// 32-element blocks, four threads per block: thread q quantises elements 8q .. 8q+7; the block's
+// extrema and, for nibble packing, the partner's codes (byte i = element i | element 16 + i << 4)
+// travel between the four lanes by shuffles.
+__global__ __launch_bounds__(256) void desc_encode32_kernel(const DescParams p, const float *src, uint16_t *dst) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t bi = gid >> 2;
+  const int q = (int)(gid & 3);
+  if (bi >= p.n_blocks) return;  // the four lanes of a block leave together
+  float s[8];
+  {
+    const float4_t a = *(const float4_t *)(src + bi * 32 + 8 * q), b = *(const float4_t *)(src + bi * 32 + 8 * q + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s[e] = a[e];
+      s[4 + e] = b[e];
+    }
+  }
+  uint16_t *blk = dst + bi * (p.block_bytes / 2);
+  if (p.packing == kNibble) {
+    const float qmax = (float)((1 << (p.bits - 1)) - 1), qmin = -(float)(1 << (p.bits - 1));
+    const int zp = 1 << (p.bits - 1);
+    float max_abs = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) max_abs = fmaxf(max_abs, fabsf(s[e]));
+    max_abs = fmaxf(max_abs, __shfl_xor(max_abs, 1, 64));
+    max_abs = fmaxf(max_abs, __shfl_xor(max_abs, 2, 64));
+    const float d = __fdiv_rn(max_abs, qmax);
+    const float id = d == 0.0f ? 0.0f : __fdiv_rn(1.0f, d);
+    uint32_t mine = 0;  // eight 4-bit codes
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int v = (int)fminf(fmaxf(roundf(__fmul_rn(s[e], id)), qmin), qmax);
+      mine |= (uint32_t)((v + zp) & 0x0f) << (4 * e);
+    }
+    const uint32_t theirs = (uint32_t)__shfl_xor((int)mine, 2, 64);  // lanes 0, 1 receive elements 16 + ...
+    if (q < 2) {
+      if (q == 0) blk[0] = float_to_half_bits(d);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t b0 = ((mine >> (8 * k)) & 0x0fu) | (((theirs >> (8 * k)) & 0x0fu) << 4);
+        const uint32_t b1 = ((mine >> (8 * k + 4)) & 0x0fu) | (((theirs >> (8 * k + 4)) & 0x0fu) << 4);
+        blk[1 + 4 * q + k] = (uint16_t)(b0 | (b1 << 8));
+      }
+    }
+  } else {
+    const float qmax = 3.0f;  // quad packing is 2-bit
+    float mn = __builtin_huge_valf(), mx = -__builtin_huge_valf();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      mn = fminf(mn, s[e]);
+      mx = fmaxf(mx, s[e]);
+    }
+    mn = fminf(mn, __shfl_xor(mn, 1, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+    mn = fminf(mn, __shfl_xor(mn, 2, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+    const float d = __fdiv_rn(__fsub_rn(mx, mn), qmax);
+    const float id = d == 0.0f ? 0.0f : __fdiv_rn(1.0f, d);
+    uint32_t w = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t qv = (uint32_t)fminf(fmaxf(roundf(__fmul_rn(__fsub_rn(s[e], mn), id)), 0.0f), qmax);
+      w |= qv << (2 * e);
+    }
+    if (q == 0) {
+      blk[0] = float_to_half_bits(d);
+      blk[1] = float_to_half_bits(mn);
+    }
+    blk[2 + q] = (uint16_t)w;
+  }
+}
+
 int check_desc(argus_hip_ctx *ctx, const argus_hip_kv_layout_desc *d, DescParams &p, const char *what) {
   int q;
   switch (d->packing) {
@@ -159,11 +282,15 @@ ARGUS_API int argus_hip_kv_decode_descriptor(argus_hip_ctx *ctx, void *stream, c
   if (n_elems == 0) return ARGUS_HIP_OK;
   if (!src || !dst || ((uintptr_t)src & 1)) return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "kv_decode_descriptor: null or odd buffer");
   p.n_blocks = n_elems / p.block_elems;
-  const dim3 grid((unsigned)((p.n_blocks + 255) / 256));
-  if (dst_dtype == ARGUS_HIP_F16)
-    hipLaunchKernelGGL(desc_decode_kernel<_Float16>, grid, dim3(256), 0, (hipStream_t)stream, p, (const uint16_t *)src, (_Float16 *)dst);
-  else
-    hipLaunchKernelGGL(desc_decode_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, p, (const uint16_t *)src, (float *)dst);
+  const bool fast = p.block_elems == 32 && ((uintptr_t)dst & 15) == 0 && p.n_blocks < (1ll << 37);
+  const dim3 grid((unsigned)(((fast ? 4 : 1) * p.n_blocks + 255) / 256));
+  if (dst_dtype == ARGUS_HIP_F16) {
+    if (fast) hipLaunchKernelGGL(desc_decode32_kernel<_Float16>, grid, dim3(256), 0, (hipStream_t)stream, p, (const uint16_t *)src, (_Float16 *)dst);
+    else hipLaunchKernelGGL(desc_decode_kernel<_Float16>, grid, dim3(256), 0, (hipStream_t)stream, p, (const uint16_t *)src, (_Float16 *)dst);
+  } else {
+    if (fast) hipLaunchKernelGGL(desc_decode32_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, p, (const uint16_t *)src, (float *)dst);
+    else hipLaunchKernelGGL(desc_decode_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, p, (const uint16_t *)src, (float *)dst);
+  }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
 }
@@ -185,8 +312,12 @@ ARGUS_API int argus_hip_kv_encode_descriptor(argus_hip_ctx *ctx, void *stream, c
   if (!src || !dst || ((uintptr_t)dst & 1) || ((uintptr_t)src & 3))
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "kv_encode_descriptor: null or misaligned buffer");
   p.n_blocks = n_elems / p.block_elems;
-  hipLaunchKernelGGL(desc_encode_kernel, dim3((unsigned)((p.n_blocks + 255) / 256)), dim3(256), 0, (hipStream_t)stream, p,
-                     (const float *)src, (uint16_t *)dst);
+  if (p.block_elems == 32 && ((uintptr_t)src & 15) == 0 && p.n_blocks < (1ll << 37))
+    hipLaunchKernelGGL(desc_encode32_kernel, dim3((unsigned)((4 * p.n_blocks + 255) / 256)), dim3(256), 0, (hipStream_t)stream, p,
+                       (const float *)src, (uint16_t *)dst);
+  else
+    hipLaunchKernelGGL(desc_encode_kernel, dim3((unsigned)((p.n_blocks + 255) / 256)), dim3(256), 0, (hipStream_t)stream, p,
+                       (const float *)src, (uint16_t *)dst);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
 }
