@@ -312,6 +312,17 @@ def bench_aux(ctx, steps, warmup):
         timed("kivi_dequant_flush_q%d_key_128_tokens" % bits,
               lambda: ctx.quant_dequant_flush(qk, view, hkv, d, R // 32, 0, 0, bits, True),
               nblk * bb + hkv * R * d * 2, "blocks -> F16 view rows")
+    # (a-6) PFA side channel: probabilities of the trailing 32 query rows of a 2048-token prefill chunk
+    # over a 8192-token prefix, 32 heads, F16 HeadMajor K
+    nq, nkv, d, sl, prefix, qwin = 32, 8, 128, 2048, 8192, 32
+    q = torch.randn((sl, nq, d), generator=g, device="cuda")
+    k = torch.randn((nkv, prefix, d), generator=g, device="cuda").half()
+    sum_out = torch.zeros((nq, prefix), device="cuda")
+    per_row = torch.zeros((qwin, prefix), device="cuda")
+    timed("pfa_scores_window32_prefix8192", lambda: ctx.prefill_attention_scores(
+        q, k, nq, nkv, d, sl, prefix, d, prefix * d, prefix - sl, qwin, sum_out=sum_out, per_row=per_row),
+        nkv * prefix * d * 2 + (nq * prefix + qwin * prefix) * 4 * 2,
+        "K read once + the two score buffers updated; %d MMAC" % (nq * qwin * prefix * d // 1000000))
     return res
 
 
