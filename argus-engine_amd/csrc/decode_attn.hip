@@ -52,7 +52,12 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
   constexpr int TILE = RPW * U;    // rows per wave iteration
   static_assert(LPR >= GT && LPR <= 64, "row group must cover the query-head tile");
 
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  // A GQA group wider than the head tile is covered by several workgroups per KV head, GT heads each
+  // (they re-read the KV rows: this kernel is the fall-back for such shapes, not their fast path).
+  const int split = blockIdx.x, kvh = blockIdx.y / p.head_chunks, b = blockIdx.z;
+  const int hchunk = blockIdx.y % p.head_chunks;
+  const int hbase = kvh * p.group + GT * hchunk;        // first query head of this workgroup
+  const int gcount = min(GT, p.group - GT * hchunk);    // and how many it has
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int grp = lane / LPR, sub = lane % LPR;
   const int c0 = sub * E;
@@ -69,7 +74,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
   float q[GT][E];
 #pragma unroll
   for (int g = 0; g < GT; ++g) {
-    const int h = kvh * p.group + min(g, p.group - 1);
+    const int h = hbase + min(g, gcount - 1);
     const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)h * D + c0;
 #pragma unroll
     for (int e = 0; e < E; ++e) q[g][e] = qp[e] * p.scale;
@@ -130,8 +135,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
         const int t = base + u * RPW + grp;
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
-          if (sub == g && g < p.group && valid[u])
-            p.scores[(int64_t)b * p.score_bs + (int64_t)(kvh * p.group + g) * p.score_stride + t] = s[u][g];
+          if (sub == g && g < gcount && valid[u])
+            p.scores[(int64_t)b * p.score_bs + (int64_t)(hbase + g) * p.score_stride + t] = s[u][g];
         }
       }
     }
@@ -203,9 +208,9 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
   }
   __syncthreads();
 
-  for (int i = threadIdx.x; i < p.group * D; i += 256) {
+  for (int i = threadIdx.x; i < gcount * D; i += 256) {
     const int g = i / D, c = i % D;
-    const int h = kvh * p.group + g;
+    const int h = hbase + g;
     float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
     const float m_ref = (mm == kNegInf) ? 0.0f : mm;
     float o = 0.0f, ll = 0.0f;
@@ -229,12 +234,12 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
     }
   }
   if (p.direct) {
-    for (int g = 0; g < p.group; ++g) {
+    for (int g = 0; g < gcount; ++g) {
       const float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
       const float m_ref = (mm == kNegInf) ? 0.0f : mm;
       float ll = 0.0f;
       for (int w = 0; w < 4; ++w) ll += lds_l[w][g] * __expf(lds_m[w][g] - m_ref);
-      if (!(ll > 0.0f && ll < __builtin_huge_valf())) uniform_fallback<KV_T>(p, b, kvh * p.group + g, D);
+      if (!(ll > 0.0f && ll < __builtin_huge_valf())) uniform_fallback<KV_T>(p, b, hbase + g, D);
     }
   }
 }
@@ -251,7 +256,8 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
   constexpr int E = KvVec<KV_T>::E;
   constexpr int tile_rows = 4 * (64 / (D / E)) * U;  // rows one workgroup consumes per iteration
 
-  const int pairs = batch * p.n_heads_kv;
+  p.head_chunks = (p.group + GT - 1) / GT;
+  const int pairs = batch * p.n_heads_kv * p.head_chunks;
   // Many more workgroups than resident slots, so the last partially filled round of the grid
   // costs little; bounded below by one tile per wave.
   const int target_wgs = ctx->compute_units * 24;
@@ -273,7 +279,7 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
     p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   }
 
-  dim3 grid(nsplit, p.n_heads_kv, batch);
+  dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
   {
     KernelTimer timer(ctx, stream);
     if (p.kv_index)
@@ -296,8 +302,7 @@ int dispatch_group(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_sco
   if (p.group <= 1) return launch_decode<D, 1, KV_T>(ctx, p, batch, want_scores, stream);
   if (p.group <= 2) return launch_decode<D, 2, KV_T>(ctx, p, batch, want_scores, stream);
   if (p.group <= 4) return launch_decode<D, 4, KV_T>(ctx, p, batch, want_scores, stream);
-  if (p.group <= 8) return launch_decode<D, 8, KV_T>(ctx, p, batch, want_scores, stream);
-  return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "GQA group %d > 8 not supported", p.group);
+  return launch_decode<D, 8, KV_T>(ctx, p, batch, want_scores, stream);  // wider groups: several head tiles per KV head
 }
 
 template <typename KV_T>

@@ -26,6 +26,7 @@ struct DecodeParams {
   float scale, softcap;
   int32_t direct;  // nsplit == 1 and no scores: first pass writes `out` itself
   int32_t slot_bound;  // slots an index list may name (the cache capacity)
+  int32_t head_chunks; // vector-ALU kernel: workgroups per KV head (GQA groups wider than its head tile)
 };
 
 // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1); the argument is clamped where

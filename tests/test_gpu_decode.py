@@ -49,6 +49,8 @@ MATRIX = [
     (8, 2, 64, 1024), (8, 2, 64, 1025), (12, 2, 128, 2047), (12, 2, 128, 2500),
     (8, 2, 128, 4096), (14, 2, 64, 1024), (8, 4, 256, 777), (32, 8, 128, 300), (6, 2, 256, 129),
     (16, 2, 64, 555), (3, 1, 128, 70), (5, 1, 64, 200),
+    # GQA groups wider than 8 (12, 16): F32 caches and short rows take several head tiles per KV head
+    (24, 2, 128, 63), (32, 2, 64, 100), (96, 8, 64, 300), (12, 1, 256, 40),
 ]
 
 
