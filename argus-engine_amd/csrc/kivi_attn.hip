@@ -44,7 +44,10 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
   constexpr int MAXD = 256;
   const DecodeParams &p = kp.d;
   const int D = kp.head_dim;
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  // a GQA group wider than the head tile: several workgroups per KV head, GT heads each
+  const int split = blockIdx.x, kvh = blockIdx.y / p.head_chunks, b = blockIdx.z;
+  const int hbase = kvh * p.group + GT * (blockIdx.y % p.head_chunks);
+  const int gcount = min(GT, p.group - GT * (int)(blockIdx.y % p.head_chunks));
   const int tid = threadIdx.x;
   const uint8_t *qk_b = kp.qk + (int64_t)b * kp.qk_bs;
   const uint8_t *qv_b = kp.qv + (int64_t)b * kp.qv_bs;
@@ -62,7 +65,7 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
 
   for (int i = tid; i < D * GT; i += 256) {
     const int ch = i / GT, g = i % GT;
-    const int h = kvh * p.group + min(g, p.group - 1);
+    const int h = hbase + min(g, gcount - 1);
     sh_q[ch][g] = p.q[(int64_t)b * p.q_bs + (int64_t)h * D + ch] * p.scale;
   }
   if (tid < GT) {
@@ -145,8 +148,8 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
         sv = (sv != sv) ? sv : capped;
       }
       if (t >= n_valid) sv = kNegInf;
-      if (p.scores && g < p.group && t < n_valid)
-        p.scores[(int64_t)b * p.score_bs + (int64_t)(kvh * p.group + g) * p.score_stride + tok0 + t] = sv;
+      if (p.scores && g < gcount && t < n_valid)
+        p.scores[(int64_t)b * p.score_bs + (int64_t)(hbase + g) * p.score_stride + tok0 + t] = sv;
       const float m_old = sh_m[g];
       const float m_new = fmaxf(m_old, group_allreduce_max<32>(sv));
       const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
@@ -200,10 +203,10 @@ __global__ __launch_bounds__(256) void kivi_split_kernel(const KiviParams kp) {
   if (vtp == 0) {
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
-      if (g >= p.group) continue;
+      if (g >= gcount) continue;
       float o = acc[g];
       for (int tp = 1; tp < vparts; ++tp) o += red[(tp * GT + g) * D + vc];
-      const int h = kvh * p.group + g;
+      const int h = hbase + g;
       const int64_t pidx = ((int64_t)b * p.n_heads_q + h) * p.nsplit + split;
       p.ws_o[pidx * D + vc] = o;
       if (vc == 0) {
@@ -317,7 +320,8 @@ int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t strea
   DecodeParams &p = kp.d;
   const int D = kp.head_dim;
   const int target_wgs = ctx->compute_units * 4;
-  const int pairs = p.n_heads_kv * batch;
+  p.head_chunks = (p.group + 7) / 8;  // head tile of the widest instantiation
+  const int pairs = p.n_heads_kv * p.head_chunks * batch;
   int nsplit = std::max(1, std::min({(target_wgs + pairs - 1) / pairs, kp.units_total, kMaxSplits}));
   kp.units_per_split = (kp.units_total + nsplit - 1) / nsplit;
   nsplit = (kp.units_total + kp.units_per_split - 1) / kp.units_per_split;
@@ -330,7 +334,7 @@ int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t strea
   p.ws_ml = ctx->ws;
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
 
-  dim3 grid(nsplit, p.n_heads_kv, batch);
+  dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
   {
     KernelTimer timer(ctx, stream);
     if (p.group <= 1) hipLaunchKernelGGL((kivi_split_kernel<BITS, 1>), grid, dim3(256), 0, stream, kp);
@@ -366,8 +370,6 @@ ARGUS_API int argus_hip_attention_gen_quant_ex(argus_hip_ctx *ctx, const argus_h
   const size_t D = a->head_dim;
   if (D != 64 && D != 128 && D != 256)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_quant: head_dim %zu not in {64,128,256}", D);
-  if (a->num_heads_q / a->num_heads_kv > 8)
-    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_quant: GQA group > 8");
   if (a->res_cap == 0 || a->res_cap % kUnit || a->q_tokens % kUnit || a->res_tokens > a->res_cap)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen_quant: q_tokens %zu res_tokens %zu res_cap %zu",
                       a->q_tokens, a->res_tokens, a->res_cap);

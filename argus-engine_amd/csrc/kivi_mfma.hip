@@ -195,12 +195,16 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM];
 
   const DecodeParams &p = kp.d;
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  // A GQA group wider than 8 is covered by several workgroups per KV head, 8 heads each (they re-read
+  // the blocks; the reference kernel runs one block per query head whatever the ratio).
+  const int split = blockIdx.x, kvh = blockIdx.y / p.head_chunks, b = blockIdx.z;
+  const int hchunk = blockIdx.y % p.head_chunks;
+  const int hbase = kvh * p.group + kMaxGroup * hchunk;  // first query head of this workgroup
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // keeps unit indices and tile addresses scalar
   const int j = lane >> 4, r = lane & 15;
   const int ra = r / GT, rh = r % GT;  // slice owner index and head of this lane during preparation
-  const int G = p.group;
+  const int G = min(kMaxGroup, p.group - kMaxGroup * hchunk);  // heads of this workgroup
   const int gpf = kp.res_cap / kUnit;
   const int q_units = kp.q_tokens / kUnit;
 
@@ -217,7 +221,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   for (int s = 0; s < NS; ++s) {
     const int kk = ra + s * NREP;
     const bool ok = kk < KK && rh < G;
-    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(kvh * G + min(rh, G - 1)) * D + 32 * min(kk, KK - 1) + 8 * j;
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(hbase + min(rh, G - 1)) * D + 32 * min(kk, KK - 1) + 8 * j;
     float qv[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) qv[e] = qp[e];  // the address is clamped
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         mt = fmaxf(mt, s[w][i]);  // a NaN logit propagates (the reference kernels have no guard)
       }
     if (p.scores && r < G) {
-      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + r) * p.score_stride + tok0 + 8 * j;
+      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(hbase + r) * p.score_stride + tok0 + 8 * j;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -454,7 +458,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     const int64_t rbase = (int64_t)b * kp.res_bs + (int64_t)kvh * kp.res_cap * D + (int64_t)ru * kUnit * D;
     const RES_T *rk = (const RES_T *)kp.res_k + rbase;
     const RES_T *rv = (const RES_T *)kp.res_v + rbase;
-    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(kvh * G + min(r, G - 1)) * D + 8 * j;
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(hbase + min(r, G - 1)) * D + 8 * j;
     float4_t s[2];
     s[0] = s[1] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -533,7 +537,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 
   for (int idx = threadIdx.x; idx < G * D; idx += 256) {
     const int g = idx / D, c = idx % D;
-    const int h = kvh * G + g;
+    const int h = hbase + g;
     const float mm = fmaxf(fmaxf(lds_m[0][g], lds_m[1][g]), fmaxf(lds_m[2][g], lds_m[3][g]));
     const float m_ref = (mm == kNegInf) ? 0.0f : mm;
     float o = 0.0f, ll = 0.0f;
@@ -556,7 +560,8 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 template <int BITS, int D>
 int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   DecodeParams &p = kp.d;
-  const int pairs = p.n_heads_kv * batch;
+  p.head_chunks = (p.group + kMaxGroup - 1) / kMaxGroup;
+  const int pairs = p.n_heads_kv * p.head_chunks * batch;
   // One round of co-resident workgroups: a second, partly filled round would run at a fraction of
   // the occupancy the unit loop needs to hide its LDS and HBM latency.
   static const int wgs_per_cu = [] {
@@ -578,7 +583,7 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   if (rc != ARGUS_HIP_OK) return rc;
   p.ws_ml = ctx->ws;
   p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
-  const dim3 grid(nsplit, p.n_heads_kv, batch);
+  const dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
   {
     KernelTimer timer(ctx, stream);
     const bool cap = p.softcap > 0.0f;
@@ -607,7 +612,6 @@ int launch_dim(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream
 bool kivi_mfma_supported(const KiviParams &kp) {
   const DecodeParams &p = kp.d;
   if (kp.head_dim != 64 && kp.head_dim != 128 && kp.head_dim != 256) return false;
-  if (p.group > kMaxGroup) return false;
   // tiles are copied as 16-byte vectors
   if ((((uintptr_t)kp.qk | (uintptr_t)kp.qv) & 15) || (kp.qk_bs & 15) || (kp.qv_bs & 15)) return false;
   // residual rows are read as 16-byte vectors

@@ -89,7 +89,9 @@ def test_reference_device_test_patterns():
 @pytest.mark.parametrize("bits", [2, 4, 8])
 @pytest.mark.parametrize("hq,hkv,d,R,n", [(8, 2, 64, 64, 203), (4, 4, 128, 32, 97), (8, 4, 256, 128, 300),
                                           (14, 2, 64, 128, 128), (32, 8, 128, 128, 1024),
-                                          (16, 8, 256, 128, 2100), (32, 4, 256, 64, 700), (3, 1, 256, 32, 1500)])
+                                          (16, 8, 256, 128, 2100), (32, 4, 256, 64, 700), (3, 1, 256, 32, 1500),
+                                          # GQA groups of 12 and 16: two head tiles per KV head
+                                          (24, 2, 128, 64, 500), (32, 2, 64, 32, 300), (16, 1, 256, 128, 260)])
 def test_kivi_attention_vs_oracle(bits, hq, hkv, d, R, n):
     rng = np.random.default_rng(bits * 1000 + n)
     k = rng.standard_normal((n, hkv, d)).astype(np.float32)
