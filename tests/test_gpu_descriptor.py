@@ -96,3 +96,45 @@ def test_q4_0_cache_through_the_floor_matches_oracle_attention():
     vd = O.decode_via_descriptor(O.DESC_Q4_0, O.encode_via_descriptor(O.DESC_Q4_0, v), n).reshape(hkv, cap, d)
     ref = O.attention_gen(q, kd.astype(np.float16), vd.astype(np.float16), hkv, L, cap)
     check_attention_out(host(out), ref)
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_codec_random_shapes_and_alignments(case):
+    # Block sizes other than 32, block counts that do not fill a wave, and buffers that start at odd
+    # element offsets (which take the one-thread-per-block kernels) against the oracle, bit for bit.
+    import torch
+    rng = np.random.default_rng(5000 + case)
+    block_elems = int(rng.choice([8, 16, 32, 32, 32, 64]))
+    kind = int(rng.integers(0, 4))
+    desc = [(block_elems, 4, O.SCALE_F16, O.PACK_NIBBLE), (block_elems, 4, O.SCALE_F16_MIN, O.PACK_NIBBLE),
+            (block_elems, 8, O.SCALE_F16, O.PACK_BYTE), (block_elems, 2, O.SCALE_F16_MIN, O.PACK_QUAD)][kind]
+    n_blocks = int(rng.choice([1, 2, 3, 63, 64, 65, 255, 1000, 4099]))
+    n = n_blocks * block_elems
+    bb = O.desc_block_bytes(desc)
+    raw = rng.integers(0, 256, size=(n_blocks, bb), dtype=np.uint8)
+    raw[:, 0:2] = rng.uniform(0.01, 2.0, n_blocks).astype(np.float16).view(np.uint8).reshape(n_blocks, 2)
+    if desc[2] == O.SCALE_F16_MIN:
+        raw[:, 2:4] = rng.uniform(-3.0, 3.0, n_blocks).astype(np.float16).view(np.uint8).reshape(n_blocks, 2)
+    raw = raw.reshape(-1)
+    ref = O.decode_via_descriptor(desc, raw, n)
+    off = int(rng.choice([0, 0, 1, 3, 4]))  # elements: an odd offset breaks the 16-byte alignment of the rows
+    d32 = torch.full((n + off + 8,), 9.0, device="cuda")
+    d16 = torch.full((n + off + 8,), 9.0, device="cuda", dtype=torch.float16)
+    src = dev(raw)
+    ctx().kv_decode_descriptor(desc, src, d32[off:], n)
+    ctx().kv_decode_descriptor(desc, src, d16[off:], n)
+    g32, g16 = host(d32), host(d16)
+    assert np.array_equal(g32[off:off + n].view(np.uint32), ref.view(np.uint32))
+    assert (g32[:off] == 9.0).all() and (g32[off + n:] == 9.0).all()
+    assert np.array_equal(g16[off:off + n].view(np.uint16), ref.astype(np.float16).view(np.uint16))
+    assert (g16[:off] == 9.0).all() and (g16[off + n:] == 9.0).all()
+    if kind in (0, 3):  # the two writable formats
+        x = (rng.standard_normal(n) * rng.choice([0.01, 1.0, 30.0])).astype(np.float32)
+        x[: block_elems] = 0.0
+        want = O.encode_via_descriptor(desc, x)
+        xs = torch.zeros(n + off, device="cuda")
+        xs[off:] = dev(x)
+        out = torch.full((want.size + 6,), 0xAB, device="cuda", dtype=torch.uint8)
+        ctx().kv_encode_descriptor(desc, xs[off:], out, n)
+        got = host(out)
+        assert np.array_equal(got[:want.size], want) and (got[want.size:] == 0xAB).all()
