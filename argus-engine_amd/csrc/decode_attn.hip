@@ -291,7 +291,7 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   if (!p.direct) {
-    hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<KV_T>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<KV_T>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
     ARGUS_HIP_CHECK(ctx, hipGetLastError());
   }
   return ARGUS_HIP_OK;

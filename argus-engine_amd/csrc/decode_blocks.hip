@@ -41,6 +41,13 @@ typedef uint32_t u32_a2 __attribute__((aligned(2)));  // code words sit at 2-byt
 
 enum { kFmtQ4_0 = 0, kFmtQ4_1 = 1, kFmtQ8_0 = 2, kFmtQ2_0 = 3 };
 
+// Orders a wave's LDS accesses for the compiler when its lanes exchange data through LDS.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <int FMT>
 struct BlockFmt {
   static constexpr bool kHasMin = FMT == kFmtQ4_1 || FMT == kFmtQ2_0;  // header is (d, m)
@@ -131,15 +138,29 @@ __device__ __forceinline__ RawBlock<FMT> load_block(const uint8_t *base, uint32_
   return b;
 }
 
+// v_permlane16_swap / v_permlane32_swap: trade the odd rows, or the upper half, of the first register
+// with the even rows, or the lower half, of the second.
+struct SwapPair {
+  uint32_t first, second;
+};
+__device__ __forceinline__ SwapPair permlane16_swap(uint32_t a, uint32_t b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+  return {r[0], r[1]};
+}
+__device__ __forceinline__ SwapPair permlane32_swap(uint32_t a, uint32_t b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  return {r[0], r[1]};
+}
+
 // 4 x 4 transpose across the four lane groups (lanes 16 apart): lane group j ends up with what lane
-// groups 0..3 held in v[j].  v_permlane16_swap trades v[0], v[2] of the odd groups with v[1], v[3]
-// of the even ones, v_permlane32_swap does the same between the halves of the wave.
+// groups 0..3 held in v[j]: the 16-lane swap trades v[0], v[2] of the odd groups with v[1], v[3]
+// of the even ones, the 32-lane swap does the same between the halves of the wave.
 __device__ __forceinline__ void transpose_lane_groups(uint32_t (&v)[4]) {
-  auto a = __builtin_amdgcn_permlane16_swap(v[0], v[1], false, false);
-  auto b = __builtin_amdgcn_permlane16_swap(v[2], v[3], false, false);
-  auto c = __builtin_amdgcn_permlane32_swap(a[0], b[0], false, false);
-  auto d = __builtin_amdgcn_permlane32_swap(a[1], b[1], false, false);
-  v[0] = c[0]; v[2] = c[1]; v[1] = d[0]; v[3] = d[1];
+  const SwapPair a = permlane16_swap(v[0], v[1]);
+  const SwapPair b = permlane16_swap(v[2], v[3]);
+  const SwapPair c = permlane32_swap(a.first, b.first);
+  const SwapPair d = permlane32_swap(a.second, b.second);
+  v[0] = c.first; v[2] = c.second; v[1] = d.first; v[3] = d.second;
 }
 
 // Lane group j holds block j of its row; afterwards piece[kk] is the lane's piece (code index j)
@@ -161,10 +182,10 @@ __device__ __forceinline__ void block_to_pieces(const RawBlock<FMT> &b, RawPiece
     for (int kk = 0; kk < 4; ++kk) piece[kk].code[w] = v[kk];
   }
   // headers: all-gather over the lane groups with the same two trades
-  auto p = __builtin_amdgcn_permlane16_swap(b.hdr, b.hdr, false, false);       // (even group's, odd group's)
-  auto lo = __builtin_amdgcn_permlane32_swap(p[0], p[0], false, false);         // (group 0's, group 2's)
-  auto hi = __builtin_amdgcn_permlane32_swap(p[1], p[1], false, false);         // (group 1's, group 3's)
-  piece[0].hdr = lo[0]; piece[2].hdr = lo[1]; piece[1].hdr = hi[0]; piece[3].hdr = hi[1];
+  const SwapPair p = permlane16_swap(b.hdr, b.hdr);        // (even group's, odd group's)
+  const SwapPair lo = permlane32_swap(p.first, p.first);   // (group 0's, group 2's)
+  const SwapPair hi = permlane32_swap(p.second, p.second); // (group 1's, group 3's)
+  piece[0].hdr = lo.first; piece[2].hdr = lo.second; piece[1].hdr = hi.first; piece[3].hdr = hi.second;
 }
 
 // Bytes b0 b1 b2 b3 of `bytes` (each < 256) -> halves {1024 + b0, 1024 + b1} and {1024 + b2, 1024 + b3}:
@@ -176,12 +197,14 @@ __device__ __forceinline__ half2_t bytes_hi(uint32_t bytes) {
   return __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, bytes, 0x04030402u));
 }
 // Two nibbles of a code word, 16 bits apart and already at bits 4..7 / 20..23 -> {64 + n, 64 + n'}.
-// One v_and_or_b32 (spelled out: this target's three-operand form takes no literal, and the
-// compiler otherwise emits the AND and the OR separately).
+// One v_and_or_b32 when the callers keep `mask` and `exponent` in vector registers (this target's
+// three-operand form takes no literal).  Plain C on purpose: an instruction written as inline asm is
+// invisible to the compiler's hazard recogniser, and a VALU write into a register that an MFMA in
+// flight still reads as its accumulator input needs wait states that only the recogniser inserts.
+// Spelled as asm, this function overwrote such registers in some builds (wrong logits for q4_1 and
+// q2_0, depending on what the scheduler placed behind the MFMAs).
 __device__ __forceinline__ half2_t nibbles(uint32_t word, uint32_t mask, uint32_t exponent) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(word), "v"(mask), "v"(exponent));
-  return __builtin_bit_cast(half2_t, r);
+  return __builtin_bit_cast(half2_t, (word & mask) | exponent);
 }
 
 // v_perm selectors that spread one 16-bit half of a dword as [byte, 0, next byte, 0] (q2_0 pieces),
@@ -304,6 +327,7 @@ __device__ float block_elem(const uint8_t *blk, int e) {
 // Uniform-weights fallback of common.rs:806-813 for a block cache: out = mean of the attended V rows.
 template <int FMT>
 struct BlockFallback {
+  static constexpr bool kHandlesRow = true;
   static __device__ bool run(const DecodeParams &p, int b, int h, int D) {
     using F = BlockFmt<FMT>;
     const int kvh = h / p.group;
@@ -531,6 +555,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
+  __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
+  const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
+  int base_last = -(1 << 30);
 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
     // ---- logits ---------------------------------------------------------------------------------
@@ -586,10 +613,6 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         }
       }
     }
-    // The requests stay behind the logits: when the scheduler was free to move them up between the
-    // last block's MFMAs, the q4_1 head_dim 256 build returned wrong logits for the iteration's last
-    // tile (register data flow of that build read correct; cause not identified).
-    __builtin_amdgcn_sched_barrier(0);
     load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
     load_idx_k(base + 2 * kWaves * TILE);
     if constexpr (SOFTCAP) {
@@ -619,17 +642,8 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         s[tw][i] = fmaxf(s[tw][i], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
         mt = fmaxf(mt, s[tw][i]);
       }
-    if (p.scores && r < G) {
-      // Logits in natural units; the combine pass rewrites them as probabilities.
-      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + r) * p.score_stride;
-#pragma unroll
-      for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int t = base + 16 * tw + 4 * j + i;
-          if (t < t_end) srow[t] = s[tw][i] * kLn2;
-        }
-    }
+    sink.store(s, base);
+    base_last = base;
 
     // ---- online softmax: the running max of a head is shared by the four lane groups -----------
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
@@ -676,14 +690,19 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
       for (int sg = 0; sg < VSEG; ++sg) {
         RawPiece<FMT> vpc[4];  // the lane's piece of tokens 4j .. 4j+3
         if constexpr (kStageV) {
-          typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
           __shared__ uint32_t v_strip[kWaves][VL][64 * 4 + 4 * 4];
           constexpr bool kShared = D == 64;  // one request serves both tiles
           const RawBlock<FMT> &mine = vblk_raw[kShared ? 0 : tw * VSEG + sg];
           uint32_t *strip = v_strip[wave][kShared ? 0 : tw * VSEG + sg];
+          // The lanes of a wave exchange data through the strip, so the write must be ordered before
+          // the other lanes' reads and those before the next write: wave-level fences (LDS operations
+          // of a wave execute in order; the fences are there for the compiler, which may otherwise
+          // move a lane's reads above its own write, since it reads addresses it did not write).
           if (!kShared || tw == 0) {
+            wave_lds_fence();  // the previous reads of this strip are done
             if constexpr (FMT == kFmtQ2_0) *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{mine.code[0], mine.code[1], 0u, 0u};
             else *(u32x4_t *)(strip + 4 * lane + 4 * j) = u32x4_t{mine.code[0], mine.code[1], mine.code[2], mine.code[3]};
+            wave_lds_fence();
           }
           // token 4j + e was loaded by lane 16j + 4(r/4) + e (head_dim 64: 16j + 8 tw + 4(r/4 % 2) + e);
           // this lane wants dword r%4 of it
@@ -730,6 +749,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
+  sink.store_tail(base_last);
 
   if constexpr (kHdrTerm) {
     constexpr float kTerm = (FMT == kFmtQ4_0) ? -CD::kZero : 1.0f;
@@ -813,7 +833,7 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
     else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, false>), grid, block, 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
-  hipLaunchKernelGGL((decode_combine_kernel<BlockFallback<FMT>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((decode_combine_kernel<BlockFallback<FMT>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
 }
@@ -838,6 +858,8 @@ int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtyp
   const int64_t rows = p.kv_index ? p.slot_bound : p.len;  // an index list may name any slot of the cache
   if (rows >= (1 << 24) || p.row_stride / 32 * 34 >= (1 << 24) || rows * (p.row_stride / 32 * 34) > 0xffffffffll)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: block-quantised head slab beyond 4 GiB");
+  if (!score_rows_addressable(p))
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: score rows of a head group beyond 2 GiB");
   switch (kv_dtype) {
     case ARGUS_HIP_Q4_0: return launch_blocks_dim<kFmtQ4_0>(ctx, p, D, batch, stream);
     case ARGUS_HIP_Q4_1: return launch_blocks_dim<kFmtQ4_1>(ctx, p, D, batch, stream);

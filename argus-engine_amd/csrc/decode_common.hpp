@@ -5,6 +5,7 @@
 #include "argus_hip_internal.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace argus_decode {
 
@@ -64,6 +65,7 @@ __device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
 template <typename KV_T>
 struct UniformFallback {
   // Scalar reference behaviour (common.rs:561-577): uniform weights.
+  static constexpr bool kHandlesRow = true;  // run() writes the whole output and score row
   static __device__ bool run(const DecodeParams &p, int b, int h, int D) {
     uniform_fallback<KV_T>(p, b, h, D);
     return true;
@@ -71,12 +73,16 @@ struct UniformFallback {
 };
 struct NoFallback {
   // The reference KIVI kernels have no guard (kivi_attn.cu:252-390): NaN propagates.
+  static constexpr bool kHandlesRow = false;
   static __device__ bool run(const DecodeParams &, int, int, int) { return false; }
 };
 
 // Second pass: log-sum-exp merge of the splits of one (sequence, Q head); optional in-place
 // logits -> probabilities rewrite of the score row.  The 256 threads are arranged as
 // (split group) x (float4 column) so the loop over splits is short and the loads are wide.
+// A long score row is shared between gridDim.z workgroups: each merges the (m, l) pairs for
+// itself (a few hundred bytes), the first also writes the output row, and every one rewrites its
+// slice of the scores (one workgroup per 32K-token row took 40 us).
 constexpr int kMaxSplits = 128;
 
 template <typename FALLBACK, int D>
@@ -85,6 +91,7 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   constexpr int NSG = 256 / CQ;            // split groups
   constexpr int PER = kMaxSplits / NSG;    // splits per thread at most
   const int h = blockIdx.x, b = blockIdx.y;
+  const bool first = blockIdx.z == 0;  // the workgroup that also merges the output row
   const int64_t pbase = ((int64_t)b * p.n_heads_q + h) * p.nsplit;
   const int cq = threadIdx.x % CQ, sg = threadIdx.x / CQ;
   __shared__ float sh_w[kMaxSplits];
@@ -95,10 +102,12 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   // re-read it and get weight zero.
   const int last = p.nsplit - 1;
   float4_t part[PER];
+  if (first) {
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    if (i * NSG > last) break;  // uniform
-    part[i] = *(const float4_t *)(p.ws_o + (pbase + min(sg + i * NSG, last)) * D + 4 * cq);
+    for (int i = 0; i < PER; ++i) {
+      if (i * NSG > last) break;  // uniform
+      part[i] = *(const float4_t *)(p.ws_o + (pbase + min(sg + i * NSG, last)) * D + 4 * cq);
+    }
   }
   if (threadIdx.x < 64) {
     constexpr int MLP = kMaxSplits / 64;
@@ -131,26 +140,137 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   __syncthreads();
   const float mm = sh_m, ll = sh_l;
   if (!(ll > 0.0f && ll < __builtin_huge_valf())) {
-    if (FALLBACK::run(p, b, h, D)) return;
+    if (!first && FALLBACK::kHandlesRow) return;  // the first workgroup writes the whole row
+    if (first && FALLBACK::run(p, b, h, D)) return;
   }
   const float inv = 1.0f / ll;  // non-finite when the fallback declined: NaN propagates
-  float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (first) {
+    float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    if (i * NSG > last) break;
-    o += part[i] * sh_w[sg + i * NSG];
-  }
-  sh_o[sg][cq] = o;
-  __syncthreads();
-  if (sg == 0) {
+    for (int i = 0; i < PER; ++i) {
+      if (i * NSG > last) break;
+      o += part[i] * sh_w[sg + i * NSG];
+    }
+    sh_o[sg][cq] = o;
+    __syncthreads();
+    if (sg == 0) {
 #pragma unroll
-    for (int g = 1; g < NSG; ++g) o += sh_o[g][cq];
-    *(float4_t *)(p.out + (int64_t)b * p.out_bs + (int64_t)h * D + 4 * cq) = o * inv;
+      for (int g = 1; g < NSG; ++g) o += sh_o[g][cq];
+      *(float4_t *)(p.out + (int64_t)b * p.out_bs + (int64_t)h * D + 4 * cq) = o * inv;
+    }
   }
   if (p.scores) {
     float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    for (int t = threadIdx.x; t < p.len; t += 256) srow[t] = __expf(srow[t] - mm) * inv;
+    const int slice = ((p.len + (int)gridDim.z - 1) / (int)gridDim.z + 255) / 256 * 256;
+    const int t_end = min(p.len, ((int)blockIdx.z + 1) * slice);
+    for (int t = (int)blockIdx.z * slice + threadIdx.x; t < t_end; t += 256) srow[t] = __expf(srow[t] - mm) * inv;
   }
+}
+
+// Where the matrix-core kernels put their logits (natural units; the combine pass rewrites them as
+// probabilities).  Out of the MFMA a lane (j, r) holds tokens 4j..4j+3 of head r for each 16-token
+// tile, so a store from those registers hands the memory system sixteen 16-byte pieces of sixteen
+// different lines per instruction.  The wave turns its TW tiles round in LDS instead: eight
+// consecutive lanes take one head's 16 TW tokens, and one instruction writes whole lines of eight
+// heads.
+// The stores go through a buffer descriptor over the score rows of the KV head's group: heads past
+// the group, token groups that reach past the chunk and a call without `scores` (zero records)
+// carry an offset outside it and the hardware drops them.  Every iteration of the token loop then
+// issues the same store with no branch around it, which keeps the compiler's counts of outstanding
+// memory operations exact (with a store on one side of a branch it assumes none, and the wait for a
+// V tile comes to include the first requests of the K tile just asked for).  A chunk ends inside a
+// lane's token group only at the end of the row; that group is written after the loop (store_tail).
+// Groups of more than 8 heads take a second store under a branch.  Rows of at most 2 GiB per group:
+// score_rows_addressable().
+// What the stores cost is set by the bytes written, not by their form: 32 heads x 32K tokens x 16
+// sequences (67 MB of logits beside 2.1 GB of K and V) take the F16 kernel from 302 to 426 us with
+// per-lane stores under a branch, with branch-free stores and with the whole-line stores below
+// alike; the staging alone is free (304 us with the store left out), a quarter of the stores costs
+// 355 us, the same stores confined to 4 KB per row (no DRAM writes) 393 us, and the fetch counter
+// shows no extra reads.  Loads and stores of a wave retire in order on this target, so a store
+// whose acknowledgement is slow under a saturated read stream holds back the loads issued after it.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <int TW>
+struct LogitSink {
+  static_assert(TW == 1 || TW == 2, "one or two 16-token tiles per wave iteration");
+  static constexpr int T = 16 * TW, ROW = T + 4, VEC = 2 * TW;  // in floats; ROW keeps 16-byte alignment
+  static constexpr int kStageFloats = 16 * ROW;                 // per wave
+  static constexpr uint32_t kDropped = 0x80000000u;
+  static constexpr float kLn2 = 0.6931471805599453f;
+  using vec_t = typename std::conditional<TW == 2, u32x4_t, u32x2_t>::type;
+
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t off[2];  // byte offset of the lane's first token in its row, for heads 0..7 and 8..15
+  float *wr;        // where lane (j, r) puts a tile's four logits
+  const float *rd;  // the lane's VEC tokens of head lane / 8
+  int tok, t_end;
+  bool on, wide;
+
+  __device__ __forceinline__ LogitSink(const DecodeParams &p, float *stage, int b, int first_head, int heads, int lane, int t_end_)
+      : t_end(t_end_) {
+    const uint32_t bytes = p.scores ? (uint32_t)((((int64_t)heads - 1) * p.score_stride + t_end_) * 4) : 0u;
+    void *rows = p.scores ? (void *)(p.scores + (int64_t)b * p.score_bs + (int64_t)first_head * p.score_stride) : nullptr;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(rows, 0, bytes, 0x00020000);
+    on = p.scores != nullptr;
+    wide = heads > 8;
+    tok = VEC * (lane & 7);
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int row = 8 * n + (lane >> 3);
+      off[n] = (row < heads) ? (uint32_t)(((int64_t)row * p.score_stride + tok) * 4) : kDropped;
+    }
+    wr = stage + (lane & 15) * ROW + 4 * (lane >> 4);
+    rd = stage + (lane >> 3) * ROW + tok;
+  }
+
+  static __device__ __forceinline__ void wave_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  __device__ __forceinline__ void emit(vec_t v, int n, int base) const {
+    const uint32_t o = (base + tok + VEC <= t_end) ? off[n] + 4u * (uint32_t)base : kDropped;
+    if constexpr (TW == 2) __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, o, 0u, 0);
+    else __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, o, 0u, 0);
+  }
+
+  // `s`: the lane's logits of the TW tiles starting at token `base`, in log2 units.
+  __device__ __forceinline__ void store(const float4_t (&s)[TW], int base) const {
+    vec_t v0 = {}, v1 = {};
+    if (on) {  // uniform; LDS traffic only
+      wave_fence();  // the reads of the previous iteration are done
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) *(float4_t *)(wr + 16 * tw) = s[tw] * kLn2;
+      wave_fence();
+      v0 = *(const vec_t *)rd;
+      if (wide) v1 = *(const vec_t *)(rd + 8 * ROW);
+    }
+    emit(v0, 0, base);
+    if (wide) emit(v1, 1, base);
+  }
+  // The token group that the end of the row cuts, if any.  `base`: the wave's last call of store(),
+  // whose logits the stage still holds.
+  __device__ __forceinline__ void store_tail(int base) const {
+    if (!on || (t_end % VEC) == 0 || base + T <= t_end) return;
+    for (int n = 0; n < (wide ? 2 : 1); ++n)
+#pragma unroll
+      for (int e = 0; e < VEC - 1; ++e) {
+        const int t = base + tok + e;
+        const bool cut = t < t_end && base + tok + VEC > t_end;
+        const float x = rd[n * 8 * ROW + e];
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, x), rsrc, cut ? off[n] + 4u * (uint32_t)(base + e) : kDropped, 0u, 0);
+      }
+  }
+};
+inline bool score_rows_addressable(const DecodeParams &p) {
+  return !p.scores || (p.score_stride >= p.len && ((int64_t)p.group * p.score_stride + 1024) * 4 <= 0x7fffffffll);
+}
+
+// Grid of the combine pass: one workgroup per (head, sequence), more along z for long score rows.
+inline dim3 combine_grid(const DecodeParams &p, int batch) {
+  const int z = p.scores ? std::max(1, std::min(64, p.len / 2048)) : 1;
+  return dim3((unsigned)p.n_heads_q, (unsigned)batch, (unsigned)z);
 }
 
 // Split count of the matrix-core kernels.  The grid is sized against the number of workgroups the

@@ -175,10 +175,14 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     }
   }
 
+  __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
+  const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
+
   float4_t o_acc[NACC];
 #pragma unroll
   for (int a = 0; a < NACC; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
+  int base_last = -(1 << 30);
 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
     // ---- logits ---------------------------------------------------------------------------------
@@ -212,17 +216,8 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
         s[tw][i] = sv;
         mt = fmaxf(mt, sv);
       }
-    if (p.scores && r < G) {
-      // Logits in natural units; the combine pass rewrites them as probabilities.
-      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + r) * p.score_stride;
-#pragma unroll
-      for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int t = base + 16 * tw + 4 * j + i;
-          if (t < t_end) srow[t] = s[tw][i] * kLn2;
-        }
-    }
+    sink.store(s, base);
+    base_last = base;
 
     // ---- online softmax: the running max of a head is shared by the four lane groups -----------
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
@@ -267,6 +262,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
+  sink.store_tail(base_last);
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
   l_run += __shfl_xor(l_run, 16, 64);
@@ -340,7 +336,7 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
     else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, false>), grid, block, 0, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
-  hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
 }
@@ -354,6 +350,7 @@ bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
   const int64_t rows = p.kv_index ? p.slot_bound : (int64_t)p.kv_start + p.len;
   if ((rows + 1024) * p.row_stride * 2 > 0x7fffffffll) return false;
   if (p.kv_index && (rows >= (1 << 24) || p.row_stride * 2 >= (1 << 24))) return false;
+  if (!score_rows_addressable(p)) return false;
   if (D == 64 || D == 128) return p.group <= 16;
   // head_dim 256: one 64-row tile per workgroup costs more set-up (Q split over 256 channels) than it
   // saves; measured against the vector-ALU kernel it only pays for long rows and wider groups

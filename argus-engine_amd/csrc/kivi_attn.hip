@@ -344,9 +344,9 @@ int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t strea
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   switch (D) {
-    case 64: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 64>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p); break;
-    case 128: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 128>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p); break;
-    default: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 256>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p); break;
+    case 64: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 64>), combine_grid(p, batch), dim3(256), 0, stream, p); break;
+    case 128: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 128>), combine_grid(p, batch), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 256>), combine_grid(p, batch), dim3(256), 0, stream, p); break;
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;

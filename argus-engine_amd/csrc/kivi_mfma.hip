@@ -593,7 +593,7 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
     else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false>), grid, dim3(256), 0, stream, kp);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
-  hipLaunchKernelGGL((decode_combine_kernel<NoFallback, D>), dim3(p.n_heads_q, batch), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((decode_combine_kernel<NoFallback, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
 }
