@@ -19,7 +19,8 @@ FORMATS = {
 }
 
 
-def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True, kv_start=0, encode=False, softcap=0.0, q_gain=1.0):
+def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True, kv_start=0, encode=False, softcap=0.0, q_gain=1.0,
+             score_pad=0):
     import argus_hip as A
     desc, name = FORMATS[fmt]
     cap = cap or L
@@ -32,10 +33,10 @@ def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True,
         v_raw = random_blocks(desc, rows * d // 32, seed + 2)
     q = normal((hq, d), seed) * np.float32(q_gain)
     out = dev(np.zeros((hq, d), np.float32))
-    sc = dev(np.zeros((hq, L), np.float32)) if scores else None
+    sc = dev(np.full((hq, L + score_pad), -7.0, np.float32)) if scores else None
     ctx().attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, cap,
                         layout=A.HEAD_MAJOR if head_major else A.SEQ_MAJOR, scores=sc,
-                        score_stride=L if scores else 0, kv_start=kv_start, kv_dtype=getattr(A, name), softcap=softcap)
+                        score_stride=L + score_pad if scores else 0, kv_start=kv_start, kv_dtype=getattr(A, name), softcap=softcap)
     # oracle: a window that starts at kv_start is the same cache with its first rows cut off
     bb = O.desc_block_bytes(desc)
     row_bytes = d // 32 * bb
@@ -49,9 +50,26 @@ def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True,
     what = "%s Hq%d Hkv%d d%d L%d cap%d %s" % (fmt, hq, hkv, d, L, cap, "HM" if head_major else "SM")
     if scores:
         check_attention_out(host(out), ref[0], what)
-        check_scores(host(sc), ref[1], what)
+        got = host(sc)
+        check_scores(got[:, :L], ref[1], what)
+        assert (got[:, L:] == -7.0).all(), what + ": score row written past its length"
     else:
         check_attention_out(host(out), ref, what)
+
+
+@pytest.mark.parametrize("L", [509, 510, 511, 512, 1021, 2050, 2051])
+def test_score_rows_with_padding_stay_untouched_past_the_length(L):
+    # the logits leave in groups of 4 (2 at head_dim 256) tokens per lane; the group that the end of the
+    # row cuts is written token by token
+    run_case("q4_0", 8, 2, 128, L, score_pad=5, seed=L)
+    run_case("q8_0", 14, 2, 64, L, score_pad=3, seed=L + 1)
+    run_case("q4_1", 8, 4, 256, L, score_pad=7, seed=L + 2)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "q2_0"])
+def test_scores_of_groups_wider_than_eight_heads(fmt):
+    run_case(fmt, 12, 1, 128, 1531, score_pad=1)
+    run_case(fmt, 32, 2, 64, 777, score_pad=2, seed=11)
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
