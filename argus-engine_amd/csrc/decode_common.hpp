@@ -28,6 +28,7 @@ struct DecodeParams {
   int32_t direct;  // nsplit == 1 and no scores: first pass writes `out` itself
   int32_t slot_bound;  // slots an index list may name (the cache capacity)
   int32_t head_chunks; // vector-ALU kernel: workgroups per KV head (GQA groups wider than its head tile)
+  int32_t stage_scores;  // matrix-core kernels: the chunk's logits wait in LDS and are written after the token loop
 };
 
 // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1); the argument is clamped where
@@ -187,8 +188,11 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
 // per-lane stores under a branch, with branch-free stores and with the whole-line stores below
 // alike; the staging alone is free (304 us with the store left out), a quarter of the stores costs
 // 355 us, the same stores confined to 4 KB per row (no DRAM writes) 393 us, and the fetch counter
-// shows no extra reads.  Loads and stores of a wave retire in order on this target, so a store
-// whose acknowledgement is slow under a saturated read stream holds back the loads issued after it.
+// shows no extra reads.  Part of it is the wave's own loads waiting behind its stores (loads and
+// stores of a wave retire in order): the F16 kernel therefore keeps a chunk's logits in LDS and
+// writes them when its token loop is over, where the chunk fits (DecodeParams::stage_scores:
+// 390 us), and uses this sink where it does not.  The rest is writes mixed into a saturated read
+// stream: 64 MB filled by another kernel meanwhile cost the plain launch 40 us as well.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 template <int TW>
@@ -280,12 +284,14 @@ inline dim3 combine_grid(const DecodeParams &p, int batch) {
 // 2-tile waves were 10 % slower than 1 round of 4-tile waves).  Cost model, in units of one tile
 // step with the device full: rounds x (tile steps per workgroup + 0.75 for set-up, merge and
 // partial write-out).  Sets p.nsplit and p.chunk (a multiple of tile_rows).
-inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slots) {
+// `max_chunk` > 0: no chunk longer than that many tokens, when the split limit allows it.
+inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slots, int max_chunk = 0) {
   const int max_splits = std::min((p.len + tile_rows - 1) / tile_rows, kMaxSplits);
   int nsplit = 1, chunk = (p.len + tile_rows - 1) / tile_rows * tile_rows;
   float best = 3.0e38f;
   for (int n = 1; n <= max_splits; ++n) {
     const int c = ((p.len + n - 1) / n + tile_rows - 1) / tile_rows * tile_rows;
+    if (max_chunk > 0 && c > max_chunk && n < max_splits) continue;
     const int ns = (p.len + c - 1) / c;
     const int64_t rounds = ((int64_t)pairs * ns + slots - 1) / slots;
     const float cost = (float)rounds * ((float)(c / tile_rows) + 0.75f);

@@ -175,6 +175,10 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     }
   }
 
+  // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
+  // then the merge area.
+  extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
+  const int stage_row = p.chunk + 4;
   __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
   const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
 
@@ -216,8 +220,15 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
         s[tw][i] = sv;
         mt = fmaxf(mt, sv);
       }
-    sink.store(s, base);
-    base_last = base;
+    if (p.stage_scores) {  // uniform; LDS only
+      if (r < G) {
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) *(float4_t *)(dyn_lds + r * stage_row + (base - t_begin) + 16 * tw + 4 * j) = s[tw] * kLn2;
+      }
+    } else {
+      sink.store(s, base);
+      base_last = base;
+    }
 
     // ---- online softmax: the running max of a head is shared by the four lane groups -----------
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
@@ -262,13 +273,29 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
-  sink.store_tail(base_last);
+  if (p.stage_scores) {
+    // The chunk's logits, whole rows at a time: no load of this workgroup is in flight any more, so
+    // nothing waits behind these stores.
+    __syncthreads();
+    const int n = t_end - t_begin;
+    for (int g = 0; g < G; ++g) {
+      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + g) * p.score_stride + t_begin;
+      const float *lrow = dyn_lds + g * stage_row;
+      const int n4 = ((((uintptr_t)srow) & 15) == 0) ? n / 4 : 0;  // 16-byte stores where the row allows them
+      for (int t = threadIdx.x; t < n4; t += 64 * kWaves) *(float4_t *)(srow + 4 * t) = *(const float4_t *)(lrow + 4 * t);
+      for (int t = 4 * n4 + threadIdx.x; t < n; t += 64 * kWaves) srow[t] = lrow[t];
+    }
+    __syncthreads();  // the merge below reuses the area
+  } else {
+    sink.store_tail(base_last);
+  }
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  __shared__ float lds_m[kWaves][16], lds_l[kWaves][16];
-  __shared__ float lds_acc[kWaves][SH::MAXH][D + 4];
+  float (*lds_m)[16] = (float (*)[16])dyn_lds;
+  float (*lds_l)[16] = lds_m + kWaves;
+  float (*lds_acc)[SH::MAXH][D + 4] = (float (*)[SH::MAXH][D + 4])(dyn_lds + 2 * kWaves * 16);
   if (j == 0) {
     lds_m[wave][r] = m_run;
     lds_l[wave][r] = l_run;
@@ -317,9 +344,25 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
     ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves, 0));
     wgs_per_cu = std::max(1, n);
   }
-  choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu);
+  // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
+  // token loop is over (kStageBytes; two workgroups per CU still fit).
+  constexpr int kStageBytes = 64 * 1024;
+  const int max_chunk = p.scores ? (kStageBytes / 4 / p.group - 4) / tile_rows * tile_rows : 0;
+  choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   const int nsplit = p.nsplit;
   p.direct = 0;
+  p.stage_scores = p.scores && p.chunk <= max_chunk;
+  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * MfmaShape<D>::MAXH * (D + 4)) * sizeof(float);
+  const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
+  static bool lds_limit_raised = false;
+  if (!lds_limit_raised) {
+    constexpr int kLimit = kStageBytes + 1024;
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    lds_limit_raised = true;
+  }
   const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
   const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
   int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
@@ -330,10 +373,10 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
     KernelTimer timer(ctx, stream);
     const dim3 grid(nsplit, p.n_heads_kv, batch), block(64 * kWaves);
     const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-    if (cap && indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, true>), grid, block, 0, stream, p);
-    else if (cap) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, false>), grid, block, 0, stream, p);
-    else if (indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, false>), grid, block, 0, stream, p);
+    if (cap && indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, true>), grid, block, lds_bytes, stream, p);
+    else if (cap) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, false>), grid, block, lds_bytes, stream, p);
+    else if (indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, true>), grid, block, lds_bytes, stream, p);
+    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, false>), grid, block, lds_bytes, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
