@@ -102,6 +102,19 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   // outputs are requested before the (m, l) pairs that weight them.  Slots past the last split
   // re-read it and get weight zero.
   const int last = p.nsplit - 1;
+  // The logits of the workgroup's slice of the score row are requested first of all (the usual
+  // slice is 2048 tokens, kAhead per thread), so the rewrite does not start a second round trip
+  // once the row's maximum and sum are known.
+  constexpr int kAhead = 8;
+  float *srow = p.scores ? p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride : nullptr;
+  const int slice = ((p.len + (int)gridDim.z - 1) / (int)gridDim.z + 255) / 256 * 256;
+  const int t_end = min(p.len, ((int)blockIdx.z + 1) * slice);
+  const int t0 = (int)blockIdx.z * slice + (int)threadIdx.x;
+  float logit[kAhead];
+  if (p.scores) {
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) logit[k] = srow[min(t0 + 256 * k, p.len - 1)];
+  }
   float4_t part[PER];
   if (first) {
 #pragma unroll
@@ -161,10 +174,12 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     }
   }
   if (p.scores) {
-    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    const int slice = ((p.len + (int)gridDim.z - 1) / (int)gridDim.z + 255) / 256 * 256;
-    const int t_end = min(p.len, ((int)blockIdx.z + 1) * slice);
-    for (int t = (int)blockIdx.z * slice + threadIdx.x; t < t_end; t += 256) srow[t] = __expf(srow[t] - mm) * inv;
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+      const int t = t0 + 256 * k;
+      if (t < t_end) srow[t] = __expf(logit[k] - mm) * inv;
+    }
+    for (int t = t0 + 256 * kAhead; t < t_end; t += 256) srow[t] = __expf(srow[t] - mm) * inv;
   }
 }
 

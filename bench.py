@@ -103,7 +103,7 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
                 gbps_wall=nbytes / wall / 1e9, gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None)
 
 
-def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1):
+def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1, scores=False):
     """Decode attention over a block-quantised cache (q4_0 / q8_0 / q2_0 rows of 18- / 34- / 12-byte blocks):
     synthetic blocks (random codes, f16 scales sized for N(0,1)-like values); algorithmic bytes are
     the attended block rows of K and V plus Q and out."""
@@ -127,12 +127,14 @@ def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1)
     vs = [blocks() for _ in range(rotate)]
     q = torch.randn((batch, hq, d), generator=g, device="cuda", dtype=torch.float32)
     out = torch.empty((batch, hq, d), device="cuda", dtype=torch.float32)
+    sc = torch.empty((batch, hq, L), device="cuda", dtype=torch.float32) if scores else None
     state = {"i": 0}
 
     def step():
         i = state["i"] % rotate
         state["i"] += 1
-        ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, L, batch=batch, kv_batch_stride=hkv * L * d, kv_dtype=kv_dtype)
+        ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, L, batch=batch, kv_batch_stride=hkv * L * d, kv_dtype=kv_dtype,
+                          scores=sc, score_stride=L if scores else 0)
 
     spin_up(step)
     for _ in range(warmup):
@@ -146,7 +148,7 @@ def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1)
     wall = (time.perf_counter() - t0) / steps
     kms = ctx.kernel_timing_end(steps)
     kernel_ms = sum(kms) / max(len(kms), 1)
-    nbytes = batch * (2 * hkv * L * row_bytes + 2 * hq * d * 4)
+    nbytes = batch * (2 * hkv * L * row_bytes + 2 * hq * d * 4 + (hq * L * 4 if scores else 0))
     return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
                 gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None,
                 f16_equivalent_gbps_kernel=decode_bytes(hq, hkv, d, L, batch, 2, False) / (kernel_ms * 1e-3) / 1e9)
@@ -456,6 +458,8 @@ def main():
             "4 KV buffer sets rotated (512 MiB > Infinity Cache)")
         add("cfg3_L4096_b16", bench_decode(ctx, 32, 8, 128, 4096, 16, es, ew, rotate=2), "2 sets rotated")
         add("cfg3_L4096_b1", bench_decode(ctx, 32, 8, 128, 4096, 1, es, ew, rotate=16), "16 sets rotated")
+        add("cfg3_L32768_b16_scores", bench_decode(ctx, 32, 8, 128, 32768, 16, es, ew, scores=True),
+            "scores emitted (67 MB of logits per call); kernel time covers the split pass only, us_per_call the combine's rewrite too")
         add("cfg1_qwen_L1024_b1", bench_decode(ctx, 14, 2, 64, 1024, 1, es, ew), "latency-bound (0.5 MiB)")
         add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
             bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=4),
@@ -469,6 +473,8 @@ def main():
             "32 caches (sequences) per launch, 629 MB: amortised rate")
         add("cfg3_q4_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q4_0 rows attended in-kernel, 604 MB of blocks")
+        add("cfg3_q4_0_blocks_L32768_b16_scores", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew, scores=True),
+            "q4_0 rows with scores emitted (67 MB of logits per call)")
         add("cfg3_q8_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q8_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q8_0 rows attended in-kernel, 1141 MB of blocks")
         add("cfg3_q2_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q2_0", 32, 8, 128, 32768, 16, es, ew),
