@@ -364,8 +364,12 @@ struct BlockShape {
   static constexpr int MAXH = (D == 256) ? 8 : 16;        // query heads per KV head (bounds the merge LDS)
 };
 
+// Waves per SIMD the register allocation aims at: 4 at head_dim 64 (128 registers), 3 at 128 (168;
+// q8_0 would spill there and stays at 2), 2 at 256.  Without the bound most instantiations came out a
+// few registers on one or the other side of a step depending on unrelated edits (q4_0 at 128: 165 or
+// 170 registers; q8_0 at 256: 256 or 257).
 template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED>
-__global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
   using CD = Codec<FMT>;
@@ -555,7 +559,16 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
+  // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
+  // then the merge area.
+  extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
+  const int stage_row = p.chunk + 4;
+  const int staged_heads = p.stage_scores ? p.group : 0;
   __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
+  // Lanes that park nothing write here: the sink's stage when the logits are staged (the sink is off
+  // then), else the start of the dynamic area (the merge uses it after the loop only).
+  static_assert(sizeof(logit_stage) >= 64 * kWaves * TW * 16, "spare slots of 16 TW bytes per lane");
+  float *spare = p.stage_scores ? &logit_stage[0][0] : dyn_lds;
   const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
   int base_last = -(1 << 30);
 
@@ -646,6 +659,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
         s[tw][i] = fmaxf(s[tw][i], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
         mt = fmaxf(mt, s[tw][i]);
       }
+    // Staged or not, the iteration issues the sink's one store (dropped when it has nothing to write):
+    // a store on one side of a branch only would make the compiler's wait counts inexact.
+    stage_logits<TW>(dyn_lds, stage_row, r, j, staged_heads, base - t_begin, s, spare);
     sink.store(s, base);
     base_last = base;
 
@@ -753,7 +769,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
     load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
-  sink.store_tail(base_last);
+  if (p.stage_scores) {
+    flush_staged_logits(p, dyn_lds, stage_row, b, kvh * G, G, t_begin, t_end);
+  } else {
+    sink.store_tail(base_last);
+    __syncthreads();  // the other waves' spare slots lie in the merge area
+  }
 
   if constexpr (kHdrTerm) {
     constexpr float kTerm = (FMT == kFmtQ4_0) ? -CD::kZero : 1.0f;
@@ -768,8 +789,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_blocks_kernel(const Decode
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  __shared__ float lds_m[kWaves][16], lds_l[kWaves][16];
-  __shared__ float lds_acc[kWaves][SH::MAXH][D + 4];
+  float (*lds_m)[16] = (float (*)[16])dyn_lds;
+  float (*lds_l)[16] = lds_m + kWaves;
+  float (*lds_acc)[SH::MAXH][D + 4] = (float (*)[SH::MAXH][D + 4])(dyn_lds + 2 * kWaves * 16);
   if (j == 0) {
     lds_m[wave][r] = m_run;
     lds_l[wave][r] = l_run;
@@ -819,8 +841,24 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
     ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_blocks_kernel<FMT, D, TW, false, false>, 64 * kWaves, 0));
     wgs_per_cu = std::max(1, n);
   }
-  choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu);
+  // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
+  // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips).
+  constexpr int kStageBytes = 48 * 1024;
+  const int max_chunk = staged_chunk_limit(p, kStageBytes, tile_rows);
+  choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   p.direct = 0;
+  p.stage_scores = p.scores && p.chunk <= max_chunk;
+  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * BlockShape<D>::MAXH * (D + 4)) * sizeof(float);
+  const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
+  static bool lds_limit_raised = false;
+  if (!lds_limit_raised) {
+    constexpr int kLimit = kStageBytes + 1024;
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
+    lds_limit_raised = true;
+  }
   const size_t n_part = (size_t)batch * p.n_heads_q * p.nsplit;
   const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
   int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
@@ -831,10 +869,10 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
     KernelTimer timer(ctx, stream);
     const dim3 grid(p.nsplit, p.n_heads_kv, batch), block(64 * kWaves);
     const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-    if (cap && indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, true>), grid, block, 0, stream, p);
-    else if (cap) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, false>), grid, block, 0, stream, p);
-    else if (indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, false>), grid, block, 0, stream, p);
+    if (cap && indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, true>), grid, block, lds_bytes, stream, p);
+    else if (cap) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, false>), grid, block, lds_bytes, stream, p);
+    else if (indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, true>), grid, block, lds_bytes, stream, p);
+    else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, false>), grid, block, lds_bytes, stream, p);
   }
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<BlockFallback<FMT>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);

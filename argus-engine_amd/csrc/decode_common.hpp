@@ -228,10 +228,10 @@ struct LogitSink {
 
   __device__ __forceinline__ LogitSink(const DecodeParams &p, float *stage, int b, int first_head, int heads, int lane, int t_end_)
       : t_end(t_end_) {
-    const uint32_t bytes = p.scores ? (uint32_t)((((int64_t)heads - 1) * p.score_stride + t_end_) * 4) : 0u;
-    void *rows = p.scores ? (void *)(p.scores + (int64_t)b * p.score_bs + (int64_t)first_head * p.score_stride) : nullptr;
+    on = p.scores != nullptr && !p.stage_scores;  // staged logits are written after the loop: every store here is dropped
+    const uint32_t bytes = on ? (uint32_t)((((int64_t)heads - 1) * p.score_stride + t_end_) * 4) : 0u;
+    void *rows = on ? (void *)(p.scores + (int64_t)b * p.score_bs + (int64_t)first_head * p.score_stride) : nullptr;
     rsrc = __builtin_amdgcn_make_buffer_rsrc(rows, 0, bytes, 0x00020000);
-    on = p.scores != nullptr;
     wide = heads > 8;
     tok = VEC * (lane & 7);
 #pragma unroll
@@ -282,6 +282,40 @@ struct LogitSink {
       }
   }
 };
+// Staged score emission (DecodeParams::stage_scores): lane (j, r) parks a tile's four logits of head r
+// in the workgroup's dynamic LDS, rows of `stage_row` floats per head, and the workgroup writes the
+// chunk's rows once its token loop is over, when none of its loads is in flight any more.
+// Branch-free on purpose (a branch here cuts the token loop's one basic block in two, and the
+// block-cache kernels then lose 10 % of their rate): lanes with nothing to park (heads past the
+// group, or staging off: `staged_heads` 0) write to a 16 TW-byte slot of their own in `spare`, an
+// area of 64 TW bytes per wave lane that nothing else uses during the loop.
+template <int TW>
+__device__ __forceinline__ void stage_logits(float *stage, int stage_row, int r, int j, int staged_heads, int tok, const float4_t (&s)[TW],
+                                             float *spare) {
+  constexpr float kLn2 = 0.6931471805599453f;
+  const bool parks = r < staged_heads;
+  float *dst = parks ? stage + r * stage_row + tok + 4 * j : spare + 4 * TW * (int)threadIdx.x;
+  const int step = parks ? 16 : 4;
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw) *(float4_t *)(dst + step * tw) = s[tw] * kLn2;
+}
+__device__ __forceinline__ void flush_staged_logits(const DecodeParams &p, const float *stage, int stage_row, int b, int first_head,
+                                                    int heads, int t_begin, int t_end) {
+  __syncthreads();
+  const int n = t_end - t_begin;
+  for (int g = 0; g < heads; ++g) {
+    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(first_head + g) * p.score_stride + t_begin;
+    const float *lrow = stage + g * stage_row;
+    const int n4 = ((((uintptr_t)srow) & 15) == 0) ? n / 4 : 0;  // 16-byte stores where the row allows them
+    for (int t = threadIdx.x; t < n4; t += blockDim.x) *(float4_t *)(srow + 4 * t) = *(const float4_t *)(lrow + 4 * t);
+    for (int t = 4 * n4 + threadIdx.x; t < n; t += blockDim.x) srow[t] = lrow[t];
+  }
+  __syncthreads();  // the caller reuses the area
+}
+// Longest chunk whose logits fit `stage_bytes` of LDS (0 without scores), for choose_splits().
+inline int staged_chunk_limit(const DecodeParams &p, int stage_bytes, int tile_rows) {
+  return p.scores ? (stage_bytes / 4 / p.group - 4) / tile_rows * tile_rows : 0;
+}
 inline bool score_rows_addressable(const DecodeParams &p) {
   return !p.scores || (p.score_stride >= p.len && ((int64_t)p.group * p.score_stride + 1024) * 4 <= 0x7fffffffll);
 }

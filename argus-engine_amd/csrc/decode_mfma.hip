@@ -179,7 +179,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
   // then the merge area.
   extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
   const int stage_row = p.chunk + 4;
+  const int staged_heads = p.stage_scores ? p.group : 0;
   __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
+  // Lanes that park nothing write here: the sink's stage when the logits are staged (the sink is off
+  // then), else the start of the dynamic area (the merge uses it after the loop only).
+  static_assert(sizeof(logit_stage) >= 64 * kWaves * TW * 16, "spare slots of 16 TW bytes per lane");
+  float *spare = p.stage_scores ? &logit_stage[0][0] : dyn_lds;
   const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
 
   float4_t o_acc[NACC];
@@ -220,15 +225,11 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
         s[tw][i] = sv;
         mt = fmaxf(mt, sv);
       }
-    if (p.stage_scores) {  // uniform; LDS only
-      if (r < G) {
-#pragma unroll
-        for (int tw = 0; tw < TW; ++tw) *(float4_t *)(dyn_lds + r * stage_row + (base - t_begin) + 16 * tw + 4 * j) = s[tw] * kLn2;
-      }
-    } else {
-      sink.store(s, base);
-      base_last = base;
-    }
+    // Staged or not, the iteration issues the sink's one store (dropped when it has nothing to write):
+    // a store on one side of a branch only would make the compiler's wait counts inexact.
+    stage_logits<TW>(dyn_lds, stage_row, r, j, staged_heads, base - t_begin, s, spare);
+    sink.store(s, base);
+    base_last = base;
 
     // ---- online softmax: the running max of a head is shared by the four lane groups -----------
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
@@ -274,20 +275,10 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
     load_idx_v(base + 2 * kWaves * TILE);
   }
   if (p.stage_scores) {
-    // The chunk's logits, whole rows at a time: no load of this workgroup is in flight any more, so
-    // nothing waits behind these stores.
-    __syncthreads();
-    const int n = t_end - t_begin;
-    for (int g = 0; g < G; ++g) {
-      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(kvh * G + g) * p.score_stride + t_begin;
-      const float *lrow = dyn_lds + g * stage_row;
-      const int n4 = ((((uintptr_t)srow) & 15) == 0) ? n / 4 : 0;  // 16-byte stores where the row allows them
-      for (int t = threadIdx.x; t < n4; t += 64 * kWaves) *(float4_t *)(srow + 4 * t) = *(const float4_t *)(lrow + 4 * t);
-      for (int t = 4 * n4 + threadIdx.x; t < n; t += 64 * kWaves) srow[t] = lrow[t];
-    }
-    __syncthreads();  // the merge below reuses the area
+    flush_staged_logits(p, dyn_lds, stage_row, b, kvh * G, G, t_begin, t_end);
   } else {
     sink.store_tail(base_last);
+    __syncthreads();  // the other waves' spare slots lie in the merge area
   }
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
@@ -347,7 +338,7 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
   // token loop is over (kStageBytes; two workgroups per CU still fit).
   constexpr int kStageBytes = 64 * 1024;
-  const int max_chunk = p.scores ? (kStageBytes / 4 / p.group - 4) / tile_rows * tile_rows : 0;
+  const int max_chunk = staged_chunk_limit(p, kStageBytes, tile_rows);
   choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   const int nsplit = p.nsplit;
   p.direct = 0;
