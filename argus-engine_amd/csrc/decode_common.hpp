@@ -5,6 +5,8 @@
 #include "argus_hip_internal.hpp"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 namespace argus_decode {
@@ -313,8 +315,13 @@ __device__ __forceinline__ void flush_staged_logits(const DecodeParams &p, const
   __syncthreads();  // the caller reuses the area
 }
 // Longest chunk whose logits fit `stage_bytes` of LDS (0 without scores), for choose_splits().
+// ARGUS_HIP_SCORES=direct (read at every call with scores) keeps the stores in the token loop, the
+// path of chunks too long to stage: for A/B measurements and for tests of that path at small sizes.
 inline int staged_chunk_limit(const DecodeParams &p, int stage_bytes, int tile_rows) {
-  return p.scores ? (stage_bytes / 4 / p.group - 4) / tile_rows * tile_rows : 0;
+  if (!p.scores) return 0;
+  const char *e = getenv("ARGUS_HIP_SCORES");
+  if (e && strcmp(e, "direct") == 0) return 0;
+  return (stage_bytes / 4 / p.group - 4) / tile_rows * tile_rows;
 }
 inline bool score_rows_addressable(const DecodeParams &p) {
   return !p.scores || (p.score_stride >= p.len && ((int64_t)p.group * p.score_stride + 1024) * 4 <= 0x7fffffffll);

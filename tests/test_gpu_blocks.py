@@ -66,6 +66,17 @@ def test_score_rows_with_padding_stay_untouched_past_the_length(L):
     run_case("q4_1", 8, 4, 256, L, score_pad=7, seed=L + 2)
 
 
+@pytest.mark.parametrize("L", [509, 511, 1021, 2051])
+def test_scores_stored_inside_the_token_loop(L, monkeypatch):
+    # the path of chunks too long for the LDS stage, taken at test sizes through ARGUS_HIP_SCORES=direct
+    monkeypatch.setenv("ARGUS_HIP_SCORES", "direct")
+    run_case("q4_0", 8, 2, 128, L, score_pad=5, seed=L)
+    run_case("q8_0", 14, 2, 64, L, score_pad=3, seed=L + 1)
+    run_case("q4_1", 8, 4, 256, L, score_pad=7, seed=L + 2)
+    run_case("q2_0", 12, 1, 128, L, score_pad=1, seed=L + 3)
+    run_case("q4_0", 32, 2, 64, L, score_pad=2, seed=L + 4)
+
+
 @pytest.mark.parametrize("fmt", ["q4_0", "q2_0"])
 def test_scores_of_groups_wider_than_eight_heads(fmt):
     run_case(fmt, 12, 1, 128, 1531, score_pad=1)

@@ -310,3 +310,20 @@ def test_argument_errors_return_negative_codes():
     sc = torch.zeros((4, 4), device="cuda")
     assert c.attention_gen(q, k, k, out, 2, 8, 8, scores=sc, score_stride=4, check=False) == A.ERR_INVALID
     assert "score_stride" in c.last_error()
+
+
+@pytest.mark.parametrize("hq,hkv,d,L", [(8, 2, 64, 1023), (8, 2, 64, 1025), (12, 2, 128, 2047), (12, 2, 128, 2500),
+                                        (32, 8, 128, 300), (24, 2, 128, 1531), (32, 2, 64, 4097), (16, 2, 128, 66)])
+def test_scores_stored_inside_the_token_loop(hq, hkv, d, L, monkeypatch):
+    # Chunks too long for the LDS stage (beyond ~100K tokens at wide groups) write their logits from
+    # inside the token loop; ARGUS_HIP_SCORES=direct takes that path at test sizes.  Odd strides, rows
+    # cut inside a lane's token group, groups wider than eight heads.
+    monkeypatch.setenv("ARGUS_HIP_SCORES", "direct")
+    cap = L + 19
+    q = normal((hq, d), 42 + L)
+    k, v = f16(normal((hkv, cap, d), 137 + L)), f16(normal((hkv, cap, d), 53 + L))
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, score_stride=cap)
+    ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, scores_stride=cap)
+    check_attention_out(got, ref, "out")
+    check_scores(sc[:, :L], p[:, :L], "scores")
+    assert np.all(sc[:, L:] == -7.0), "score columns beyond cache_seq_len must stay untouched"
