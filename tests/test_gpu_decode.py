@@ -146,6 +146,31 @@ def test_softcap_index_and_window_start():
     check_attention_out(got, ref)
 
 
+@pytest.mark.parametrize("L", [2, 33, 65])
+def test_scores_of_a_short_row_are_normalised_by_the_unrounded_sum(L):
+    # The matrix cores consume f16-rounded weights; the scores are exp / sum(exp) in f32.  Over a few
+    # dozen tokens a sum of the rounded weights differs from the f32 sum by up to 2^-12 and moved every
+    # score of a head past the 1e-4 bar (Hq48 Hkv8 d128 L65, soft-cap 30: 1.07e-4 on two heads).
+    # Inputs follow that draw: generator 1100269, Q doubled, window starting at slot 1 of capacity L+6.
+    hq, hkv, d, cap, start = 48, 8, 128, L + 6, 1
+    rng = np.random.default_rng(1100269)
+    shape = [int(rng.choice([64, 128, 256])), int(rng.choice([1, 2, 3, 4, 8])), int(rng.choice([1, 2, 3, 4, 6, 7, 8, 12, 16])),
+             int(rng.choice([1, 3, 17, 63, 64, 65, 100, 257, 700, 1500, 4097, 9000, 20000]))]
+    assert shape == [128, 8, 6, 65]  # the draws that picked the shape, so that Q, K and V are that case's
+    rng.integers(0, 50), rng.choice(["f16", "f32", "q4_0", "q4_1", "q8_0", "q2_0"]), rng.integers(0, 2)
+    rng.choice([0.0, 0.0, 7.0, 30.0]), rng.integers(0, 3), rng.integers(0, 7), rng.integers(0, 4)
+    q = rng.standard_normal((hq, d)).astype(np.float32) * np.float32(2.0)
+    k = f16(rng.standard_normal((hkv, cap, d)).astype(np.float32))
+    v = f16(rng.standard_normal((hkv, cap, d)).astype(np.float32))
+    for softcap in (30.0, 0.0):
+        got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, softcap=softcap, kv_start=start)
+        ref, p = O.attention_gen(q, np.ascontiguousarray(k[:, start:]), np.ascontiguousarray(v[:, start:]), hkv, L,
+                                 cap - start, scores=True, softcap=softcap)
+        check_attention_out(got, ref)
+        check_scores(sc, p)
+        assert np.abs(sc.sum(axis=1) - 1.0).max() < 1e-5
+
+
 @pytest.mark.parametrize("hq,hkv,d,L,cap", [(32, 8, 128, 1500, 1536), (14, 2, 64, 777, 800)])
 def test_softcap_on_the_matrix_core_path(hq, hkv, d, L, cap):
     # F16 KV, no index list, d in {64, 128}: soft-capped logits run through the MFMA kernel; same
