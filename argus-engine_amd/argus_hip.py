@@ -22,6 +22,8 @@ EXPORTED_SYMBOLS = [
     "argus_hip_get_device_info", "argus_hip_kernel_timing_begin", "argus_hip_kernel_timing_end",
     "argus_hip_malloc", "argus_hip_free", "argus_hip_write_buffer",
     "argus_hip_read_buffer", "argus_hip_copy_slice", "argus_hip_synchronize",
+    "argus_hip_create_ex", "argus_hip_reserve_workspace", "argus_hip_kernel_timing_end2",
+    "argus_hip_write_buffer_range", "argus_hip_buffer_shift", "argus_hip_last_decode_plan",
     "argus_hip_attention_gen", "argus_hip_flash_attention_prefill", "argus_hip_prefill_attention_scores",
     "argus_hip_has_quant_attn_kernel", "argus_hip_attention_gen_quant",
     "argus_hip_attention_gen_quant_ex", "argus_hip_gather_update_quant", "argus_hip_quant_flush",
@@ -48,6 +50,17 @@ class DeviceInfo(C.Structure):
     _fields_ = [("compute_units", C.c_int32), ("clock_mhz", C.c_int32),
                 ("wavefront_size", C.c_int32), ("lds_bytes_per_block", C.c_int32),
                 ("hbm_bytes", C.c_int64), ("name", C.c_char * 128), ("gcn_arch", C.c_char * 64)]
+
+
+class CreateOpts(C.Structure):
+    _fields_ = [("max_batch", C.c_int32), ("max_heads_q", C.c_int32), ("max_head_dim", C.c_int32),
+                ("max_seq_len", C.c_int32)]
+
+
+class DecodePlan(C.Structure):
+    _fields_ = [("nsplit", C.c_int32), ("chunk", C.c_int32), ("wgs_per_cu", C.c_int32),
+                ("lds_bytes", C.c_int32), ("launches", C.c_int32), ("kernel", C.c_int32),
+                ("staged_scores", C.c_int32)]
 
 
 class AttentionGenArgs(C.Structure):
@@ -140,6 +153,12 @@ class ScoreReduceArgs(C.Structure):
 def _bind():
     vp, i32 = C.c_void_p, C.c_int32
     lib.argus_hip_create.argtypes = [C.c_int, C.POINTER(vp)]
+    lib.argus_hip_create_ex.argtypes = [C.c_int, C.POINTER(CreateOpts), C.POINTER(vp)]
+    lib.argus_hip_reserve_workspace.argtypes = [vp, C.c_size_t]
+    lib.argus_hip_kernel_timing_end2.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(C.c_float), i32, C.POINTER(i32)]
+    lib.argus_hip_write_buffer_range.argtypes = [vp, vp, vp, C.c_size_t, vp, C.c_size_t]
+    lib.argus_hip_buffer_shift.argtypes = [vp, vp, vp, vp, C.c_size_t]
+    lib.argus_hip_last_decode_plan.argtypes = [vp, C.POINTER(DecodePlan)]
     lib.argus_hip_destroy.argtypes = [vp]
     lib.argus_hip_abi_version.argtypes = []
     lib.argus_hip_last_error.argtypes = [vp]
@@ -207,9 +226,13 @@ class Context:
     """Owns one argus_hip_ctx.  Methods take torch CUDA tensors and return the C return code
     (raising ArgusHipError on a negative one unless check=False)."""
 
-    def __init__(self, device=0):
+    def __init__(self, device=0, max_batch=0, max_heads_q=0, max_head_dim=0, max_seq_len=0):
         h = C.c_void_p()
-        rc = lib.argus_hip_create(device, C.byref(h))
+        if max_batch or max_heads_q or max_head_dim or max_seq_len:
+            opts = CreateOpts(max_batch, max_heads_q, max_head_dim, max_seq_len)
+            rc = lib.argus_hip_create_ex(device, C.byref(opts), C.byref(h))
+        else:
+            rc = lib.argus_hip_create(device, C.byref(h))
         if rc != OK:
             raise ArgusHipError(rc, "argus_hip_create failed (no HIP device?)")
         self.handle = h
@@ -247,6 +270,36 @@ class Context:
         n = C.c_int32(0)
         self._check(lib.argus_hip_kernel_timing_end(self.handle, buf, capacity, C.byref(n)))
         return [buf[i] for i in range(min(n.value, capacity))]
+
+    def kernel_timing_end2(self, capacity=4096):
+        """(dominant-kernel ms, tail ms) per call: the tail is the combine pass of a split-KV decode."""
+        buf, tail = (C.c_float * capacity)(), (C.c_float * capacity)()
+        n = C.c_int32(0)
+        self._check(lib.argus_hip_kernel_timing_end2(self.handle, buf, tail, capacity, C.byref(n)))
+        m = min(n.value, capacity)
+        return [buf[i] for i in range(m)], [tail[i] for i in range(m)]
+
+    def last_decode_plan(self):
+        p = DecodePlan()
+        self._check(lib.argus_hip_last_decode_plan(self.handle, C.byref(p)))
+        return {f: getattr(p, f) for f, _ in DecodePlan._fields_}
+
+    def reserve_workspace(self, nbytes):
+        return self._check(lib.argus_hip_reserve_workspace(self.handle, nbytes))
+
+    def buffer_shift(self, t, src_offset, dst_offset, count, check=True):
+        """Backend::buffer_shift: move `count` elements inside tensor `t` (memmove semantics)."""
+        es = t.element_size()
+        base = t.data_ptr()
+        return self._check(lib.argus_hip_buffer_shift(self.handle, _stream(), base + dst_offset * es, base + src_offset * es,
+                                                      count * es), check)
+
+    def copy_slice(self, dst, src, nbytes, check=True):
+        return self._check(lib.argus_hip_copy_slice(self.handle, _stream(), dst, src, nbytes), check)
+
+    def write_buffer_range(self, t, dst_offset_bytes, host_array, check=True):
+        return self._check(lib.argus_hip_write_buffer_range(self.handle, _stream(), t.data_ptr(), dst_offset_bytes,
+                                                            host_array.ctypes.data, host_array.nbytes), check)
 
     # -- (a-1) ---------------------------------------------------------------------------
     def attention_gen(self, q, k, v, out, num_heads_kv, cache_seq_len, capacity=0,

@@ -13,36 +13,69 @@
 
 #define ARGUS_API extern "C" __attribute__((visibility("default")))
 
+// Environment switches, read once when the context is created.
+struct ArgusEnv {
+  bool decode_valu = false;    // ARGUS_HIP_DECODE=valu: vector-ALU decode kernel for A/B measurements
+  bool scores_direct = false;  // ARGUS_HIP_SCORES=direct: score stores stay in the token loop
+  bool kivi_valu = false;      // ARGUS_HIP_KIVI=valu: vector-ALU KIVI kernel
+};
+
+// What a launcher has learnt about one kernel on this context's device: resident workgroups per
+// compute unit at the LDS size it launches with, and whether the dynamic-LDS limit was raised.
+struct KernelFacts {
+  const void *fn;
+  uint32_t lds_bytes;
+  int wgs_per_cu;
+};
+
 struct argus_hip_ctx {
   int device = 0;
   int compute_units = 0;
   hipDeviceProp_t props;
+  ArgusEnv env;
   // Split-KV partial workspace: per (sequence, Q head, split) one (m, l) pair and one
-  // un-normalised output row.  Grown on demand, never shrunk.
+  // un-normalised output row.  Sized at creation (argus_hip_create_ex) or by
+  // argus_hip_reserve_workspace; a call that needs more grows it, which stalls the device.
   float *ws = nullptr;
   size_t ws_bytes = 0;
-  // Event pairs of argus_hip_kernel_timing_begin/_end; ev_used counts events handed out.
+  // Scratch of the PFA side channel (logits of the trailing query rows); freed after a call that
+  // made it large.
+  float *pfa_ws = nullptr;
+  size_t pfa_ws_bytes = 0;
+  // Per-device launch facts (the kernels' function attributes are per device).
+  std::vector<KernelFacts> facts;
+  std::vector<const void *> lds_raised;
+  // How the last split-KV decode call was cut (argus_hip_last_decode_plan).
+  argus_hip_decode_plan plan = {};
+  // Event triples of argus_hip_kernel_timing_begin/_end: before the dominant kernel, after it,
+  // after the combine pass (or whatever else the call launched).
   std::vector<hipEvent_t> ev;
   size_t ev_used = 0;
   bool timing = false;
   char err[512] = {0};
 };
 
-// Brackets the launches issued during its lifetime with one event pair when timing is armed.
+// Brackets the launches issued during its lifetime when timing is armed: mark() closes the first
+// interval (the dominant kernel), the destructor the second (the combine pass).
 struct KernelTimer {
   argus_hip_ctx *ctx;
   hipStream_t stream;
-  bool on;
-  KernelTimer(argus_hip_ctx *c, hipStream_t s) : ctx(c), stream(s), on(false) {
-    if (c->timing && c->ev_used + 2 <= c->ev.size()) {
+  bool on, marked;
+  KernelTimer(argus_hip_ctx *c, hipStream_t s) : ctx(c), stream(s), on(false), marked(false) {
+    if (c->timing && c->ev_used + 3 <= c->ev.size()) {
       on = true;
       (void)hipEventRecord(c->ev[c->ev_used], s);
     }
   }
+  void mark() {
+    if (on && !marked) (void)hipEventRecord(ctx->ev[ctx->ev_used + 1], stream);
+    marked = true;
+  }
   ~KernelTimer() {
     if (on) {
-      (void)hipEventRecord(ctx->ev[ctx->ev_used + 1], stream);
-      ctx->ev_used += 2;
+      if (!marked) (void)hipEventRecord(ctx->ev[ctx->ev_used + 1], stream);
+      (void)hipEventRecord(ctx->ev[ctx->ev_used + 2], stream);
+      ctx->ev_used += 3;
     }
   }
 };
@@ -67,6 +100,32 @@ inline int argus_fail(argus_hip_ctx *ctx, int code, const char *fmt, ...) {
 // Ensures the context workspace holds at least `bytes`; reallocation frees the old buffer
 // (hipFree synchronises the device, so no launch still reads it).
 int argus_ws_reserve(argus_hip_ctx *ctx, size_t bytes);
+inline float *argus_ws(argus_hip_ctx *ctx) { return ctx->ws; }
+
+// Resident workgroups per compute unit of `fn` at `block` threads and `lds_bytes` of dynamic LDS,
+// queried once per (kernel, LDS size) on this context.
+template <typename F>
+int argus_wgs_per_cu(argus_hip_ctx *ctx, F fn, int block, size_t lds_bytes) {
+  for (const KernelFacts &k : ctx->facts)
+    if (k.fn == (const void *)fn && k.lds_bytes == (uint32_t)lds_bytes) return k.wgs_per_cu;
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, block, lds_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    n = 1;
+  }
+  n = n < 1 ? 1 : n;
+  ctx->facts.push_back(KernelFacts{(const void *)fn, (uint32_t)lds_bytes, n});
+  return n;
+}
+// Raises the dynamic-LDS limit of `fn` to `bytes`, once per kernel on this context.
+template <typename F>
+hipError_t argus_raise_lds_limit(argus_hip_ctx *ctx, F fn, int bytes) {
+  for (const void *k : ctx->lds_raised)
+    if (k == (const void *)fn) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) ctx->lds_raised.push_back((const void *)fn);
+  return e;
+}
 
 #if defined(__HIPCC__)
 // ---- wave64 cross-lane helpers ------------------------------------------------------------

@@ -1,6 +1,8 @@
 // Context, device query and the memory helpers behind the engine's Memory / Buffer impls.
 #include "argus_hip_internal.hpp"
 
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -21,9 +23,17 @@ int argus_ws_reserve(argus_hip_ctx *ctx, size_t bytes) {
 
 ARGUS_API int argus_hip_abi_version(void) { return ARGUS_HIP_ABI_VERSION; }
 
-ARGUS_API int argus_hip_create(int device, argus_hip_ctx **out) {
+namespace {
+bool env_is(const char *name, const char *value) {
+  const char *e = getenv(name);
+  return e && strcmp(e, value) == 0;
+}
+}  // namespace
+
+ARGUS_API int argus_hip_create_ex(int device, const argus_hip_create_opts *opts, argus_hip_ctx **out) {
   if (!out) return ARGUS_HIP_ERR_INVALID;
   *out = nullptr;
+  if (opts && (opts->max_batch < 0 || opts->max_heads_q < 0 || opts->max_head_dim < 0)) return ARGUS_HIP_ERR_INVALID;
   int n = 0;
   if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
     (void)hipGetLastError();
@@ -39,7 +49,18 @@ ARGUS_API int argus_hip_create(int device, argus_hip_ctx **out) {
     return ARGUS_HIP_ERR_RUNTIME;
   }
   ctx->compute_units = ctx->props.multiProcessorCount;
-  int rc = argus_ws_reserve(ctx, (size_t)8 << 20);
+  ctx->env.decode_valu = env_is("ARGUS_HIP_DECODE", "valu");
+  ctx->env.scores_direct = env_is("ARGUS_HIP_SCORES", "direct");
+  ctx->env.kivi_valu = env_is("ARGUS_HIP_KIVI", "valu");
+  // The split-KV partials of the largest call the caller announces: every (sequence, Q head) may be
+  // cut into kMaxSplitsHint pieces of head_dim + 2 floats.  Without a hint 8 MiB, which covers 16
+  // sequences of the Llama-3-8B head shape at the split counts the launchers choose.
+  size_t want = (size_t)8 << 20;
+  if (opts && opts->max_batch > 0 && opts->max_heads_q > 0 && opts->max_head_dim > 0) {
+    const size_t n_part = (size_t)opts->max_batch * opts->max_heads_q * 128;
+    want = std::max(want, n_part * ((size_t)opts->max_head_dim + 2) * sizeof(float) + 256);
+  }
+  int rc = argus_ws_reserve(ctx, want);
   if (rc != ARGUS_HIP_OK) {
     delete ctx;
     return rc;
@@ -48,9 +69,17 @@ ARGUS_API int argus_hip_create(int device, argus_hip_ctx **out) {
   return ARGUS_HIP_OK;
 }
 
+ARGUS_API int argus_hip_create(int device, argus_hip_ctx **out) { return argus_hip_create_ex(device, nullptr, out); }
+
+ARGUS_API int argus_hip_reserve_workspace(argus_hip_ctx *ctx, size_t bytes) {
+  if (!ctx) return ARGUS_HIP_ERR_INVALID;
+  return argus_ws_reserve(ctx, bytes);
+}
+
 ARGUS_API int argus_hip_destroy(argus_hip_ctx *ctx) {
   if (!ctx) return ARGUS_HIP_ERR_INVALID;
   if (ctx->ws) (void)hipFree(ctx->ws);
+  if (ctx->pfa_ws) (void)hipFree(ctx->pfa_ws);
   for (hipEvent_t e : ctx->ev) (void)hipEventDestroy(e);
   delete ctx;
   return ARGUS_HIP_OK;
@@ -70,6 +99,12 @@ ARGUS_API int argus_hip_get_device_info(const argus_hip_ctx *ctx, argus_hip_devi
   info->hbm_bytes = (int64_t)ctx->props.totalGlobalMem;
   strncpy(info->name, ctx->props.name, sizeof(info->name) - 1);
   strncpy(info->gcn_arch, ctx->props.gcnArchName, sizeof(info->gcn_arch) - 1);
+  return ARGUS_HIP_OK;
+}
+
+ARGUS_API int argus_hip_last_decode_plan(const argus_hip_ctx *ctx, argus_hip_decode_plan *plan) {
+  if (!ctx || !plan) return ARGUS_HIP_ERR_INVALID;
+  *plan = ctx->plan;
   return ARGUS_HIP_OK;
 }
 
@@ -107,18 +142,59 @@ ARGUS_API int argus_hip_read_buffer(argus_hip_ctx *ctx, void *stream, void *dst_
   return ARGUS_HIP_OK;
 }
 
+ARGUS_API int argus_hip_write_buffer_range(argus_hip_ctx *ctx, void *stream, void *dst_dev, size_t dst_offset,
+                                           const void *src_host, size_t bytes) {
+  if (!ctx || (bytes && (!dst_dev || !src_host))) return ARGUS_HIP_ERR_INVALID;
+  return argus_hip_write_buffer(ctx, stream, (char *)dst_dev + dst_offset, src_host, bytes);
+}
+
 ARGUS_API int argus_hip_copy_slice(argus_hip_ctx *ctx, void *stream, void *dst_dev,
                                    const void *src_dev, size_t bytes) {
   if (!ctx || (bytes && (!dst_dev || !src_dev))) return ARGUS_HIP_ERR_INVALID;
-  if (!bytes) return ARGUS_HIP_OK;
-  // hipMemcpyAsync handles overlapping device ranges as memmove does not; buffer_shift callers
-  // (engine/src/backend.rs:1119) move towards lower addresses, which a forward copy handles,
-  // but to stay safe for any overlap the shift goes through a non-overlapping check.
+  if (!bytes || dst_dev == src_dev) return ARGUS_HIP_OK;
+  // Backend::copy_slice copies between two tensors (engine/src/backend.rs:1119); ranges that
+  // overlap inside one buffer belong to buffer_shift and are handed over to it.
   const char *s = (const char *)src_dev;
   char *d = (char *)dst_dev;
-  if ((d < s + bytes) && (s < d + bytes) && d != s)
-    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "copy_slice: overlapping ranges");
+  if ((d < s + bytes) && (s < d + bytes)) return argus_hip_buffer_shift(ctx, stream, dst_dev, src_dev, bytes);
   ARGUS_HIP_CHECK(ctx, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+  return ARGUS_HIP_OK;
+}
+
+// Backend::buffer_shift is std::ptr::copy, i.e. memmove (engine/src/backend.rs:1085-1112): the
+// ranges may overlap, as when a cache prefix is pruned or the KIVI residual ring moves its
+// remaining rows to the front (engine/src/kv/quant_window_cache.rs:1820-1841).  The move is cut into
+// pieces that are each a plain copy between disjoint ranges, issued in the order that never
+// overwrites bytes still to be read (ascending addresses when the destination lies below the
+// source, descending otherwise).  A piece is at most as long as the distance between the ranges;
+// when that distance is short the pieces go through the workspace instead (source piece ->
+// workspace -> destination piece), so the number of copies stays bytes / workspace size.
+ARGUS_API int argus_hip_buffer_shift(argus_hip_ctx *ctx, void *stream, void *dst_dev, const void *src_dev, size_t bytes) {
+  if (!ctx || (bytes && (!dst_dev || !src_dev))) return ARGUS_HIP_ERR_INVALID;
+  if (!bytes || dst_dev == src_dev) return ARGUS_HIP_OK;
+  const char *s = (const char *)src_dev;
+  char *d = (char *)dst_dev;
+  hipStream_t st = (hipStream_t)stream;
+  if (!((d < s + bytes) && (s < d + bytes))) {
+    ARGUS_HIP_CHECK(ctx, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, st));
+    return ARGUS_HIP_OK;
+  }
+  const bool forward = d < s;
+  const size_t dist = forward ? (size_t)(s - d) : (size_t)(d - s);
+  constexpr size_t kDirectMin = (size_t)1 << 20;  // pieces shorter than this are staged instead
+  const bool staged = dist < kDirectMin && dist < bytes && ctx->ws_bytes > dist;
+  const size_t piece = staged ? ctx->ws_bytes : dist;
+  const size_t n = (bytes + piece - 1) / piece;
+  for (size_t i = 0; i < n; ++i) {
+    const size_t k = forward ? i : n - 1 - i;
+    const size_t off = k * piece, len = std::min(piece, bytes - off);
+    if (staged) {
+      ARGUS_HIP_CHECK(ctx, hipMemcpyAsync(ctx->ws, s + off, len, hipMemcpyDeviceToDevice, st));
+      ARGUS_HIP_CHECK(ctx, hipMemcpyAsync(d + off, ctx->ws, len, hipMemcpyDeviceToDevice, st));
+    } else {
+      ARGUS_HIP_CHECK(ctx, hipMemcpyAsync(d + off, s + off, len, hipMemcpyDeviceToDevice, st));
+    }
+  }
   return ARGUS_HIP_OK;
 }
 
@@ -130,7 +206,7 @@ ARGUS_API int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream) {
 
 ARGUS_API int argus_hip_kernel_timing_begin(argus_hip_ctx *ctx, int32_t max_launches) {
   if (!ctx || max_launches <= 0) return ARGUS_HIP_ERR_INVALID;
-  while (ctx->ev.size() < (size_t)max_launches * 2) {
+  while (ctx->ev.size() < (size_t)max_launches * 3) {
     hipEvent_t e;
     ARGUS_HIP_CHECK(ctx, hipEventCreate(&e));
     ctx->ev.push_back(e);
@@ -140,14 +216,21 @@ ARGUS_API int argus_hip_kernel_timing_begin(argus_hip_ctx *ctx, int32_t max_laun
   return ARGUS_HIP_OK;
 }
 
-ARGUS_API int argus_hip_kernel_timing_end(argus_hip_ctx *ctx, float *ms_out, int32_t capacity, int32_t *n_out) {
+ARGUS_API int argus_hip_kernel_timing_end2(argus_hip_ctx *ctx, float *ms_out, float *tail_ms_out, int32_t capacity,
+                                           int32_t *n_out) {
   if (!ctx || !n_out || (capacity > 0 && !ms_out)) return ARGUS_HIP_ERR_INVALID;
   ctx->timing = false;
-  const size_t n = ctx->ev_used / 2;
+  const size_t n = ctx->ev_used / 3;
   *n_out = (int32_t)n;
   if (n) ARGUS_HIP_CHECK(ctx, hipEventSynchronize(ctx->ev[ctx->ev_used - 1]));
-  for (size_t i = 0; i < n && i < (size_t)capacity; ++i)
-    ARGUS_HIP_CHECK(ctx, hipEventElapsedTime(&ms_out[i], ctx->ev[2 * i], ctx->ev[2 * i + 1]));
+  for (size_t i = 0; i < n && i < (size_t)capacity; ++i) {
+    ARGUS_HIP_CHECK(ctx, hipEventElapsedTime(&ms_out[i], ctx->ev[3 * i], ctx->ev[3 * i + 1]));
+    if (tail_ms_out) ARGUS_HIP_CHECK(ctx, hipEventElapsedTime(&tail_ms_out[i], ctx->ev[3 * i + 1], ctx->ev[3 * i + 2]));
+  }
   ctx->ev_used = 0;
   return ARGUS_HIP_OK;
+}
+
+ARGUS_API int argus_hip_kernel_timing_end(argus_hip_ctx *ctx, float *ms_out, int32_t capacity, int32_t *n_out) {
+  return argus_hip_kernel_timing_end2(ctx, ms_out, nullptr, capacity, n_out);
 }

@@ -103,7 +103,9 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
       const int t = base + u * RPW + grp;
       valid[u] = FULL || t < t_end;
       const int tc = valid[u] ? t : (t_end - 1);
-      const int64_t slot = use_idx ? (int64_t)idx[tc] : (int64_t)(p.kv_start + tc);
+      // a slot outside the cache (stale or negative list entry) is clamped to the last one: the rows
+      // are fetched with plain loads, which nothing else bounds
+      const int64_t slot = use_idx ? (int64_t)min((uint32_t)idx[tc], (uint32_t)(p.slot_bound - 1)) : (int64_t)(p.kv_start + tc);
       kr[u] = __builtin_nontemporal_load((const vec_t *)(kb + slot * p.row_stride));
       vr[u] = __builtin_nontemporal_load((const vec_t *)(vb + slot * p.row_stride));
     }
@@ -271,24 +273,20 @@ int launch_decode(argus_hip_ctx *ctx, DecodeParams &p, int batch, bool want_scor
   p.direct = (nsplit == 1 && !want_scores) ? 1 : 0;
 
   if (!p.direct) {
-    const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
-    const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
-    int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+    const int rc = reserve_partials(ctx, p, batch, D);
     if (rc != ARGUS_HIP_OK) return rc;
-    p.ws_ml = ctx->ws;
-    p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
   }
+  ctx->plan = argus_hip_decode_plan{nsplit, chunk, 0, 0, p.direct ? 1 : 2, 0, 0};
 
   dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
-  {
-    KernelTimer timer(ctx, stream);
-    if (p.kv_index)
-      hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kGeneric>), grid, dim3(256), 0, stream, p);
-    else if (p.softcap > 0.0f)
-      hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kSoftcap>), grid, dim3(256), 0, stream, p);
-    else
-      hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kPlain>), grid, dim3(256), 0, stream, p);
-  }
+  KernelTimer timer(ctx, stream);
+  if (p.kv_index)
+    hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kGeneric>), grid, dim3(256), 0, stream, p);
+  else if (p.softcap > 0.0f)
+    hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kSoftcap>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((decode_split_kernel<D, GT, KV_T, U, kPlain>), grid, dim3(256), 0, stream, p);
+  timer.mark();
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   if (!p.direct) {
     hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<KV_T>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
@@ -338,6 +336,12 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: batch / kv heads beyond grid limits");
 
   const int D = a->head_dim;
+  if (D != 64 && D != 128 && D != 256)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: head_dim %d not in {64,128,256}", D);
+  // An index list names slots of a HeadMajor cache of `capacity` rows (of the `capacity` first
+  // positions of a SeqMajor one); the kernels treat a slot outside [0, capacity) as a masked token.
+  if (a->kv_index && a->capacity <= 0)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: kv_index needs capacity > 0 (got %d)", a->capacity);
   DecodeParams p{};
   p.q = a->q;
   p.k = a->k_cache;
@@ -379,11 +383,8 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
 
   hipStream_t stream = (hipStream_t)a->stream;
   const bool want_scores = a->scores_out != nullptr;
-  // ARGUS_HIP_DECODE=valu keeps the vector-ALU kernel for A/B measurements.
-  static const bool force_valu = [] {
-    const char *e = getenv("ARGUS_HIP_DECODE");
-    return e && strcmp(e, "valu") == 0;
-  }();
+  // ARGUS_HIP_DECODE=valu (read when the context is created) keeps the vector-ALU kernel for A/B measurements.
+  const bool force_valu = ctx->env.decode_valu;
   if (blocks) return launch_decode_blocks(ctx, p, D, a->kv_dtype, a->batch, stream);
   if (!force_valu && decode_mfma_supported(p, D, a->kv_dtype)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
   switch (a->kv_dtype) {

@@ -337,7 +337,7 @@ struct BlockFallback {
     for (int c = threadIdx.x; c < D; c += blockDim.x) {
       float acc = 0.0f;
       for (int t = 0; t < p.len; ++t) {
-        const int64_t slot = idx ? idx[t] : (p.kv_start + t);
+        const int64_t slot = idx ? (int64_t)min((uint32_t)idx[t], (uint32_t)(p.slot_bound - 1)) : (p.kv_start + t);
         acc += u * block_elem<FMT>(vb + (slot * p.row_stride / 32 + c / 32) * F::BB, c % 32);
       }
       p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = acc;
@@ -423,6 +423,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   constexpr int NKR = (D == 64) ? 1 : TW;                               // K rows a lane addresses per iteration
   constexpr int NVR = kStageV ? ((D == 64) ? 1 : TW) : 4 * TW;          // V rows
   const int32_t *idx = INDEXED ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
+  // Rows are fetched with plain loads: a slot outside the cache (stale or negative entry of the
+  // list) is clamped to the last one, so the list can never steer a load out of the head's slab.
+  const uint32_t slot_max = (uint32_t)(p.slot_bound - 1);
   int k_row[INDEXED ? NKR : 1], v_row[INDEXED ? NVR : 1];
   auto k_tok = [&](int base, int i) { return min((D == 64) ? base + 16 * (j >> 1) + r : base + 16 * i + r, last); };
   auto v_tok = [&](int base, int i) {
@@ -432,13 +435,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   auto load_idx_k = [&](int base) {
     if constexpr (INDEXED) {
 #pragma unroll
-      for (int i = 0; i < NKR; ++i) k_row[i] = idx[k_tok(base, i)];
+      for (int i = 0; i < NKR; ++i) k_row[i] = (int)min((uint32_t)idx[k_tok(base, i)], slot_max);
     }
   };
   auto load_idx_v = [&](int base) {
     if constexpr (INDEXED) {
 #pragma unroll
-      for (int i = 0; i < NVR; ++i) v_row[i] = idx[v_tok(base, i)];
+      for (int i = 0; i < NVR; ++i) v_row[i] = (int)min((uint32_t)idx[v_tok(base, i)], slot_max);
     }
   };
   auto k_rowof = [&](int base, int i) -> uint32_t {
@@ -835,45 +838,27 @@ template <int FMT, int D>
 int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
   constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
   constexpr int tile_rows = kWaves * 16 * TW;
-  static int wgs_per_cu = 0;  // per instantiation; single inference thread
-  if (wgs_per_cu == 0) {
-    int n = 0;
-    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_blocks_kernel<FMT, D, TW, false, false>, 64 * kWaves, 0));
-    wgs_per_cu = std::max(1, n);
-  }
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
   // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips).
   constexpr int kStageBytes = 48 * 1024;
-  const int max_chunk = staged_chunk_limit(p, kStageBytes, tile_rows);
+  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * BlockShape<D>::MAXH * (D + 4)) * sizeof(float);
+  const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
+  const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_blocks_kernel<FMT, D, TW, false, false>, 64 * kWaves,
+                                          max_chunk > 0 ? (size_t)kStageBytes : merge_bytes);
   choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   p.direct = 0;
   p.stage_scores = p.scores && p.chunk <= max_chunk;
-  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * BlockShape<D>::MAXH * (D + 4)) * sizeof(float);
   const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
-  static bool lds_limit_raised = false;
-  if (!lds_limit_raised) {
-    constexpr int kLimit = kStageBytes + 1024;
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_blocks_kernel<FMT, D, TW, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    lds_limit_raised = true;
-  }
-  const size_t n_part = (size_t)batch * p.n_heads_q * p.nsplit;
-  const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
-  int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+  const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
+  auto kern = cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true> : decode_blocks_kernel<FMT, D, TW, true, false>)
+                  : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true> : decode_blocks_kernel<FMT, D, TW, false, false>);
+  ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + 1024));
+  const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
-  p.ws_ml = ctx->ws;
-  p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
-  {
-    KernelTimer timer(ctx, stream);
-    const dim3 grid(p.nsplit, p.n_heads_kv, batch), block(64 * kWaves);
-    const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-    if (cap && indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, true>), grid, block, lds_bytes, stream, p);
-    else if (cap) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, true, false>), grid, block, lds_bytes, stream, p);
-    else if (indexed) hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, true>), grid, block, lds_bytes, stream, p);
-    else hipLaunchKernelGGL((decode_blocks_kernel<FMT, D, TW, false, false>), grid, block, lds_bytes, stream, p);
-  }
+  ctx->plan = argus_hip_decode_plan{p.nsplit, p.chunk, wgs_per_cu, (int32_t)lds_bytes, 2, 2, p.stage_scores};
+  KernelTimer timer(ctx, stream);
+  hipLaunchKernelGGL(kern, dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), lds_bytes, stream, p);
+  timer.mark();
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<BlockFallback<FMT>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
@@ -885,13 +870,18 @@ int launch_blocks_dim(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hip
   switch (D) {
     case 64: return launch_blocks<FMT, 64>(ctx, p, batch, stream);
     case 128: return launch_blocks<FMT, 128>(ctx, p, batch, stream);
-    default: return launch_blocks<FMT, 256>(ctx, p, batch, stream);
+    case 256: return launch_blocks<FMT, 256>(ctx, p, batch, stream);
+    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: head_dim %d not in {64,128,256}", D);
   }
 }
 
 }  // namespace
 
 int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtype, int batch, hipStream_t stream) {
+  // The kernels lay rows, partials and LDS out for these three widths; any other would run the
+  // wrong instantiation over the caller's buffers.
+  if (D != 64 && D != 128 && D != 256)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: head_dim %d not in {64,128,256}", D);
   if (p.group > ((D == 256) ? 8 : 16))
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: %d query heads per KV head on a block-quantised cache", p.group);
   if ((p.row_stride % 32) || (p.head_stride % 32) || (p.kv_bs % 32))
@@ -906,7 +896,8 @@ int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtyp
     case ARGUS_HIP_Q4_0: return launch_blocks_dim<kFmtQ4_0>(ctx, p, D, batch, stream);
     case ARGUS_HIP_Q4_1: return launch_blocks_dim<kFmtQ4_1>(ctx, p, D, batch, stream);
     case ARGUS_HIP_Q2_0: return launch_blocks_dim<kFmtQ2_0>(ctx, p, D, batch, stream);
-    default: return launch_blocks_dim<kFmtQ8_0>(ctx, p, D, batch, stream);
+    case ARGUS_HIP_Q8_0: return launch_blocks_dim<kFmtQ8_0>(ctx, p, D, batch, stream);
+    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: kv dtype %d is not a block format", kv_dtype);
   }
 }
 

@@ -53,7 +53,7 @@ __device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
   for (int c = threadIdx.x; c < D; c += blockDim.x) {
     float acc = 0.0f;
     for (int t = 0; t < p.len; ++t) {
-      const int64_t slot = idx ? idx[t] : (p.kv_start + t);
+      const int64_t slot = idx ? (int64_t)min((uint32_t)idx[t], (uint32_t)(p.slot_bound - 1)) : (p.kv_start + t);
       acc += u * (float)vb[slot * p.row_stride + c];
     }
     p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = acc;
@@ -315,13 +315,21 @@ __device__ __forceinline__ void flush_staged_logits(const DecodeParams &p, const
   __syncthreads();  // the caller reuses the area
 }
 // Longest chunk whose logits fit `stage_bytes` of LDS (0 without scores), for choose_splits().
-// ARGUS_HIP_SCORES=direct (read at every call with scores) keeps the stores in the token loop, the
+// ARGUS_HIP_SCORES=direct (read when the context is created) keeps the stores in the token loop, the
 // path of chunks too long to stage: for A/B measurements and for tests of that path at small sizes.
-inline int staged_chunk_limit(const DecodeParams &p, int stage_bytes, int tile_rows) {
-  if (!p.scores) return 0;
-  const char *e = getenv("ARGUS_HIP_SCORES");
-  if (e && strcmp(e, "direct") == 0) return 0;
+inline int staged_chunk_limit(const argus_hip_ctx *ctx, const DecodeParams &p, int stage_bytes, int tile_rows) {
+  if (!p.scores || ctx->env.scores_direct) return 0;
   return (stage_bytes / 4 / p.group - 4) / tile_rows * tile_rows;
+}
+// Places the split partials of a launch (p.nsplit set) in the context workspace.
+inline int reserve_partials(argus_hip_ctx *ctx, DecodeParams &p, int batch, int D) {
+  const size_t n_part = (size_t)batch * p.n_heads_q * p.nsplit;
+  const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
+  const int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+  if (rc != ARGUS_HIP_OK) return rc;
+  p.ws_ml = argus_ws(ctx);
+  p.ws_o = (float *)((char *)argus_ws(ctx) + ml_bytes);
+  return ARGUS_HIP_OK;
 }
 inline bool score_rows_addressable(const DecodeParams &p) {
   return !p.scores || (p.score_stride >= p.len && ((int64_t)p.group * p.score_stride + 1024) * 4 <= 0x7fffffffll);

@@ -331,46 +331,28 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   constexpr int TW = (D <= 128) ? 2 : 1;
   constexpr int tile_rows = kWaves * 16 * TW;  // one tile per wave
   const int pairs = batch * p.n_heads_kv;
-  static int wgs_per_cu = 0;  // per head_dim instantiation; single inference thread
-  if (wgs_per_cu == 0) {
-    int n = 0;
-    ARGUS_HIP_CHECK(ctx, hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves, 0));
-    wgs_per_cu = std::max(1, n);
-  }
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
-  // token loop is over (kStageBytes; two workgroups per CU still fit).
+  // token loop is over (kStageBytes; two workgroups per CU still fit).  The resident round is counted
+  // at the LDS size the launch may reach.
   constexpr int kStageBytes = 64 * 1024;
-  const int max_chunk = staged_chunk_limit(p, kStageBytes, tile_rows);
+  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * MfmaShape<D>::MAXH * (D + 4)) * sizeof(float);
+  const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
+  const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves,
+                                          max_chunk > 0 ? (size_t)kStageBytes : merge_bytes);
   choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
-  const int nsplit = p.nsplit;
   p.direct = 0;
   p.stage_scores = p.scores && p.chunk <= max_chunk;
-  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * MfmaShape<D>::MAXH * (D + 4)) * sizeof(float);
   const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
-  static bool lds_limit_raised = false;
-  if (!lds_limit_raised) {
-    constexpr int kLimit = kStageBytes + 1024;
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)decode_mfma_kernel<D, TW, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLimit));
-    lds_limit_raised = true;
-  }
-  const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
-  const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
-  int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+  const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
+  auto kern = cap ? (indexed ? decode_mfma_kernel<D, TW, true, true> : decode_mfma_kernel<D, TW, true, false>)
+                  : (indexed ? decode_mfma_kernel<D, TW, false, true> : decode_mfma_kernel<D, TW, false, false>);
+  ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + 1024));
+  const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
-  p.ws_ml = ctx->ws;
-  p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
-  {
-    KernelTimer timer(ctx, stream);
-    const dim3 grid(nsplit, p.n_heads_kv, batch), block(64 * kWaves);
-    const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-    if (cap && indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, true>), grid, block, lds_bytes, stream, p);
-    else if (cap) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, true, false>), grid, block, lds_bytes, stream, p);
-    else if (indexed) hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, true>), grid, block, lds_bytes, stream, p);
-    else hipLaunchKernelGGL((decode_mfma_kernel<D, TW, false, false>), grid, block, lds_bytes, stream, p);
-  }
+  ctx->plan = argus_hip_decode_plan{p.nsplit, p.chunk, wgs_per_cu, (int32_t)lds_bytes, 2, 1, p.stage_scores};
+  KernelTimer timer(ctx, stream);
+  hipLaunchKernelGGL(kern, dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), lds_bytes, stream, p);
+  timer.mark();
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());

@@ -311,11 +311,8 @@ __global__ __launch_bounds__(128) void kivi_flush_v_kernel(const float *__restri
 
 template <int BITS>
 int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
-  // ARGUS_HIP_KIVI=valu keeps the vector-ALU kernel for A/B measurements.
-  static const bool force_valu = [] {
-    const char *e = getenv("ARGUS_HIP_KIVI");
-    return e && strcmp(e, "valu") == 0;
-  }();
+  // ARGUS_HIP_KIVI=valu (read when the context is created) keeps the vector-ALU kernel for A/B measurements.
+  const bool force_valu = ctx->env.kivi_valu;
   if (!force_valu && kivi_mfma_supported(kp)) return launch_kivi_mfma(ctx, kp, BITS, batch, stream);
   DecodeParams &p = kp.d;
   const int D = kp.head_dim;
@@ -327,21 +324,17 @@ int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t strea
   nsplit = (kp.units_total + kp.units_per_split - 1) / kp.units_per_split;
   p.nsplit = nsplit;
   p.direct = 0;
-  const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
-  const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
-  int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+  const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
-  p.ws_ml = ctx->ws;
-  p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
+  ctx->plan = argus_hip_decode_plan{nsplit, kp.units_per_split * kUnit, 0, 0, 2, 4, 0};
 
   dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
-  {
-    KernelTimer timer(ctx, stream);
-    if (p.group <= 1) hipLaunchKernelGGL((kivi_split_kernel<BITS, 1>), grid, dim3(256), 0, stream, kp);
-    else if (p.group <= 2) hipLaunchKernelGGL((kivi_split_kernel<BITS, 2>), grid, dim3(256), 0, stream, kp);
-    else if (p.group <= 4) hipLaunchKernelGGL((kivi_split_kernel<BITS, 4>), grid, dim3(256), 0, stream, kp);
-    else hipLaunchKernelGGL((kivi_split_kernel<BITS, 8>), grid, dim3(256), 0, stream, kp);
-  }
+  KernelTimer timer(ctx, stream);
+  if (p.group <= 1) hipLaunchKernelGGL((kivi_split_kernel<BITS, 1>), grid, dim3(256), 0, stream, kp);
+  else if (p.group <= 2) hipLaunchKernelGGL((kivi_split_kernel<BITS, 2>), grid, dim3(256), 0, stream, kp);
+  else if (p.group <= 4) hipLaunchKernelGGL((kivi_split_kernel<BITS, 4>), grid, dim3(256), 0, stream, kp);
+  else hipLaunchKernelGGL((kivi_split_kernel<BITS, 8>), grid, dim3(256), 0, stream, kp);
+  timer.mark();
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   switch (D) {
     case 64: hipLaunchKernelGGL((decode_combine_kernel<NoFallback, 64>), combine_grid(p, batch), dim3(256), 0, stream, p); break;

@@ -564,12 +564,8 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   const int pairs = p.n_heads_kv * p.head_chunks * batch;
   // One round of co-resident workgroups: a second, partly filled round would run at a fraction of
   // the occupancy the unit loop needs to hide its LDS and HBM latency.
-  static const int wgs_per_cu = [] {
-    int n4 = 0, n8 = 0;
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n4, kivi_mfma_kernel<BITS, D, 4, false>, 256, 0);
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&n8, kivi_mfma_kernel<BITS, D, 8, false>, 256, 0);
-    return std::max(1, std::min(n4, n8));
-  }();
+  const int wgs_per_cu = std::min(argus_wgs_per_cu(ctx, kivi_mfma_kernel<BITS, D, 4, false>, 256, 0),
+                                  argus_wgs_per_cu(ctx, kivi_mfma_kernel<BITS, D, 8, false>, 256, 0));
   const int slots = ctx->compute_units * wgs_per_cu;
   const int max_splits = (kp.units_total + 3) / 4;  // at least one unit per wave
   int nsplit = std::max(1, std::min({slots / pairs, max_splits, kMaxSplits}));
@@ -577,21 +573,17 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   nsplit = (kp.units_total + kp.units_per_split - 1) / kp.units_per_split;
   p.nsplit = nsplit;
   p.direct = 0;
-  const size_t n_part = (size_t)batch * p.n_heads_q * nsplit;
-  const size_t ml_bytes = (n_part * 2 * sizeof(float) + 255) / 256 * 256;
-  int rc = argus_ws_reserve(ctx, ml_bytes + n_part * D * sizeof(float));
+  const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
-  p.ws_ml = ctx->ws;
-  p.ws_o = (float *)((char *)ctx->ws + ml_bytes);
+  ctx->plan = argus_hip_decode_plan{nsplit, kp.units_per_split * kUnit, wgs_per_cu, 0, 2, 3, 0};
   const dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
-  {
-    KernelTimer timer(ctx, stream);
-    const bool cap = p.softcap > 0.0f;
-    if (p.group <= 4 && cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, true>), grid, dim3(256), 0, stream, kp);
-    else if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, false>), grid, dim3(256), 0, stream, kp);
-    else if (cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, true>), grid, dim3(256), 0, stream, kp);
-    else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false>), grid, dim3(256), 0, stream, kp);
-  }
+  KernelTimer timer(ctx, stream);
+  const bool cap = p.softcap > 0.0f;
+  if (p.group <= 4 && cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, true>), grid, dim3(256), 0, stream, kp);
+  else if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, false>), grid, dim3(256), 0, stream, kp);
+  else if (cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, true>), grid, dim3(256), 0, stream, kp);
+  else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false>), grid, dim3(256), 0, stream, kp);
+  timer.mark();
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<NoFallback, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
@@ -610,7 +602,6 @@ int launch_dim(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream
 }  // namespace
 
 bool kivi_mfma_supported(const KiviParams &kp) {
-  const DecodeParams &p = kp.d;
   if (kp.head_dim != 64 && kp.head_dim != 128 && kp.head_dim != 256) return false;
   // tiles are copied as 16-byte vectors
   if ((((uintptr_t)kp.qk | (uintptr_t)kp.qv) & 15) || (kp.qk_bs & 15) || (kp.qv_bs & 15)) return false;

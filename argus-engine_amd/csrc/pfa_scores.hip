@@ -223,10 +223,34 @@ ARGUS_API int argus_hip_prefill_attention_scores(argus_hip_ctx *ctx, const argus
   const size_t stat_bytes = ((size_t)p.n_heads_q * p.qwin * 2 * sizeof(float) + 255) / 256 * 256;
   const size_t logit_bytes = (size_t)p.n_heads_q * p.qwin * p.prefix_len * sizeof(float);
   const bool keep_logits = p.head_dim % 64 == 0 && logit_bytes <= ((size_t)1 << 30) && ((uintptr_t)a->q & 15) == 0;
-  int rc = argus_ws_reserve(ctx, stat_bytes + (keep_logits ? logit_bytes : 0));
-  if (rc != ARGUS_HIP_OK) return rc;
-  p.stats = ctx->ws;
-  p.logits = keep_logits ? (float *)((char *)ctx->ws + stat_bytes) : nullptr;
+  // The logits live in a scratch buffer of their own (not the split-KV workspace, which stays at the
+  // size the decode calls need).  It is kept between calls while small; a call that made it larger
+  // than kKeepBytes gives it back before returning, which costs one stream synchronisation per
+  // prefill chunk and layer.
+  constexpr size_t kKeepBytes = (size_t)64 << 20;
+  const size_t need = stat_bytes + (keep_logits ? logit_bytes : 0);
+  if (need > ctx->pfa_ws_bytes) {
+    if (ctx->pfa_ws) {
+      ARGUS_HIP_CHECK(ctx, hipFree(ctx->pfa_ws));  // synchronises: no earlier call still reads it
+      ctx->pfa_ws = nullptr;
+      ctx->pfa_ws_bytes = 0;
+    }
+    if (hipMalloc((void **)&ctx->pfa_ws, need) != hipSuccess) {
+      (void)hipGetLastError();
+      ctx->pfa_ws = nullptr;
+      return argus_fail(ctx, ARGUS_HIP_ERR_NOMEM, "prefill_attention_scores: scratch of %zu bytes", need);
+    }
+    ctx->pfa_ws_bytes = need;
+  }
+  p.stats = ctx->pfa_ws;
+  p.logits = keep_logits ? (float *)((char *)ctx->pfa_ws + stat_bytes) : nullptr;
   hipStream_t stream = (hipStream_t)a->stream;
-  return a->k_dtype == ARGUS_HIP_F16 ? launch<_Float16>(ctx, p, stream) : launch<float>(ctx, p, stream);
+  const int rc = a->k_dtype == ARGUS_HIP_F16 ? launch<_Float16>(ctx, p, stream) : launch<float>(ctx, p, stream);
+  if (ctx->pfa_ws_bytes > kKeepBytes) {
+    (void)hipStreamSynchronize(stream);
+    (void)hipFree(ctx->pfa_ws);
+    ctx->pfa_ws = nullptr;
+    ctx->pfa_ws_bytes = 0;
+  }
+  return rc;
 }

@@ -488,11 +488,7 @@ int launch_ng(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream, size_t l
   const int64_t wgs = (int64_t)p.batch * p.n_heads_kv * p.group_chunks * ((p.n_qtiles + 1) / 2);
   if (wgs > 0x7fffffff) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: grid too large");
   auto kern = prefill_kernel<D, HPW, NG, KV_T>;
-  static bool attr_set = false;  // per instantiation; single inference thread
-  if (!attr_set && lds_bytes > 48 * 1024) {
-    ARGUS_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    attr_set = true;
-  }
+  if (lds_bytes > 48 * 1024) ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, (int)lds_bytes));
   {
     KernelTimer timer(ctx, stream);
     hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(256 * NG), lds_bytes, stream, p);

@@ -58,9 +58,15 @@ class HipGpuScoreAccumulator;
 class HipBackend {
  public:
   // Counterpart of the "hip" arm of engine/src/session/init.rs:203-468.
-  static Result<std::shared_ptr<HipBackend>> create(int device = 0) {
+  // `max_*`: the largest attention call the session will issue (the engine knows them from the model
+  // config and --max-seq-len, and pre-allocates its own buffers from the same numbers,
+  // crates/argus-extension-api/src/lib.rs:1903-1907); the split-KV workspace is sized once from
+  // them so that no call allocates.
+  static Result<std::shared_ptr<HipBackend>> create(int device = 0, int max_batch = 0, int max_heads_q = 0, int max_head_dim = 0,
+                                                    int max_seq_len = 0) {
     argus_hip_ctx *ctx = nullptr;
-    const int rc = argus_hip_create(device, &ctx);
+    const argus_hip_create_opts opts = {max_batch, max_heads_q, max_head_dim, max_seq_len};
+    const int rc = argus_hip_create_ex(device, &opts, &ctx);
     if (rc != ARGUS_HIP_OK) return Result<std::shared_ptr<HipBackend>>::Err("argus_hip_create failed: code " + std::to_string(rc));
     return Result<std::shared_ptr<HipBackend>>::Ok(std::shared_ptr<HipBackend>(new HipBackend(ctx)));
   }
@@ -75,7 +81,8 @@ class HipBackend {
   bool supports_kv_scatter_batch() const { return true; }
   argus_hip_ctx *ctx() const { return ctx_; }
 
-  // ---- memory (Backend::{read_buffer, write_buffer, copy_slice, synchronize}) ---------------
+  // ---- memory (Backend::{read_buffer, write_buffer, write_buffer_range, copy_slice, buffer_shift,
+  //      synchronize}, engine/src/backend.rs:610, 710, 736, 1085, 1119, 762) ---------------------
   Result<void *> alloc(size_t bytes) {
     void *p = nullptr;
     if (argus_hip_malloc(ctx_, bytes, &p) != ARGUS_HIP_OK) return Result<void *>::Err(last_error());
@@ -85,6 +92,22 @@ class HipBackend {
   Status write_buffer(void *dst_dev, const void *src_host, size_t bytes) { return wrap(argus_hip_write_buffer(ctx_, nullptr, dst_dev, src_host, bytes)); }
   Status read_buffer(void *dst_host, const void *src_dev, size_t bytes) { return wrap(argus_hip_read_buffer(ctx_, nullptr, dst_host, src_dev, bytes)); }
   Status copy_slice(void *dst_dev, const void *src_dev, size_t bytes) { return wrap(argus_hip_copy_slice(ctx_, nullptr, dst_dev, src_dev, bytes)); }
+  // Backend::write_buffer_range(t, src, dst_offset): bounds-checked like the trait default
+  // (engine/src/backend.rs:736-757).
+  Status write_buffer_range(void *dst_dev, size_t dst_size, const void *src_host, size_t bytes, size_t dst_offset) {
+    if (dst_offset + bytes < dst_offset) return Status::Err("write_buffer_range: offset+len overflow");
+    if (dst_offset + bytes > dst_size)
+      return Status::Err("write_buffer_range: out of bounds (" + std::to_string(dst_offset) + " + " + std::to_string(bytes) + " > " +
+                         std::to_string(dst_size) + ")");
+    return wrap(argus_hip_write_buffer_range(ctx_, nullptr, dst_dev, dst_offset, src_host, bytes));
+  }
+  // Backend::buffer_shift(tensor, src_offset, dst_offset, count): offsets and count in elements of
+  // the tensor's dtype, overlap-safe like memmove (engine/src/backend.rs:1082-1112).
+  Status buffer_shift(Tensor &t, size_t src_offset, size_t dst_offset, size_t count) {
+    if (!t.ptr) return Status::Err("Null pointer in buffer_shift");
+    const size_t ts = t.dtype == DType::F32 ? 4 : t.dtype == DType::F16 ? 2 : t.dtype == DType::Q4_0 ? 18 : 1;
+    return wrap(argus_hip_buffer_shift(ctx_, nullptr, (char *)t.ptr + dst_offset * ts, (const char *)t.ptr + src_offset * ts, count * ts));
+  }
   Status synchronize() { return wrap(argus_hip_synchronize(ctx_, nullptr)); }
 
   // ---- Backend::attention_gen (engine/src/backend.rs:284-295) ---------------------------------

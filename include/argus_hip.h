@@ -5,7 +5,10 @@
  * `int` (0 = ok, negative = error, never throws or aborts: the engine's release
  * profile is panic=abort, crates/argus-extension-api/src/lib.rs:1680) and runs on
  * the single in-order stream the engine lends (NULL = the default stream,
- * engine/src/kv/quant_window_cuda.rs:38-46).  The engine owns every Q / KV / out /
+ * engine/src/kv/quant_window_cuda.rs:38-46).  A context serves ONE stream at a time: its split-KV
+ * workspace is handed to every attention call, so calls issued on different streams without
+ * ordering between them race on the partial results (the reference backends are single-stream too,
+ * engine/src/backend/cuda_pc/gpu_score.rs:40-50).  The engine owns every Q / KV / out /
  * score buffer and lends raw device pointers for the duration of one call; the
  * library never frees or retains them (crates/argus-extension-api/src/lib.rs:1593).
  *
@@ -55,6 +58,20 @@ typedef struct argus_hip_ctx argus_hip_ctx;
  * device, reads its CU count and allocates the split-KV partial workspace.  Fails with
  * ARGUS_HIP_ERR_RUNTIME (and *out = NULL) when no HIP device is present. */
 int argus_hip_create(int device, argus_hip_ctx **out);
+/* The reference pre-allocates every buffer at max_seq_len and lends it for the session, with no
+ * allocator callback into the engine (crates/argus-extension-api/src/lib.rs:1903-1907).  The one
+ * buffer this library owns is the split-KV workspace; create_ex sizes it once for the largest call
+ * the caller will issue (zero fields / NULL opts: 8 MiB), so that no attention call allocates.  A
+ * call beyond the hint still works: it grows the workspace, which synchronises the device.
+ * The environment switches ARGUS_HIP_DECODE / ARGUS_HIP_SCORES / ARGUS_HIP_KIVI are read here. */
+typedef struct argus_hip_create_opts {
+  int32_t max_batch;    /* sequences (or KIVI caches) per attention call */
+  int32_t max_heads_q;  /* query heads */
+  int32_t max_head_dim; /* 64, 128 or 256 */
+  int32_t max_seq_len;  /* informational: the split count is bounded whatever the length */
+} argus_hip_create_opts;
+int argus_hip_create_ex(int device, const argus_hip_create_opts *opts, argus_hip_ctx **out);
+int argus_hip_reserve_workspace(argus_hip_ctx *ctx, size_t bytes);
 int argus_hip_destroy(argus_hip_ctx *ctx);
 int argus_hip_abi_version(void);
 /* Last error text of this context (single inference thread, like the reference backends). */
@@ -79,6 +96,10 @@ int argus_hip_get_device_info(const argus_hip_ctx *ctx, argus_hip_device_info *i
  * per-launch durations in milliseconds (at most `capacity`; *n_out = launches recorded). */
 int argus_hip_kernel_timing_begin(argus_hip_ctx *ctx, int32_t max_launches);
 int argus_hip_kernel_timing_end(argus_hip_ctx *ctx, float *ms_out, int32_t capacity, int32_t *n_out);
+/* Same, and in tail_ms_out (may be NULL) the time from the end of the dominant kernel to the end of
+ * the call's last launch: the combine pass of a split-KV decode, zero for single-kernel calls. */
+int argus_hip_kernel_timing_end2(argus_hip_ctx *ctx, float *ms_out, float *tail_ms_out, int32_t capacity,
+                                 int32_t *n_out);
 
 /* ---- memory helpers for the Rust `Memory` / `Buffer` impls ------------------------------- */
 /* Backend::{read_buffer, write_buffer, write_buffer_range, copy_slice, buffer_shift,
@@ -88,6 +109,14 @@ int argus_hip_free(argus_hip_ctx *ctx, void *dev_ptr);
 int argus_hip_write_buffer(argus_hip_ctx *ctx, void *stream, void *dst_dev, const void *src_host, size_t bytes);
 int argus_hip_read_buffer(argus_hip_ctx *ctx, void *stream, void *dst_host, const void *src_dev, size_t bytes);
 int argus_hip_copy_slice(argus_hip_ctx *ctx, void *stream, void *dst_dev, const void *src_dev, size_t bytes);
+/* Backend::write_buffer_range (engine/src/backend.rs:736): host bytes into dst_dev + dst_offset. */
+int argus_hip_write_buffer_range(argus_hip_ctx *ctx, void *stream, void *dst_dev, size_t dst_offset,
+                                 const void *src_host, size_t bytes);
+/* Backend::buffer_shift (engine/src/backend.rs:1085-1112): std::ptr::copy inside one buffer, i.e.
+ * memmove -- the ranges may overlap in either direction (prefix prune; the KIVI residual ring moving
+ * its remaining rows to the front, engine/src/kv/quant_window_cache.rs:1820-1841).  Uses the
+ * context workspace as staging when the ranges lie less than 1 MiB apart. */
+int argus_hip_buffer_shift(argus_hip_ctx *ctx, void *stream, void *dst_dev, const void *src_dev, size_t bytes);
 int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream);
 
 /* ---- (a-1) single-query GQA decode attention ---------------------------------------------- */
@@ -106,6 +135,9 @@ int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream);
  *   kv_start               : first attended slot (windowed layers pass cache_len - window);
  *   kv_index               : logical token t lives in slot kv_index[t]
  *                            (SelectiveRead gather, engine/src/kv/standard_format.rs:2052-2184);
+ *                            `capacity` (> 0, both layouts) bounds the slots: an entry outside
+ *                            [0, capacity) never reaches memory outside the head's rows (it reads
+ *                            zeros or the last slot; the result for such a list is unspecified);
  *   softcap                : cap*tanh(s/cap) after scaling
  *                            (engine/kernels/flash_attn_f32_f16.cl:563-565; host passes 0);
  *   scale                  : 0 selects 1/sqrt(head_dim) (x86.rs:192).
@@ -143,6 +175,20 @@ typedef struct argus_hip_attention_gen_args {
   float scale;
 } argus_hip_attention_gen_args;
 int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args);
+
+/* How the last attention_gen / attention_gen_quant call on this context was cut along the KV length
+ * (diagnostics for benchmarks and tests; the reference has no split-KV on this path outside
+ * engine/src/backend/cpu/neon.rs:261-300). */
+typedef struct argus_hip_decode_plan {
+  int32_t nsplit;        /* workgroups per (sequence, KV head) */
+  int32_t chunk;         /* tokens per split */
+  int32_t wgs_per_cu;    /* resident workgroups per compute unit the plan assumed */
+  int32_t lds_bytes;     /* dynamic LDS of the launch */
+  int32_t launches;      /* kernels launched by the call (1 = no combine pass) */
+  int32_t kernel;        /* 0 vector-ALU, 1 matrix-core F16, 2 block formats, 3 KIVI matrix-core, 4 KIVI vector-ALU */
+  int32_t staged_scores; /* 1: the logits of a chunk waited in LDS; 0: stored from inside the token loop (or no scores) */
+} argus_hip_decode_plan;
+int argus_hip_last_decode_plan(const argus_hip_ctx *ctx, argus_hip_decode_plan *plan);
 
 /* ---- (a-2) causal GQA flash-attention prefill ---------------------------------------------- */
 /* Backend::flash_attention_prefill, engine/src/backend.rs:1011-1027 (CUDA host

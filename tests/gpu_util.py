@@ -14,6 +14,28 @@ def ctx():
     return _ctx
 
 
+_direct_ctx = None
+
+
+def direct_ctx():
+    """A second context created under ARGUS_HIP_SCORES=direct (the switches are read when a context
+    is created): its score-emitting decode calls store their logits from inside the token loop."""
+    global _direct_ctx
+    if _direct_ctx is None:
+        import os
+        import argus_hip
+        old = os.environ.get("ARGUS_HIP_SCORES")
+        os.environ["ARGUS_HIP_SCORES"] = "direct"
+        try:
+            _direct_ctx = argus_hip.Context(0)
+        finally:
+            if old is None:
+                del os.environ["ARGUS_HIP_SCORES"]
+            else:
+                os.environ["ARGUS_HIP_SCORES"] = old
+    return _direct_ctx
+
+
 def dev(a):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()

@@ -36,7 +36,8 @@ def test_struct_layouts_match_header_field_order():
              "argus_hip_quant_gather_args": A.QuantGatherArgs, "argus_hip_quant_flush_args": A.QuantFlushArgs,
              "argus_hip_quant_dequant_flush_args": A.QuantDequantFlushArgs,
              "argus_hip_quant_scatter_residual_args": A.QuantScatterResidualArgs,
-             "argus_hip_score_reduce_args": A.ScoreReduceArgs, "argus_hip_device_info": A.DeviceInfo}
+             "argus_hip_score_reduce_args": A.ScoreReduceArgs, "argus_hip_device_info": A.DeviceInfo,
+             "argus_hip_create_opts": A.CreateOpts, "argus_hip_decode_plan": A.DecodePlan}
     for cname, cls in pairs.items():
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), text, re.S).group(1)
         fields = []
@@ -64,5 +65,11 @@ def test_degraded_without_device_or_context():
     assert A.lib.argus_hip_flash_attention_prefill(None, None) < 0
     assert A.lib.argus_hip_kv_scatter_f32_to_f16(None, None, None, None, None, None, 1, 64, 8, 0) == A.ERR_INVALID
     assert A.lib.argus_hip_destroy(None) == A.ERR_INVALID
+    opts = A.CreateOpts(16, 32, 128, 32768)
+    assert A.lib.argus_hip_create_ex(0, C.byref(opts), C.byref(h)) == A.ERR_RUNTIME and not h.value
+    assert A.lib.argus_hip_buffer_shift(None, None, None, None, 16) == A.ERR_INVALID
+    assert A.lib.argus_hip_write_buffer_range(None, None, None, 0, None, 16) == A.ERR_INVALID
+    assert A.lib.argus_hip_reserve_workspace(None, 1 << 20) == A.ERR_INVALID
+    assert A.lib.argus_hip_last_decode_plan(None, None) == A.ERR_INVALID
     with pytest.raises(A.ArgusHipError):
         A.Context(0)

@@ -7,7 +7,7 @@ import pytest
 
 import oracle as O
 from blocks_util import random_blocks
-from gpu_util import ctx, dev, host, normal, check_attention_out, check_scores
+from gpu_util import ctx, dev, direct_ctx, host, normal, check_attention_out, check_scores
 
 pytestmark = pytest.mark.gpu
 
@@ -20,7 +20,7 @@ FORMATS = {
 
 
 def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True, kv_start=0, encode=False, softcap=0.0, q_gain=1.0,
-             score_pad=0):
+             score_pad=0, context=None):
     import argus_hip as A
     desc, name = FORMATS[fmt]
     cap = cap or L
@@ -34,7 +34,7 @@ def run_case(fmt, hq, hkv, d, L, cap=None, head_major=True, seed=7, scores=True,
     q = normal((hq, d), seed) * np.float32(q_gain)
     out = dev(np.zeros((hq, d), np.float32))
     sc = dev(np.full((hq, L + score_pad), -7.0, np.float32)) if scores else None
-    ctx().attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, cap,
+    (context or ctx()).attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, cap,
                         layout=A.HEAD_MAJOR if head_major else A.SEQ_MAJOR, scores=sc,
                         score_stride=L + score_pad if scores else 0, kv_start=kv_start, kv_dtype=getattr(A, name), softcap=softcap)
     # oracle: a window that starts at kv_start is the same cache with its first rows cut off
@@ -67,14 +67,16 @@ def test_score_rows_with_padding_stay_untouched_past_the_length(L):
 
 
 @pytest.mark.parametrize("L", [509, 511, 1021, 2051])
-def test_scores_stored_inside_the_token_loop(L, monkeypatch):
-    # the path of chunks too long for the LDS stage, taken at test sizes through ARGUS_HIP_SCORES=direct
-    monkeypatch.setenv("ARGUS_HIP_SCORES", "direct")
-    run_case("q4_0", 8, 2, 128, L, score_pad=5, seed=L)
-    run_case("q8_0", 14, 2, 64, L, score_pad=3, seed=L + 1)
-    run_case("q4_1", 8, 4, 256, L, score_pad=7, seed=L + 2)
-    run_case("q2_0", 12, 1, 128, L, score_pad=1, seed=L + 3)
-    run_case("q4_0", 32, 2, 64, L, score_pad=2, seed=L + 4)
+def test_scores_stored_inside_the_token_loop(L):
+    # the path of chunks too long for the LDS stage, taken at test sizes by a context created under
+    # ARGUS_HIP_SCORES=direct
+    c = direct_ctx()
+    run_case("q4_0", 8, 2, 128, L, score_pad=5, seed=L, context=c)
+    assert c.last_decode_plan()["staged_scores"] == 0 and c.last_decode_plan()["kernel"] == 2
+    run_case("q8_0", 14, 2, 64, L, score_pad=3, seed=L + 1, context=c)
+    run_case("q4_1", 8, 4, 256, L, score_pad=7, seed=L + 2, context=c)
+    run_case("q2_0", 12, 1, 128, L, score_pad=1, seed=L + 3, context=c)
+    run_case("q4_0", 32, 2, 64, L, score_pad=2, seed=L + 4, context=c)
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "q2_0"])

@@ -4,12 +4,12 @@ import pytest
 
 import oracle as O
 import textbook as T
-from gpu_util import check_attention_out, check_scores, ctx, dev, host, normal
+from gpu_util import check_attention_out, check_scores, ctx, dev, direct_ctx, host, normal
 
 pytestmark = pytest.mark.gpu
 
 
-def run_decode(q, k, v, hkv, L, capacity, layout=0, scores=False, score_stride=None, **kw):
+def run_decode(q, k, v, hkv, L, capacity, layout=0, scores=False, score_stride=None, context=None, **kw):
     import torch
     import argus_hip as A
     qd, kd, vd = dev(q), dev(k), dev(v)
@@ -19,8 +19,8 @@ def run_decode(q, k, v, hkv, L, capacity, layout=0, scores=False, score_stride=N
     if scores:
         stride = score_stride or L
         sc = torch.full(q.shape[:-1] + (stride,), -7.0, dtype=torch.float32, device="cuda")
-    ctx().attention_gen(qd, kd, vd, out, hkv, L, capacity, layout=layout, scores=sc,
-                        score_stride=stride, **kw)
+    (context or ctx()).attention_gen(qd, kd, vd, out, hkv, L, capacity, layout=layout, scores=sc,
+                                     score_stride=stride, **kw)
     return (host(out), host(sc)) if scores else host(out)
 
 
@@ -63,7 +63,8 @@ def test_decode_matrix(hq, hkv, d, L, kv):
     v = normal((hkv, cap, d), 53 + L)
     if kv == "f16":
         k, v = f16(k), f16(v)
-    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, score_stride=cap)
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, score_stride=cap, context=direct_ctx())
+    assert direct_ctx().last_decode_plan()["staged_scores"] == 0, "logits were staged in LDS after all"
     ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, scores_stride=cap)
     check_attention_out(got, ref, "out")
     check_scores(sc[:, :L], p[:, :L], "scores")
@@ -320,6 +321,70 @@ def test_config3_batch16_at_32k_properties_and_sampled_parity():
     assert (out2[0] - out[0]).abs().max().item() < 3e-5
 
 
+def test_config3_batch16_at_4k():
+    # BASELINE config 3 at its shorter length: 16 independent sequences of 4096 tokens in one launch,
+    # every one checked against the oracle, with and without scores.
+    b, hq, hkv, d, L = 16, 32, 8, 128, 4096
+    q = normal((b, hq, d), 42)
+    k = f16(normal((b, hkv, L, d), 137))
+    v = f16(normal((b, hkv, L, d), 53))
+    got, sc = run_decode(q, k, v, hkv, L, L, scores=True, batch=b, kv_batch_stride=hkv * L * d)
+    plain = run_decode(q, k, v, hkv, L, L, batch=b, kv_batch_stride=hkv * L * d)
+    for i in range(b):
+        ref, p = O.attention_gen(q[i], k[i], v[i], hkv, L, L, scores=True, impl="avx2")
+        check_attention_out(got[i], ref, "seq %d" % i)
+        check_attention_out(plain[i], ref, "seq %d, no scores" % i)
+        check_scores(sc[i], p, "seq %d" % i)
+
+
+def test_index_list_with_slots_at_and_beyond_the_capacity():
+    # Slots near capacity-1 are ordinary; an entry outside [0, capacity) must never steer a load out
+    # of the cache (the attended row for it is unspecified, so only the in-range lists are compared).
+    # Short rows, F32 caches and block formats read rows with plain loads, F16 rows through a bounded
+    # buffer descriptor: both kinds are covered.  The caches sit at the end of their allocations.
+    import argus_hip as A
+    hq, hkv, d, cap = 8, 2, 128, 96
+    for L, kind in ((40, "f16"), (80, "f16"), (40, "f32"), (80, "f32")):
+        q = normal((hq, d), L)
+        k, v = normal((hkv, cap, d), L + 1), normal((hkv, cap, d), L + 2)
+        if kind == "f16":
+            k, v = f16(k), f16(v)
+        idx = (cap - 1 - np.arange(L)).astype(np.int32)  # cap-1, cap-2, ...
+        got = run_decode(q, k, v, hkv, L, cap, kv_index=dev(idx))
+        check_attention_out(got, O.attention_gen(q, k, v, hkv, L, cap, kv_index=idx), "%s L%d" % (kind, L))
+        bad = idx.copy()
+        bad[3], bad[7] = cap + 5000000, -3
+        out = run_decode(q, k, v, hkv, L, cap, kv_index=dev(bad))
+        assert np.all(np.isfinite(out)), "%s L%d: stale slots" % (kind, L)
+    q = dev(normal((hq, d), 1))
+    kd = dev(f16(normal((hkv, cap, d), 2)))
+    out = dev(np.zeros((hq, d), np.float32))
+    ix = dev(np.arange(40, dtype=np.int32))
+    assert ctx().attention_gen(q, kd, kd, out, hkv, 40, 0, kv_index=ix, check=False) == A.ERR_INVALID
+    assert "capacity" in ctx().last_error()
+
+
+def test_head_dim_outside_the_kernels_is_refused_for_every_cache_type():
+    # return codes only: nothing is launched
+    import torch
+    import argus_hip as A
+    c = ctx()
+    for d in (32, 80, 96, 512):
+        q = torch.zeros((4, d), device="cuda")
+        out = torch.zeros((4, d), device="cuda")
+        kf = torch.zeros((2, 8, d), device="cuda", dtype=torch.float16)
+        assert c.attention_gen(q, kf, kf, out, 2, 8, 8, check=False) == A.ERR_UNSUPPORTED, d
+        assert c.attention_gen(q, kf.float(), kf.float(), out, 2, 8, 8, check=False) == A.ERR_UNSUPPORTED, d
+        if d % 32 == 0:
+            for kvt, bb in ((A.Q4_0, 18), (A.Q4_1, 20), (A.Q8_0, 34), (A.Q2_0, 12)):
+                blk = torch.zeros(2 * 8 * (d // 32) * bb + 64, device="cuda", dtype=torch.uint8)
+                assert c.attention_gen(q, blk, blk, out, 2, 8, 8, kv_dtype=kvt, check=False) == A.ERR_UNSUPPORTED, (d, kvt)
+                assert "head_dim" in c.last_error()
+    q = torch.zeros((4, 128), device="cuda")
+    blk = torch.zeros(1 << 16, device="cuda", dtype=torch.uint8)
+    assert c.attention_gen(q, blk, blk, q.clone(), 2, 8, 8, kv_dtype=9, check=False) == A.ERR_UNSUPPORTED
+
+
 def test_argument_errors_return_negative_codes():
     import torch
     import argus_hip as A
@@ -339,15 +404,15 @@ def test_argument_errors_return_negative_codes():
 
 @pytest.mark.parametrize("hq,hkv,d,L", [(8, 2, 64, 1023), (8, 2, 64, 1025), (12, 2, 128, 2047), (12, 2, 128, 2500),
                                         (32, 8, 128, 300), (24, 2, 128, 1531), (32, 2, 64, 4097), (16, 2, 128, 66)])
-def test_scores_stored_inside_the_token_loop(hq, hkv, d, L, monkeypatch):
+def test_scores_stored_inside_the_token_loop(hq, hkv, d, L):
     # Chunks too long for the LDS stage (beyond ~100K tokens at wide groups) write their logits from
-    # inside the token loop; ARGUS_HIP_SCORES=direct takes that path at test sizes.  Odd strides, rows
-    # cut inside a lane's token group, groups wider than eight heads.
-    monkeypatch.setenv("ARGUS_HIP_SCORES", "direct")
+    # inside the token loop; a context created under ARGUS_HIP_SCORES=direct takes that path at test
+    # sizes.  Odd strides, rows cut inside a lane's token group, groups wider than eight heads.
     cap = L + 19
     q = normal((hq, d), 42 + L)
     k, v = f16(normal((hkv, cap, d), 137 + L)), f16(normal((hkv, cap, d), 53 + L))
-    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, score_stride=cap)
+    got, sc = run_decode(q, k, v, hkv, L, cap, scores=True, score_stride=cap, context=direct_ctx())
+    assert direct_ctx().last_decode_plan()["staged_scores"] == 0, "logits were staged in LDS after all"
     ref, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, scores_stride=cap)
     check_attention_out(got, ref, "out")
     check_scores(sc[:, :L], p[:, :L], "scores")
