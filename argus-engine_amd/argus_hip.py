@@ -24,7 +24,7 @@ EXPORTED_SYMBOLS = [
     "argus_hip_read_buffer", "argus_hip_copy_slice", "argus_hip_synchronize",
     "argus_hip_create_ex", "argus_hip_reserve_workspace", "argus_hip_kernel_timing_end2",
     "argus_hip_write_buffer_range", "argus_hip_buffer_shift", "argus_hip_last_decode_plan",
-    "argus_hip_attention_gen", "argus_hip_flash_attention_prefill", "argus_hip_prefill_attention_scores",
+    "argus_hip_attention_gen", "argus_hip_attention_gen_noalloc", "argus_hip_flash_attention_prefill", "argus_hip_prefill_attention_scores",
     "argus_hip_has_quant_attn_kernel", "argus_hip_attention_gen_quant",
     "argus_hip_attention_gen_quant_ex", "argus_hip_gather_update_quant", "argus_hip_quant_flush",
     "argus_hip_quant_dequant_flush", "argus_hip_quant_scatter_residual",
@@ -173,6 +173,7 @@ def _bind():
     lib.argus_hip_copy_slice.argtypes = [vp, vp, vp, vp, C.c_size_t]
     lib.argus_hip_synchronize.argtypes = [vp, vp]
     lib.argus_hip_attention_gen.argtypes = [vp, C.POINTER(AttentionGenArgs)]
+    lib.argus_hip_attention_gen_noalloc.argtypes = [vp, C.POINTER(AttentionGenArgs)]
     lib.argus_hip_flash_attention_prefill.argtypes = [vp, C.POINTER(PrefillArgs)]
     lib.argus_hip_prefill_attention_scores.argtypes = [vp, C.POINTER(PfaArgs)]
     lib.argus_hip_kv_decode_descriptor.argtypes = [vp, vp, C.POINTER(KvLayoutDesc), vp, vp, C.c_int32, C.c_int64]
@@ -305,9 +306,10 @@ class Context:
     def attention_gen(self, q, k, v, out, num_heads_kv, cache_seq_len, capacity=0,
                       layout=HEAD_MAJOR, scores=None, score_stride=0, kv_index=None, kv_start=0,
                       batch=1, kv_batch_stride=0, index_batch_stride=0, softcap=0.0, scale=0.0,
-                      check=True, kv_dtype=None):
+                      check=True, kv_dtype=None, noalloc=False):
         """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride].
-        kv_dtype: Q4_0 / Q4_1 / Q8_0 / Q2_0 for uint8 tensors of blocks (default: from the tensor dtype)."""
+        kv_dtype: Q4_0 / Q4_1 / Q8_0 / Q2_0 for uint8 tensors of blocks (default: from the tensor dtype).
+        noalloc: go through argus_hip_attention_gen_noalloc (partials in the library's static array)."""
         hq, d = q.shape[-2], q.shape[-1]
         a = AttentionGenArgs(
             stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),
@@ -317,7 +319,8 @@ class Context:
             batch=batch, score_stride=score_stride, q_batch_stride=0, out_batch_stride=0,
             kv_batch_stride=kv_batch_stride, score_batch_stride=0,
             index_batch_stride=index_batch_stride, softcap=softcap, scale=scale)
-        return self._check(lib.argus_hip_attention_gen(self.handle, C.byref(a)), check)
+        fn = lib.argus_hip_attention_gen_noalloc if noalloc else lib.argus_hip_attention_gen
+        return self._check(fn(self.handle, C.byref(a)), check)
 
     # -- (a-2) ---------------------------------------------------------------------------
     def flash_attention_prefill(self, q, k, v, out, n_heads_q, n_heads_kv, seq_len, cache_seq_len,

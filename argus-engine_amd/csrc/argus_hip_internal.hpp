@@ -38,6 +38,12 @@ struct argus_hip_ctx {
   // argus_hip_reserve_workspace; a call that needs more grows it, which stalls the device.
   float *ws = nullptr;
   size_t ws_bytes = 0;
+  // This device's copy of the library's static scratch array (looked up when the context is
+  // created), and the lending of it: while ws_override is set, launchers take their partials from
+  // there instead of `ws` and never allocate.
+  float *scratch = nullptr;
+  float *ws_override = nullptr;
+  size_t ws_override_bytes = 0;
   // Scratch of the PFA side channel (logits of the trailing query rows); freed after a call that
   // made it large.
   float *pfa_ws = nullptr;
@@ -98,9 +104,10 @@ inline int argus_fail(argus_hip_ctx *ctx, int code, const char *fmt, ...) {
   } while (0)
 
 // Ensures the context workspace holds at least `bytes`; reallocation frees the old buffer
-// (hipFree synchronises the device, so no launch still reads it).
+// (hipFree synchronises the device, so no launch still reads it).  With a lent workspace
+// (ws_override) nothing is allocated: a request beyond it fails with ARGUS_HIP_ERR_NOMEM.
 int argus_ws_reserve(argus_hip_ctx *ctx, size_t bytes);
-inline float *argus_ws(argus_hip_ctx *ctx) { return ctx->ws; }
+inline float *argus_ws(argus_hip_ctx *ctx) { return ctx->ws_override ? ctx->ws_override : ctx->ws; }
 
 // Resident workgroups per compute unit of `fn` at `block` threads and `lds_bytes` of dynamic LDS,
 // queried once per (kernel, LDS size) on this context.

@@ -6,7 +6,39 @@
 #include <cstring>
 #include <new>
 
+// Scratch of the entry point that allocates nothing (argus_hip_attention_gen_noalloc): the split-KV
+// partials of one call.  Each device the library runs on holds its own copy of this array, at its
+// own address, until the process ends.  Host code never uses the array's name as an address: the
+// per-device address comes from hipGetSymbolAddress when a context is created on that device.
+constexpr size_t kScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static void *g_scratch_addr[kMaxDevices] = {nullptr};
+
+// With `device` current: the address of that device's copy of `scratch`, looked up once per device.
+static int scratch_lookup(argus_hip_ctx *ctx, int device) {
+  if (device < 0 || device >= kMaxDevices) return ARGUS_HIP_OK;  // no scratch there: the entry point refuses
+  if (!g_scratch_addr[device]) {
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return argus_fail(ctx, ARGUS_HIP_ERR_RUNTIME, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    }
+    g_scratch_addr[device] = ptr;
+  }
+  ctx->scratch = (float *)g_scratch_addr[device];
+  return ARGUS_HIP_OK;
+}
+
 int argus_ws_reserve(argus_hip_ctx *ctx, size_t bytes) {
+  if (ctx->ws_override) {
+    if (bytes <= ctx->ws_override_bytes) return ARGUS_HIP_OK;
+    return argus_fail(ctx, ARGUS_HIP_ERR_NOMEM,
+                      "attention_gen_noalloc: the call needs %zu bytes of split-KV partials, the static scratch holds %zu "
+                      "(use argus_hip_attention_gen, or fewer sequences per call)",
+                      bytes, ctx->ws_override_bytes);
+  }
   if (bytes <= ctx->ws_bytes) return ARGUS_HIP_OK;
   size_t want = ctx->ws_bytes ? ctx->ws_bytes : (size_t)1 << 22;
   while (want < bytes) want <<= 1;
@@ -61,7 +93,9 @@ ARGUS_API int argus_hip_create_ex(int device, const argus_hip_create_opts *opts,
     want = std::max(want, n_part * ((size_t)opts->max_head_dim + 2) * sizeof(float) + 256);
   }
   int rc = argus_ws_reserve(ctx, want);
+  if (rc == ARGUS_HIP_OK) rc = scratch_lookup(ctx, device);
   if (rc != ARGUS_HIP_OK) {
+    if (ctx->ws) (void)hipFree(ctx->ws);
     delete ctx;
     return rc;
   }
@@ -100,6 +134,20 @@ ARGUS_API int argus_hip_get_device_info(const argus_hip_ctx *ctx, argus_hip_devi
   strncpy(info->name, ctx->props.name, sizeof(info->name) - 1);
   strncpy(info->gcn_arch, ctx->props.gcnArchName, sizeof(info->gcn_arch) - 1);
   return ARGUS_HIP_OK;
+}
+
+// argus_hip_attention_gen with the split-KV partials in this device's copy of `scratch`: no
+// hipMalloc, hipFree or other allocating call on the way.  The partials a launch reads are all
+// written by the same launch's first pass, so nothing in the array has to start at zero.
+ARGUS_API int argus_hip_attention_gen_noalloc(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args) {
+  if (!ctx || !args) return ARGUS_HIP_ERR_INVALID;
+  if (!ctx->scratch) return argus_fail(ctx, ARGUS_HIP_ERR_RUNTIME, "attention_gen_noalloc: no static scratch on device %d", ctx->device);
+  ctx->ws_override = ctx->scratch;
+  ctx->ws_override_bytes = kScratchBytes;
+  const int rc = argus_hip_attention_gen(ctx, args);
+  ctx->ws_override = nullptr;
+  ctx->ws_override_bytes = 0;
+  return rc;
 }
 
 ARGUS_API int argus_hip_last_decode_plan(const argus_hip_ctx *ctx, argus_hip_decode_plan *plan) {

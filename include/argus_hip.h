@@ -176,6 +176,18 @@ typedef struct argus_hip_attention_gen_args {
 } argus_hip_attention_gen_args;
 int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, kernels and
+ * results as argus_hip_attention_gen, but the split-KV partials live in a 16 MiB static device array
+ * of the library (one copy per GPU, held until the process ends) and the call makes no hipMalloc /
+ * hipFree / allocating library call.  A call whose partials exceed the array -- batch * num_heads_q
+ * * splits * (head_dim + 2) * 4 bytes, e.g. more than ~250 sequences of the Llama-3-8B head shape
+ * without scores -- returns ARGUS_HIP_ERR_NOMEM with the sizes in argus_hip_last_error.  Every call
+ * on a GPU shares that GPU's array: calls that overlap on one GPU (different streams or contexts)
+ * race; nothing in the array needs clearing between calls.  Kernels are loaded on their first
+ * launch, so issue one call of each shape class before capturing. */
+int argus_hip_attention_gen_noalloc(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args);
+
 /* How the last attention_gen / attention_gen_quant call on this context was cut along the KV length
  * (diagnostics for benchmarks and tests; the reference has no split-KV on this path outside
  * engine/src/backend/cpu/neon.rs:261-300). */
