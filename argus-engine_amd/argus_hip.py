@@ -16,6 +16,13 @@ OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_RUNTIME, ERR_NOMEM = 0, -1, -2, -3, -4
 F32, F16 = 0, 1
 Q4_0, Q4_1, Q8_0, Q2_0 = 2, 3, 4, 5  # block-quantised cache rows (attention_gen)
 HEAD_MAJOR, SEQ_MAJOR = 0, 1
+# KVLayoutDesc tuples (block_elems, bits, scale_layout, packing) of the named --kv-format formats,
+# crates/argus-extension-api/src/lib.rs:1111-1159: scale_layout 1 PerBlockF16 / 2 PerBlockF16WithMin,
+# packing 1 Nibble / 2 Byte / 3 Quad.
+DESC_Q4_0 = (32, 4, 1, 1)
+DESC_Q4_1 = (32, 4, 2, 1)
+DESC_Q8_0 = (32, 8, 1, 2)
+DESC_Q2_0 = (32, 2, 2, 3)
 
 EXPORTED_SYMBOLS = [
     "argus_hip_create", "argus_hip_destroy", "argus_hip_abi_version", "argus_hip_last_error",

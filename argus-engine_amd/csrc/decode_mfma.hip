@@ -316,12 +316,30 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const DecodePa
       o += lds_acc[w][g][c] * f;
       ll += lds_l[w][g] * f;
     }
+    if (p.direct) {
+      // One split and no scores: the row is finished here and no combine pass follows.  A row
+      // without any finite logit is left to the fallback below.
+      if (ll > 0.0f && ll < __builtin_huge_valf()) p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = o / ll;
+      continue;
+    }
     // Partials are handed to the combine pass in natural-log units.
     const int64_t pidx = ((int64_t)b * p.n_heads_q + h) * p.nsplit + split;
     p.ws_o[pidx * D + c] = o;
     if (c == 0) {
       p.ws_ml[pidx * 2 + 0] = mm * kLn2;
       p.ws_ml[pidx * 2 + 1] = ll;
+    }
+  }
+  if (p.direct) {
+    for (int g = 0; g < G; ++g) {
+      float mm = lds_m[0][g];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, lds_m[w][g]);
+      const float m_ref = (mm == kNegInf) ? 0.0f : mm;
+      float ll = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) ll += lds_l[w][g] * __builtin_amdgcn_exp2f(lds_m[w][g] - m_ref);
+      if (!(ll > 0.0f && ll < __builtin_huge_valf())) uniform_fallback<_Float16>(p, b, kvh * G + g, D);  // uniform per workgroup
     }
   }
 }
@@ -340,19 +358,22 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves,
                                           max_chunk > 0 ? (size_t)kStageBytes : merge_bytes);
   choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
-  p.direct = 0;
+  p.direct = (p.nsplit == 1 && !p.scores) ? 1 : 0;  // the split pass writes `out` itself: one launch
   p.stage_scores = p.scores && p.chunk <= max_chunk;
   const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
   auto kern = cap ? (indexed ? decode_mfma_kernel<D, TW, true, true> : decode_mfma_kernel<D, TW, true, false>)
                   : (indexed ? decode_mfma_kernel<D, TW, false, true> : decode_mfma_kernel<D, TW, false, false>);
   ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + 1024));
-  const int rc = reserve_partials(ctx, p, batch, D);
-  if (rc != ARGUS_HIP_OK) return rc;
-  ctx->plan = argus_hip_decode_plan{p.nsplit, p.chunk, wgs_per_cu, (int32_t)lds_bytes, 2, 1, p.stage_scores};
+  if (!p.direct) {
+    const int rc = reserve_partials(ctx, p, batch, D);
+    if (rc != ARGUS_HIP_OK) return rc;
+  }
+  ctx->plan = argus_hip_decode_plan{p.nsplit, p.chunk, wgs_per_cu, (int32_t)lds_bytes, p.direct ? 1 : 2, 1, p.stage_scores};
   KernelTimer timer(ctx, stream);
   hipLaunchKernelGGL(kern, dim3(p.nsplit, p.n_heads_kv, batch), dim3(64 * kWaves), lds_bytes, stream, p);
   timer.mark();
+  if (p.direct) return hipGetLastError() == hipSuccess ? ARGUS_HIP_OK : argus_fail(ctx, ARGUS_HIP_ERR_RUNTIME, "decode launch failed");
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<UniformFallback<_Float16>, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
   ARGUS_HIP_CHECK(ctx, hipGetLastError());

@@ -190,6 +190,68 @@ class HipBackend {
 };
 
 // CudaScoreReduceBackend twin: the args struct is the reference POD field for field.
+// The compaction executor of the KV container on device buffers: KVCache::shift_positions,
+// shift_positions_for_head, compact_keep_positions and compact_keep_positions_for_head
+// (engine/src/kv/kv_cache.rs:1002-1100, 1266-1350), which is what a committed keep-list turns into
+// (engine/src/kv/cache_handle.rs:154-210).  Every move is Backend::buffer_shift, overlap-safe; the
+// caller sets current_pos afterwards, as in the reference.  F16 / F32 caches of either layout; the
+// per-head variants need HeadMajor.
+struct HipKvCache {
+  HipBackend *be = nullptr;
+  Tensor k, v;  // HeadMajor [kv_heads, capacity, head_dim] or SeqMajor [capacity, kv_heads, head_dim]
+  size_t kv_heads = 0, capacity = 0, head_dim = 0, current_pos = 0;
+  bool head_major = true;
+
+  Status shift_positions(size_t src_pos, size_t dst_pos, size_t count) {
+    if (count == 0 || src_pos == dst_pos) return OkStatus();
+    if (!head_major) {
+      const size_t epp = kv_heads * head_dim;
+      Status s = be->buffer_shift(k, src_pos * epp, dst_pos * epp, count * epp);
+      return s.ok() ? be->buffer_shift(v, src_pos * epp, dst_pos * epp, count * epp) : s;
+    }
+    for (size_t h = 0; h < kv_heads; ++h) {
+      Status s = shift_positions_for_head(h, src_pos, dst_pos, count);
+      if (!s.ok()) return s;
+    }
+    return OkStatus();
+  }
+  Status shift_positions_for_head(size_t head, size_t src_pos, size_t dst_pos, size_t count) {
+    if (!head_major) return Status::Err("shift_positions_for_head requires HeadMajor layout");
+    if (count == 0 || src_pos == dst_pos) return OkStatus();
+    const size_t base = head * capacity * head_dim;
+    Status s = be->buffer_shift(k, base + src_pos * head_dim, base + dst_pos * head_dim, count * head_dim);
+    return s.ok() ? be->buffer_shift(v, base + src_pos * head_dim, base + dst_pos * head_dim, count * head_dim) : s;
+  }
+  // `keep` ascending.  Consecutive source positions merge into one shift; a run already in place
+  // is skipped.  head < 0: every head.
+  Status compact_keep(const std::vector<size_t> &keep, size_t write_start, long head) {
+    if (keep.empty()) return OkStatus();
+    auto flush = [&](size_t src, size_t dst, size_t count) {
+      if (src == dst) return OkStatus();
+      return head < 0 ? shift_positions(src, dst, count) : shift_positions_for_head((size_t)head, src, dst, count);
+    };
+    size_t write_pos = write_start, src0 = keep[0], dst0 = write_pos, count = 1;
+    ++write_pos;
+    for (size_t i = 1; i < keep.size(); ++i) {
+      if (keep[i] == src0 + count) {
+        ++count;
+      } else {
+        Status s = flush(src0, dst0, count);
+        if (!s.ok()) return s;
+        src0 = keep[i];
+        dst0 = write_pos;
+        count = 1;
+      }
+      ++write_pos;
+    }
+    return flush(src0, dst0, count);
+  }
+  Status compact_keep_positions(const std::vector<size_t> &keep, size_t write_start) { return compact_keep(keep, write_start, -1); }
+  Status compact_keep_positions_for_head(size_t head, const std::vector<size_t> &keep, size_t write_start) {
+    return compact_keep(keep, write_start, (long)head);
+  }
+};
+
 class HipScoreReduceBackend {
  public:
   explicit HipScoreReduceBackend(argus_hip_ctx *ctx) : ctx_(ctx) {}

@@ -64,6 +64,37 @@ def time_region(fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def measure(ctx, step, steps, warmup):
+    """(wall seconds per step, dominant-kernel ms, tail ms).  The wall clock is taken over a pass that
+    records no events; the kernel durations come from a second pass in which the library brackets the
+    dominant kernel and the rest of the call (the combine pass) with HIP events on the launch stream."""
+    import torch
+    spin_up(step)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    ctx.kernel_timing_begin(steps)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    kms, tail = ctx.kernel_timing_end2(steps)
+    n = max(len(kms), 1)
+    return wall, sum(kms) / n, sum(tail) / n
+
+
+def result(wall, kernel_ms, tail_ms, nbytes, **more):
+    r = dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, combine_ms=tail_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
+             gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None,
+             gbps_kernels=nbytes / ((kernel_ms + tail_ms) * 1e-3) / 1e9 if kernel_ms else None)
+    r.update(more)
+    return r
+
+
 def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores=False, softcap=0.0,
                  rotate=1, seed=137):
     """Returns dict(ms_per_step, kernel_ms, bytes).  `rotate` distinct KV buffers are cycled so a
@@ -77,30 +108,19 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
         vs.append(torch.randn((batch, hkv, cap, d), generator=g, device="cuda", dtype=torch.float32).half())
     q = torch.randn((batch, hq, d), generator=g, device="cuda", dtype=torch.float32)
     out = torch.empty((batch, hq, d), device="cuda", dtype=torch.float32)
-    sc = torch.empty((batch, hq, cap), device="cuda", dtype=torch.float32) if scores else None
+    scs = [torch.empty((batch, hq, cap), device="cuda", dtype=torch.float32) for _ in range(rotate)] if scores else None
     state = {"i": 0}
 
     def step():
         i = state["i"] % rotate
         state["i"] += 1
-        ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, cap, scores=sc, score_stride=cap if scores else 0,
-                          batch=batch, kv_batch_stride=hkv * cap * d, softcap=softcap)
+        ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, cap, scores=scs[i] if scores else None,
+                          score_stride=cap if scores else 0, batch=batch, kv_batch_stride=hkv * cap * d, softcap=softcap)
 
-    spin_up(step)
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    ctx.kernel_timing_begin(steps)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    kms = ctx.kernel_timing_end(steps)
-    nbytes = decode_bytes(hq, hkv, d, L, batch, 2, scores)
-    kernel_ms = sum(kms) / max(len(kms), 1)
-    return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes,
-                gbps_wall=nbytes / wall / 1e9, gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None)
+    wall, kernel_ms, tail_ms = measure(ctx, step, steps, warmup)
+    r = result(wall, kernel_ms, tail_ms, decode_bytes(hq, hkv, d, L, batch, 2, scores))
+    r["plan"] = ctx.last_decode_plan()
+    return r
 
 
 def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1, scores=False):
@@ -136,22 +156,10 @@ def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1,
         ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, L, batch=batch, kv_batch_stride=hkv * L * d, kv_dtype=kv_dtype,
                           scores=sc, score_stride=L if scores else 0)
 
-    spin_up(step)
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    ctx.kernel_timing_begin(steps)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    kms = ctx.kernel_timing_end(steps)
-    kernel_ms = sum(kms) / max(len(kms), 1)
+    wall, kernel_ms, tail_ms = measure(ctx, step, steps, warmup)
     nbytes = batch * (2 * hkv * L * row_bytes + 2 * hq * d * 4 + (hq * L * 4 if scores else 0))
-    return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
-                gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None,
-                f16_equivalent_gbps_kernel=decode_bytes(hq, hkv, d, L, batch, 2, False) / (kernel_ms * 1e-3) / 1e9)
+    return result(wall, kernel_ms, tail_ms, nbytes,
+                  f16_equivalent_gbps_kernel=decode_bytes(hq, hkv, d, L, batch, 2, False) / (kernel_ms * 1e-3) / 1e9)
 
 
 def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res_cap=128, res_f16=False,
@@ -190,21 +198,9 @@ def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res
                                 1.0 / d ** 0.5, bits, batch=batch, block_batch_stride_bytes=nblk1 * bb,
                                 res_batch_stride=hkv * res_cap * d)
 
-    spin_up(step)
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    ctx.kernel_timing_begin(steps)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    kms = ctx.kernel_timing_end(steps)
+    wall, kernel_ms, tail_ms = measure(ctx, step, steps, warmup)
     nbytes = 2 * nblk * bb + batch * (2 * hkv * res_tokens * d * (2 if res_f16 else 4) + hq * d * 4 * 2)
-    kernel_ms = sum(kms) / max(len(kms), 1)
-    return dict(ms_per_step=wall * 1e3, kernel_ms=kernel_ms, bytes=nbytes, gbps_wall=nbytes / wall / 1e9,
-                gbps_kernel=nbytes / (kernel_ms * 1e-3) / 1e9)
+    return result(wall, kernel_ms, tail_ms, nbytes)
 
 
 def bench_prefill(ctx, steps, warmup, hq=32, hkv=8, d=64, s=2048, batch=1, f16_io=True):
@@ -221,18 +217,7 @@ def bench_prefill(ctx, steps, warmup, hq=32, hkv=8, d=64, s=2048, batch=1, f16_i
         rc = ctx.flash_attention_prefill(q, k, v, out, hq, hkv, s, s, d, s, batch_size=batch)
         assert rc == 1
 
-    spin_up(step)
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    ctx.kernel_timing_begin(steps)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
-    kms = ctx.kernel_timing_end(steps)
-    kernel_ms = sum(kms) / max(len(kms), 1)
+    wall, kernel_ms, _ = measure(ctx, step, steps, warmup)
     flops = 4 * hq * d * s * (s + 1) // 2 * batch
     return dict(us_per_call=round(wall * 1e6, 2), kernel_us=round(kernel_ms * 1e3, 2), causal_flops=flops,
                 tflops_kernel=round(flops / (kernel_ms * 1e-3) / 1e12, 1),
@@ -264,16 +249,24 @@ def bench_aux(ctx, steps, warmup):
 
     # (a-4) H2O score reduce: 32 layers x 32 heads of probabilities over 32768 positions
     nl, hq, hkv, L = 32, 32, 8, 32768
-    scores = torch.rand((nl, hq, L), generator=g, device="cuda")
+    # three score buffers of 137 MB are cycled: 411 MB, beyond the 256 MB Infinity Cache, so the rate is an HBM rate
+    bufs = [torch.rand((nl, hq, L), generator=g, device="cuda") for _ in range(3)]
     imp = torch.zeros(L, device="cuda")
     himp = torch.zeros(hkv * L, device="cuda")
     lf = torch.zeros(nl * L, device="cuda")
-    spin_up(lambda: ctx.score_reduce(scores, imp, himp, 0.9, nl, hq, hkv, L, L, L))
-    timed("score_reduce_L32768_32x32", lambda: ctx.score_reduce(scores, imp, himp, 0.9, nl, hq, hkv, L, L, L),
-          scores.numel() * 4 + 2 * (imp.numel() + himp.numel()) * 4, "fused importance + per-KV-head importance")
-    timed("score_reduce_per_layer_L32768_32x32", lambda: ctx.score_reduce_per_layer(scores, lf, 0.9, nl, hq, hkv, L, L, L),
-          scores.numel() * 4 + 2 * lf.numel() * 4, "per-layer importance")
-    del scores
+    turn = {"i": 0}
+
+    def next_scores():
+        turn["i"] += 1
+        return bufs[turn["i"] % len(bufs)]
+
+    spin_up(lambda: ctx.score_reduce(next_scores(), imp, himp, 0.9, nl, hq, hkv, L, L, L))
+    timed("score_reduce_L32768_32x32", lambda: ctx.score_reduce(next_scores(), imp, himp, 0.9, nl, hq, hkv, L, L, L),
+          bufs[0].numel() * 4 + 2 * (imp.numel() + himp.numel()) * 4,
+          "fused importance + per-KV-head importance; 3 score buffers cycled (411 MB)")
+    timed("score_reduce_per_layer_L32768_32x32", lambda: ctx.score_reduce_per_layer(next_scores(), lf, 0.9, nl, hq, hkv, L, L, L),
+          bufs[0].numel() * 4 + 2 * lf.numel() * 4, "per-layer importance; 3 score buffers cycled (411 MB)")
+    del bufs
 
     # (f-1) KV scatter of a 2048-token prefill chunk, F32 rows -> F16 HeadMajor cache
     hkv, d, cap, sl = 8, 128, 32768, 2048
@@ -288,7 +281,7 @@ def bench_aux(ctx, steps, warmup):
           2 * hkv * d * 6, "decode step: launch latency")
 
     # (f-4) descriptor codec over one layer's cache of 32768 tokens (8 KV heads x 128)
-    import oracle as O
+    import argus_hip as O  # the named descriptors
     n = 32768 * hkv * d
     x = torch.randn(n, generator=g, device="cuda")
     for name, desc, bb in (("q4_0", O.DESC_Q4_0, 18), ("q2_0", O.DESC_Q2_0, 12)):
@@ -355,9 +348,73 @@ def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
 
 
 # HBM bytes per launch of the primary workload's kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs
-# scaled by what the same counters read for a plain 1 GiB copy (x2.000 and x1.000); the runs and
-# their commands are summarised in profiles/decode_mfma_cfg3_L32768_b16_hbm_traffic.md.
+# scaled by what the same counters read for a plain 1 GiB copy (x2.000 and x1.000).  Counters cannot
+# be read from inside this process, so the figure is the one of the profile run named beside it in
+# the output (`traffic_source`), not a measurement of this run.
 DECODE_TRAFFIC_BYTES = 2_153_496_471
+DECODE_TRAFFIC_SOURCE = "profiles/decode_mfma_cfg3_L32768_b16_hbm_traffic.md"
+
+
+def bench_layer_loop(ctx, steps, warmup, hq=32, hkv=8, d=128, L=4096, layers=32):
+    """What a decode step of a model issues: one attention call per layer, back to back on one
+    stream, each layer with its own KV cache (32 x 16.8 MB = 537 MB, beyond the Infinity Cache).
+    Eager: the calls are issued from this process (its per-call cost is part of the figure).
+    Graph: the same 32 calls of the entry point that allocates nothing, captured once into a HIP
+    graph and replayed -- kernels only on the stream.  Returns microseconds per token (32 layers)."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(9)
+    ks = [torch.randn((hkv, L, d), generator=g, device="cuda").half() for _ in range(layers)]
+    vs = [torch.randn((hkv, L, d), generator=g, device="cuda").half() for _ in range(layers)]
+    q = torch.randn((layers, hq, d), generator=g, device="cuda")
+    out = torch.empty((layers, hq, d), device="cuda")
+
+    def token(noalloc=False):
+        for i in range(layers):
+            ctx.attention_gen(q[i], ks[i], vs[i], out[i], hkv, L, L, noalloc=noalloc)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    spin_up(token)
+    res = {"layers": layers, "kv_len": L, "eager_us_per_token": round(timed(token), 2)}
+    eager = out.clone()
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            token(noalloc=True)  # kernels loaded, launch facts cached before the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        out.zero_()
+        with torch.cuda.graph(graph, stream=side):
+            token(noalloc=True)
+        ok = True
+        for _ in range(3):  # every replay is checked against the eager result, with eager work in between
+            out.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            ok = ok and bool(torch.equal(out, eager))
+        res["graph_replays_match_eager"] = ok
+        res["graph_us_per_token"] = round(timed(graph.replay), 2)
+    except Exception as e:  # capture is optional: report why it is missing
+        res["graph_error"] = str(e)[:200]
+    nbytes = layers * decode_bytes(hq, hkv, d, L, 1)
+    res["bytes_per_token"] = nbytes
+    for k in ("eager", "graph"):
+        if k + "_us_per_token" in res:
+            res[k + "_gbps"] = round(nbytes / res[k + "_us_per_token"] / 1e3, 1)
+    return res
 
 
 def main():
@@ -369,7 +426,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
                     choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1",
-                             "q8_0", "copy_calib", "aux"],
+                             "q8_0", "copy_calib", "aux", "layers"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -397,6 +454,8 @@ def main():
             res = {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}
         elif w == "aux":
             res = bench_aux(ctx, args.steps, args.warmup)
+        elif w == "layers":
+            res = bench_layer_loop(ctx, args.steps, args.warmup)
         elif w == "decode_b1":
             res = bench_decode(ctx, 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=4)
         elif w == "prefill":
@@ -409,7 +468,7 @@ def main():
             res = bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=8)
         elif w == "cfg5":
             res = bench_decode(ctx, 8, 4, 256, 2048, 8, args.steps, args.warmup, capacity=4096, scores=True,
-                               softcap=50.0, rotate=4)
+                               softcap=50.0, rotate=8)
         else:
             res = bench_kivi(ctx, 4 if w == "kivi_q4" else 8, args.steps, args.warmup, batch=32, rotate=2)
         print(json.dumps({"workload": w, "steps": args.steps, "warmup": args.warmup, "result": res}))
@@ -432,13 +491,19 @@ def main():
         "data": "synthetic",
         "config": {"workload": "BASELINE config 3: split-KV decode attention, Llama-3.1-8B shape "
                                "(Hq32 Hkv8 d128), F16 KV, KV length 32768, batch 16, seeded N(0,1)",
-                   "kv_dtype": "f16", "accumulate": "f32", "batch": batch, "kv_len": L,
+                   "kv_dtype": "f16", "accumulate": "f32",
+                   "mfma_operands": "f16 (K and V as stored; Q as f16 hi + lo pair, probabilities rounded to f16); "
+                                    "logits, softmax, sums and outputs f32",
+                   "batch": batch, "kv_len": L,
                    "us_per_call": round(r["ms_per_step"] * 1e3, 2),
                    "tokens_per_s": round(batch / (r["ms_per_step"] * 1e-3), 1)},
         "roofline": {"bound": "hbm", "achieved": round(r["gbps_kernel"], 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(r["gbps_kernel"] / HBM_PEAK_GBPS, 4), "traffic": DECODE_TRAFFIC_BYTES,
+                     "traffic_source": DECODE_TRAFFIC_SOURCE,
                      "kernel": "decode_mfma_kernel<128,2>", "kernel_ms": round(r["kernel_ms"], 5),
-                     "algorithmic_bytes": r["bytes"]},
+                     "combine_ms": round(r["combine_ms"], 5),
+                     "frac_with_combine": round(r["gbps_kernels"] / HBM_PEAK_GBPS, 4),
+                     "algorithmic_bytes": r["bytes"], "plan": r["plan"]},
         "device": {"name": info.name.decode(), "arch": info.gcn_arch.decode(), "cus": info.compute_units,
                    "clock_mhz": info.clock_mhz},
     }
@@ -450,8 +515,10 @@ def main():
         def add(name, res, note=""):
             ex[name] = {"us_per_call": round(res["ms_per_step"] * 1e3, 2),
                         "kernel_us": round(res["kernel_ms"] * 1e3, 2),
+                        "combine_us": round(res["combine_ms"] * 1e3, 2),
                         "gbps_kernel": round(res["gbps_kernel"], 1),
                         "hbm_frac_kernel": round(res["gbps_kernel"] / HBM_PEAK_GBPS, 4),
+                        "hbm_frac_with_combine": round(res["gbps_kernels"] / HBM_PEAK_GBPS, 4),
                         "bytes": res["bytes"], "note": note}
 
         add("cfg3_L32768_b1", bench_decode(ctx, 32, 8, 128, 32768, 1, es, ew, rotate=4),
@@ -459,11 +526,11 @@ def main():
         add("cfg3_L4096_b16", bench_decode(ctx, 32, 8, 128, 4096, 16, es, ew, rotate=2), "2 sets rotated")
         add("cfg3_L4096_b1", bench_decode(ctx, 32, 8, 128, 4096, 1, es, ew, rotate=16), "16 sets rotated")
         add("cfg3_L32768_b16_scores", bench_decode(ctx, 32, 8, 128, 32768, 16, es, ew, scores=True),
-            "scores emitted (67 MB of logits per call); kernel time covers the split pass only, us_per_call the combine's rewrite too")
+            "scores emitted (67 MB of logits per call); combine_us is the pass that rewrites them as probabilities")
         add("cfg1_qwen_L1024_b1", bench_decode(ctx, 14, 2, 64, 1024, 1, es, ew), "latency-bound (0.5 MiB)")
         add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
-            bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=4),
-            "scores emitted; kernel time covers the split pass only")
+            bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=8),
+            "scores emitted; 8 KV and score buffer sets rotated (537 MB of attended rows)")
         add("cfg4_kivi_q4_L8192_res128_f32", bench_kivi(ctx, 4, es, ew), "8 block sets rotated; single launch, 11.4 MB")
         add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")
         add("cfg4_kivi_q4_L8192_res128_f16", bench_kivi(ctx, 4, es, ew, res_f16=True), "F16 residual window")
@@ -486,6 +553,9 @@ def main():
         ex["cfg2_prefill_llama1b_S2048_f16"] = bench_prefill(ctx, es, ew)
         ex["cfg2_prefill_llama1b_S2048_f32io"] = bench_prefill(ctx, es, ew, f16_io=False)
         ex["prefill_llama8b_d128_S8192_f16"] = bench_prefill(ctx, max(5, es // 4), 2, hq=32, hkv=8, d=128, s=8192)
+        ex["prefill_d64_by_seq_len"] = {str(sl): bench_prefill(ctx, max(5, es // 4), 2, s=sl)["mfma_frac_kernel"]
+                                        for sl in (1024, 2048, 4096, 8192, 16384)}
+        ex["decode_32_layers_cfg3_L4096_b1"] = bench_layer_loop(ctx, max(5, es // 4), 2)
         line["extras"] = ex
 
     if not args.no_cpu:

@@ -192,6 +192,17 @@ static float vec_dot_f16_f32_avx2(int k, const float *a, const uint16_t *b) {
 static void vec_mad_f16_avx2(int k, float *out, const uint16_t *v, float weight) {
   const __m256 w = _mm256_set1_ps(weight);
   int i = 0;
+  /* main loop: 32 elements per iteration, as x86.rs:682-705 */
+  for (; i + 32 <= k; i += 32) {
+    __m256 v0 = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(v + i)));
+    __m256 v1 = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(v + i + 8)));
+    __m256 v2 = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(v + i + 16)));
+    __m256 v3 = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(v + i + 24)));
+    _mm256_storeu_ps(out + i, _mm256_fmadd_ps(w, v0, _mm256_loadu_ps(out + i)));
+    _mm256_storeu_ps(out + i + 8, _mm256_fmadd_ps(w, v1, _mm256_loadu_ps(out + i + 8)));
+    _mm256_storeu_ps(out + i + 16, _mm256_fmadd_ps(w, v2, _mm256_loadu_ps(out + i + 16)));
+    _mm256_storeu_ps(out + i + 24, _mm256_fmadd_ps(w, v3, _mm256_loadu_ps(out + i + 24)));
+  }
   for (; i + 8 <= k; i += 8) {
     __m256 v0 = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(v + i)));
     _mm256_storeu_ps(out + i, _mm256_fmadd_ps(w, v0, _mm256_loadu_ps(out + i)));

@@ -346,6 +346,61 @@ def compact_keep(src, keep, dst_capacity):
     return dst
 
 
+def h2o_keep_spec(current, hh_size, recent_size, protected_prefix=0, importance=None, head_scores=None):
+    """H2o::partition + H2o::keep_spec, crates/techniques/h2o/src/lib.rs:118-160.
+    Returns None (already within the absolute budget prefix + hh_size + recent_size),
+    ("per_head", [keep per KV head]) when per-(kv_head, pos) scores are present, else
+    ("layer", keep) from the flat importance, or from recency alone when there are no scores
+    (the whole evictable budget hh_size + recent_size goes to the recent window, lib.rs:95-106).
+    importance: [>= 0 entries]; positions past its end score 0.0 (`imp.get(pos).unwrap_or(0.0)`).
+    head_scores: [n_kv_heads, >= current]."""
+    prefix = min(protected_prefix, current)
+    if current <= prefix + hh_size + recent_size:
+        return None
+    if head_scores is not None:
+        hs = np.asarray(head_scores, np.float32)
+        return "per_head", [compile_keep_top_k(current, prefix, recent_size, hh_size, hs[h, :current]) for h in range(hs.shape[0])]
+    if importance is not None:
+        imp = np.zeros(current, np.float32)
+        n = min(current, len(importance))
+        imp[:n] = np.asarray(importance, np.float32)[:n]
+        return "layer", compile_keep_top_k(current, prefix, recent_size, hh_size, imp)
+    return "layer", compile_keep_top_k(current, prefix, hh_size + recent_size, 0, None)
+
+
+def keep_batches(keep, write_start=0):
+    """The runs KVCache::compact_keep_positions moves (engine/src/kv/kv_cache.rs:1266-1306): consecutive
+    source positions merge into one shift; a run already in place is skipped.  Yields (src, dst, count)
+    in the order the reference issues them."""
+    keep = [int(x) for x in keep]
+    if not keep:
+        return
+    write_pos = write_start
+    src0, dst0, count = keep[0], write_pos, 1
+    write_pos += 1
+    for pos in keep[1:]:
+        if pos == src0 + count:
+            count += 1
+        else:
+            if src0 != dst0:
+                yield src0, dst0, count
+            src0, dst0, count = pos, write_pos, 1
+        write_pos += 1
+    if src0 != dst0:
+        yield src0, dst0, count
+
+
+def compact_keep_in_place(cache, keep, head=None, write_start=0):
+    """compact_keep_positions / compact_keep_positions_for_head on a HeadMajor [Hkv, cap, d] array, in
+    place, through the same overlap-safe row shifts (shift_positions, kv_cache.rs:1002-1100: one
+    buffer_shift per head and run)."""
+    heads = range(cache.shape[0]) if head is None else (head,)
+    for src, dst, count in keep_batches(keep, write_start):
+        for h in heads:
+            cache[h, dst:dst + count] = cache[h, src:src + count].copy()  # memmove
+    return cache
+
+
 def kv_scatter(k_src, v_src, k_dst, v_dst, write_pos_start):
     """kv_scatter_f32_to_f16[_batch] / _f32_batch.  src [S, Hkv, d] f32; dst [Hkv, cap, d]."""
     k_src = np.ascontiguousarray(k_src, np.float32)

@@ -309,8 +309,60 @@ static void test_quant_attn(HipBackend &be) {
   printf("[kivi] degraded handle, gather_update, residual-only attention + host score read-back ok\n");
 }
 
+// A committed keep-list on a device cache: compaction through overlapping buffer_shift runs must
+// equal the gather cache[:, keep] (engine/src/kv/naive_reference.rs), per layer and per head; then
+// write_buffer_range into the freed tail.
+static void test_compaction_and_memory(HipBackend &be) {
+  const size_t hkv = 3, cap = 64, hd = 64, cur = 50;
+  std::vector<float> host_k(hkv * cap * hd), host_v(hkv * cap * hd);
+  for (size_t i = 0; i < host_k.size(); ++i) {
+    host_k[i] = (float)(i % 977) * 0.25f;
+    host_v[i] = -(float)(i % 613);
+  }
+  DevBuf dk(&be, host_k.size() * 4, host_k.data()), dv(&be, host_v.size() * 4, host_v.data());
+  HipKvCache c;
+  c.be = &be;
+  c.k = Tensor{dk.p, DType::F32, {1, hkv, cap, hd}, true};
+  c.v = Tensor{dv.p, DType::F32, {1, hkv, cap, hd}, true};
+  c.kv_heads = hkv; c.capacity = cap; c.head_dim = hd; c.current_pos = cur; c.head_major = true;
+  // sinks 0..3, two heavy runs, the recent window: runs overlap their destinations
+  std::vector<size_t> keep = {0, 1, 2, 3, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 30, 31, 40, 41, 42, 43, 44, 45, 46, 47, 48, 49};
+  CHECK(c.compact_keep_positions(keep, 0).ok(), "compact_keep_positions");
+  std::vector<float> got(host_k.size());
+  be.read_buffer(got.data(), dk.p, got.size() * 4);
+  bool same = true;
+  for (size_t h = 0; h < hkv; ++h)
+    for (size_t i = 0; i < keep.size(); ++i)
+      for (size_t d = 0; d < hd; ++d) same = same && got[(h * cap + i) * hd + d] == host_k[(h * cap + keep[i]) * hd + d];
+  CHECK(same, "compacted K rows equal the gather");
+  be.read_buffer(got.data(), dv.p, got.size() * 4);
+  same = true;
+  for (size_t h = 0; h < hkv; ++h)
+    for (size_t i = 0; i < keep.size(); ++i)
+      for (size_t d = 0; d < hd; ++d) same = same && got[(h * cap + i) * hd + d] == host_v[(h * cap + keep[i]) * hd + d];
+  CHECK(same, "compacted V rows equal the gather");
+  // per head: head 1 of a fresh copy only
+  be.write_buffer(dk.p, host_k.data(), host_k.size() * 4);
+  std::vector<size_t> keep1 = {2, 3, 4, 20, 21, 22, 23, 49};
+  CHECK(c.compact_keep_positions_for_head(1, keep1, 0).ok(), "compact_keep_positions_for_head");
+  be.read_buffer(got.data(), dk.p, got.size() * 4);
+  same = true;
+  for (size_t i = 0; i < keep1.size(); ++i)
+    for (size_t d = 0; d < hd; ++d) same = same && got[(1 * cap + i) * hd + d] == host_k[(1 * cap + keep1[i]) * hd + d];
+  for (size_t i = 0; i < cap * hd; ++i) same = same && got[i] == host_k[i] && got[2 * cap * hd + i] == host_k[2 * cap * hd + i];
+  CHECK(same, "per-head compaction moves that head only");
+  // write_buffer_range: bounds-checked upload into the tail
+  std::vector<float> patch(hd, 7.5f);
+  CHECK(be.write_buffer_range(dk.p, host_k.size() * 4, patch.data(), hd * 4, (cap - 1) * hd * 4).ok(), "write_buffer_range");
+  CHECK(!be.write_buffer_range(dk.p, host_k.size() * 4, patch.data(), hd * 4, host_k.size() * 4 - 8).ok(), "write_buffer_range out of bounds");
+  be.read_buffer(got.data(), dk.p, got.size() * 4);
+  CHECK(got[(cap - 1) * hd] == 7.5f && got[(cap - 1) * hd + hd - 1] == 7.5f && got[(cap - 1) * hd - 1] == host_k[(cap - 1) * hd - 1],
+        "write_buffer_range landed at the offset");
+  printf("[kv] compaction through buffer_shift (layer and per head), write_buffer_range ok\n");
+}
+
 int main() {
-  auto r = HipBackend::create(0);
+  auto r = HipBackend::create(0, 16, 32, 128, 32768);
   if (!r.ok()) {
     printf("no HIP device: %s\n", r.error().c_str());
     return 77;
@@ -322,6 +374,7 @@ int main() {
   test_accumulator_binding(be);
   test_prefill_and_scatter(be);
   test_quant_attn(be);
+  test_compaction_and_memory(be);
   if (g_fail) {
     printf("%d check(s) FAILED\n", g_fail);
     return 1;

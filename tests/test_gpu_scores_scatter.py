@@ -124,3 +124,74 @@ def test_config5_post_eviction_h2o_flow(batch, softcap):
         check_scores(host(himp), oh, "head importance")
         flat, head = T.score_reduce(T.decode_attention(q[b], kc[b], vc[b], hkv, L, softcap=softcap)[1][None], hkv)
         check_scores(host(imp)[:L], flat, "importance vs f64")
+
+
+@pytest.mark.parametrize("hq,hkv,d,L,cap,softcap", [(8, 4, 256, 3000, 4096, 50.0), (32, 8, 128, 2500, 4096, 0.0)])
+def test_h2o_loop_scores_to_keep_list_to_post_eviction_attention(hq, hkv, d, L, cap, softcap):
+    # The loop BASELINE config 5 feeds, closed on the device: three decode steps emit scores, the fused
+    # reduce accumulates importance (decay 0) and per-KV-head importance, H2O's keep-spec
+    # (crates/techniques/h2o/src/lib.rs:138-160: flat, then per head) turns them into keep-lists on
+    # the host, and the next decode attends the survivors (a) through kv_index over the untouched
+    # cache, (b) over a cache compacted in place on the device by the reference's runs of overlapping
+    # buffer_shift moves (engine/src/kv/kv_cache.rs:1266-1350) -- both must equal the oracle's
+    # gather-then-attend, and the keep-lists made from device scores must be the oracle's.
+    import torch
+    steps, hh, recent, prefix = 3, 256, 512, 4
+    k = f16(normal((hkv, cap, d), 137))
+    v = f16(normal((hkv, cap, d), 53))
+    kd, vd = dev(k), dev(v)
+    imp = torch.zeros(cap, device="cuda")
+    himp = torch.zeros(hkv * cap, device="cuda")
+    oi, oh = np.zeros(cap, np.float32), np.zeros(hkv * cap, np.float32)
+    for s in range(steps):
+        q = normal((hq, d), 42 + s)
+        out = torch.empty((hq, d), device="cuda")
+        sc = torch.zeros((hq, cap), device="cuda")
+        ctx().attention_gen(dev(q), kd, vd, out, hkv, L, cap, scores=sc, score_stride=cap, softcap=softcap)
+        ctx().score_reduce(sc, imp, himp, 1.0, 1, hq, hkv, L, cap, cap)
+        _, p = O.attention_gen(q, k, v, hkv, L, cap, scores=True, scores_stride=cap, softcap=softcap)
+        O.score_fused_reduce(p, oi, oh, 1.0, 1, hq, hkv, L, cap, cap)
+    check_scores(host(imp)[:L], oi[:L], "cumulative importance")
+    check_scores(host(himp).reshape(hkv, cap)[:, :L], oh.reshape(hkv, cap)[:, :L], "cumulative head importance")
+
+    q = normal((hq, d), 99)
+    # (1) flat keep-list from the layer-wide importance
+    kind, keep = O.h2o_keep_spec(L, hh, recent, prefix, importance=host(imp))
+    kind_o, keep_o = O.h2o_keep_spec(L, hh, recent, prefix, importance=oi)
+    assert kind == kind_o == "layer" and len(keep) == prefix + hh + recent
+    assert np.array_equal(keep, keep_o), "keep-list from device scores differs from the oracle's"
+    n = len(keep)
+    ref = O.attention_gen(q, O.compact_keep(k, keep, cap), O.compact_keep(v, keep, cap), hkv, n, cap, softcap=softcap)
+    out = torch.empty((hq, d), device="cuda")
+    ctx().attention_gen(dev(q), kd, vd, out, hkv, n, cap, kv_index=dev(keep.astype(np.int32)), softcap=softcap)
+    check_attention_out(host(out), ref, "through kv_index")
+    kc, vc = kd.clone(), vd.clone()
+    for src, dst, count in O.keep_batches(keep):
+        for h in range(hkv):
+            base = h * cap * d
+            ctx().buffer_shift(kc, base + src * d, base + dst * d, count * d)
+            ctx().buffer_shift(vc, base + src * d, base + dst * d, count * d)
+    assert np.array_equal(host(kc)[:, :n], k[:, keep]) and np.array_equal(host(vc)[:, :n], v[:, keep])
+    ctx().attention_gen(dev(q), kc, vc, out, hkv, n, cap, softcap=softcap)
+    check_attention_out(host(out), ref, "over the compacted cache")
+
+    # (2) per-head keep-lists from the per-KV-head importance: every head compacts its own survivors
+    kind, heads = O.h2o_keep_spec(L, hh, recent, prefix, head_scores=host(himp).reshape(hkv, cap))
+    kind_o, heads_o = O.h2o_keep_spec(L, hh, recent, prefix, head_scores=oh.reshape(hkv, cap))
+    assert kind == kind_o == "per_head"
+    assert all(np.array_equal(a, b) for a, b in zip(heads, heads_o)), "per-head keep-lists differ from the oracle's"
+    assert any(not np.array_equal(heads[0], h) for h in heads[1:]), "heads should rank their own heavy hitters"
+    kc, vc = kd.clone(), vd.clone()
+    kg, vg = np.zeros_like(k), np.zeros_like(v)
+    for h in range(hkv):
+        kg[h, :n], vg[h, :n] = k[h, heads[h]], v[h, heads[h]]
+        base = h * cap * d
+        for src, dst, count in O.keep_batches(heads[h]):
+            ctx().buffer_shift(kc, base + src * d, base + dst * d, count * d)
+            ctx().buffer_shift(vc, base + src * d, base + dst * d, count * d)
+    assert np.array_equal(host(kc)[:, :n], kg[:, :n]) and np.array_equal(host(vc)[:, :n], vg[:, :n])
+    sc = torch.zeros((hq, cap), device="cuda")
+    ctx().attention_gen(dev(q), kc, vc, out, hkv, n, cap, scores=sc, score_stride=cap, softcap=softcap)
+    ref, p = O.attention_gen(q, kg, vg, hkv, n, cap, scores=True, scores_stride=cap, softcap=softcap)
+    check_attention_out(host(out), ref, "per-head compaction")
+    check_scores(host(sc)[:, :n], p[:, :n], "scores after per-head compaction")
