@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
           if (sub == g && g < gcount && valid[u])
-            p.scores[(int64_t)b * p.score_bs + (int64_t)(hbase + g) * p.score_stride + t] = s[u][g];
+            __builtin_nontemporal_store(s[u][g], p.scores + (int64_t)b * p.score_bs + (int64_t)(hbase + g) * p.score_stride + t);
         }
       }
     }

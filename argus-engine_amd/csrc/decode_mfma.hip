@@ -350,9 +350,12 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   constexpr int tile_rows = kWaves * 16 * TW;  // one tile per wave
   const int pairs = batch * p.n_heads_kv;
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
-  // token loop is over (kStageBytes; two workgroups per CU still fit).  The resident round is counted
-  // at the LDS size the launch may reach.
-  constexpr int kStageBytes = 64 * 1024;
+  // token loop is over (kStageBytes; two workgroups per CU still fit beside the 9 KB of static LDS).
+  // 66 KB and not 64: a group of four heads then stages chunks of 4096 tokens (4 x 4100 floats), so a
+  // 32K-token row is 8 chunks and 16 sequences x 8 KV heads fill exactly two resident rounds; at
+  // 64 KB the same row took 9 chunks, i.e. 2.25 rounds, and the thin third round cost 30 % of the
+  // launch.  The resident round is counted at the LDS size the launch may reach.
+  constexpr int kStageBytes = 66 * 1024;
   constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * MfmaShape<D>::MAXH * (D + 4)) * sizeof(float);
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
   const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves,
