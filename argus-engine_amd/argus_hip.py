@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = [
     "argus_hip_score_reduce", "argus_hip_score_reduce_per_layer",
     "argus_hip_kv_scatter_f32_to_f16", "argus_hip_kv_scatter_f32_to_f16_batch",
     "argus_hip_kv_scatter_f32_batch", "argus_hip_kv_decode_descriptor", "argus_hip_kv_encode_descriptor",
+    "argus_hip_attention_gen_desc",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -181,6 +182,7 @@ def _bind():
     lib.argus_hip_synchronize.argtypes = [vp, vp]
     lib.argus_hip_attention_gen.argtypes = [vp, C.POINTER(AttentionGenArgs)]
     lib.argus_hip_attention_gen_noalloc.argtypes = [vp, C.POINTER(AttentionGenArgs)]
+    lib.argus_hip_attention_gen_desc.argtypes = [vp, C.POINTER(AttentionGenArgs), C.POINTER(KvLayoutDesc)]
     lib.argus_hip_flash_attention_prefill.argtypes = [vp, C.POINTER(PrefillArgs)]
     lib.argus_hip_prefill_attention_scores.argtypes = [vp, C.POINTER(PfaArgs)]
     lib.argus_hip_kv_decode_descriptor.argtypes = [vp, vp, C.POINTER(KvLayoutDesc), vp, vp, C.c_int32, C.c_int64]
@@ -313,19 +315,24 @@ class Context:
     def attention_gen(self, q, k, v, out, num_heads_kv, cache_seq_len, capacity=0,
                       layout=HEAD_MAJOR, scores=None, score_stride=0, kv_index=None, kv_start=0,
                       batch=1, kv_batch_stride=0, index_batch_stride=0, softcap=0.0, scale=0.0,
-                      check=True, kv_dtype=None, noalloc=False):
+                      check=True, kv_dtype=None, noalloc=False, desc=None):
         """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride].
         kv_dtype: Q4_0 / Q4_1 / Q8_0 / Q2_0 for uint8 tensors of blocks (default: from the tensor dtype).
-        noalloc: go through argus_hip_attention_gen_noalloc (partials in the library's static array)."""
+        noalloc: go through argus_hip_attention_gen_noalloc (partials in the library's static array).
+        desc: KVLayoutDesc tuple of a uint8 cache of blocks: go through argus_hip_attention_gen_desc."""
         hq, d = q.shape[-2], q.shape[-1]
         a = AttentionGenArgs(
             stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),
             scores_out=_ptr(scores), kv_index=_ptr(kv_index), num_heads_q=hq,
             num_heads_kv=num_heads_kv, head_dim=d, cache_seq_len=cache_seq_len, capacity=capacity,
-            kv_start=kv_start, layout=layout, kv_dtype=_kv_dtype(k) if kv_dtype is None else kv_dtype,
+            kv_start=kv_start, layout=layout,
+            kv_dtype=0 if desc is not None else _kv_dtype(k) if kv_dtype is None else kv_dtype,
             batch=batch, score_stride=score_stride, q_batch_stride=0, out_batch_stride=0,
             kv_batch_stride=kv_batch_stride, score_batch_stride=0,
             index_batch_stride=index_batch_stride, softcap=softcap, scale=scale)
+        if desc is not None:
+            dd = KvLayoutDesc(*desc)
+            return self._check(lib.argus_hip_attention_gen_desc(self.handle, C.byref(a), C.byref(dd)), check)
         fn = lib.argus_hip_attention_gen_noalloc if noalloc else lib.argus_hip_attention_gen
         return self._check(fn(self.handle, C.byref(a)), check)
 

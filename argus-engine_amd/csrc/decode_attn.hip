@@ -40,6 +40,28 @@ struct KvVec<float> {
   static constexpr int E = 4;
   using vec = float4_t;
 };
+// Descriptor-driven rows: a lane decodes 8 consecutive channels of its row's block.
+typedef float float8_t __attribute__((ext_vector_type(8)));
+template <>
+struct KvVec<DescRow> {
+  static constexpr int E = 8;
+  using vec = float8_t;
+};
+
+// The lane's piece (E channels from c0) of the row in `slot` of one KV head.
+template <typename KV_T>
+__device__ __forceinline__ typename KvVec<KV_T>::vec load_row_piece(const DecodeParams &p, const void *cache, int64_t head_elem, int64_t slot,
+                                                                     int c0) {
+  using vec_t = typename KvVec<KV_T>::vec;
+  if constexpr (std::is_same<KV_T, DescRow>::value) {
+    const int64_t elem = head_elem + slot * p.row_stride + c0;
+    float v[8];
+    desc_decode8(p, (const uint8_t *)cache + desc_block_offset(p, elem), (int)(elem % p.desc_block_elems), v);
+    return float8_t{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]};
+  } else {
+    return __builtin_nontemporal_load((const vec_t *)((const KV_T *)cache + head_elem + slot * p.row_stride + c0));
+  }
+}
 
 enum DecodeMode { kPlain = 0, kSoftcap = 1, kGeneric = 2 };
 
@@ -65,8 +87,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
   const int t_begin = split * p.chunk;
   const int t_end = min(p.len, t_begin + p.chunk);
 
-  const KV_T *kb = (const KV_T *)p.k + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride + c0;
-  const KV_T *vb = (const KV_T *)p.v + (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride + c0;
+  const int64_t head_elem = (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride;  // first element of this KV head's rows
   const int32_t *idx = p.kv_index ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
 
   // This lane's slice of every query head of the group (heads beyond the group are clamped
@@ -106,8 +127,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
       // a slot outside the cache (stale or negative list entry) is clamped to the last one: the rows
       // are fetched with plain loads, which nothing else bounds
       const int64_t slot = use_idx ? (int64_t)min((uint32_t)idx[tc], (uint32_t)(p.slot_bound - 1)) : (int64_t)(p.kv_start + tc);
-      kr[u] = __builtin_nontemporal_load((const vec_t *)(kb + slot * p.row_stride));
-      vr[u] = __builtin_nontemporal_load((const vec_t *)(vb + slot * p.row_stride));
+      kr[u] = load_row_piece<KV_T>(p, p.k, head_elem, slot, c0);
+      vr[u] = load_row_piece<KV_T>(p, p.v, head_elem, slot, c0);
     }
 
     float s[U][GT];
@@ -249,6 +270,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
 template <int D, int GT, typename KV_T>
 constexpr int unroll_for() {
   // Keep q + acc + in-flight K/V rows inside the register file at >= 2 waves per SIMD.
+  if (std::is_same<KV_T, DescRow>::value) return GT >= 4 ? 1 : 2;  // decoded rows are 8 floats per piece
   return GT >= 8 ? 2 : (GT >= 4 ? 4 : 8);
 }
 
@@ -315,7 +337,11 @@ int dispatch_dim(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, bool wan
 
 }  // namespace
 
-ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *a) {
+// kv_dtype value used internally for rows described by `desc`
+constexpr int kKvDesc = 100;
+
+static int attention_gen_impl(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *a, int kv_dtype,
+                              const argus_hip_kv_layout_desc *desc, int desc_block_bytes) {
   if (!ctx || !a) return ARGUS_HIP_ERR_INVALID;
   if (!a->q || !a->k_cache || !a->v_cache || !a->out)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: null tensor pointer");
@@ -373,10 +399,18 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
   if (a->batch > 1 && p.kv_bs == 0)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: batch > 1 needs kv_batch_stride");
   // The kernels move K/V rows and output rows as 16-byte vectors.
-  const bool blocks = a->kv_dtype == ARGUS_HIP_Q4_0 || a->kv_dtype == ARGUS_HIP_Q4_1 || a->kv_dtype == ARGUS_HIP_Q8_0 ||
-                      a->kv_dtype == ARGUS_HIP_Q2_0;
-  const int64_t kv_vec = blocks ? 32 : (a->kv_dtype == ARGUS_HIP_F16 ? 8 : 4);
-  if (((uintptr_t)a->k_cache | (uintptr_t)a->v_cache | (uintptr_t)a->out) & 15)
+  const bool blocks = kv_dtype == ARGUS_HIP_Q4_0 || kv_dtype == ARGUS_HIP_Q4_1 || kv_dtype == ARGUS_HIP_Q8_0 || kv_dtype == ARGUS_HIP_Q2_0;
+  const int64_t kv_vec = kv_dtype == kKvDesc ? desc->block_elems : blocks ? 32 : (kv_dtype == ARGUS_HIP_F16 ? 8 : 4);
+  if (kv_dtype == kKvDesc) {
+    p.desc_block_elems = (int32_t)desc->block_elems;
+    p.desc_bits = desc->bits;
+    p.desc_scale_layout = (int32_t)desc->scale_layout;
+    p.desc_packing = (int32_t)desc->packing;
+    p.desc_block_bytes = desc_block_bytes;
+    // rows are whole blocks; blocks are read as 16-bit units
+    if ((p.row_stride % kv_vec) || (p.head_stride % kv_vec) || (((uintptr_t)a->k_cache | (uintptr_t)a->v_cache) & 1) || ((uintptr_t)a->out & 15))
+      return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen_desc: strides must be whole blocks, caches 2-byte and out 16-byte aligned");
+  } else if (((uintptr_t)a->k_cache | (uintptr_t)a->v_cache | (uintptr_t)a->out) & 15)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: k/v/out must be 16-byte aligned");
   if ((p.kv_bs % kv_vec) || (p.out_bs % 4))
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: batch strides must keep 16-byte alignment");
@@ -385,11 +419,53 @@ ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attent
   const bool want_scores = a->scores_out != nullptr;
   // ARGUS_HIP_DECODE=valu (read when the context is created) keeps the vector-ALU kernel for A/B measurements.
   const bool force_valu = ctx->env.decode_valu;
-  if (blocks) return launch_decode_blocks(ctx, p, D, a->kv_dtype, a->batch, stream);
-  if (!force_valu && decode_mfma_supported(p, D, a->kv_dtype)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
-  switch (a->kv_dtype) {
+  if (blocks) return launch_decode_blocks(ctx, p, D, kv_dtype, a->batch, stream);
+  if (!force_valu && decode_mfma_supported(p, D, kv_dtype)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
+  switch (kv_dtype) {
     case ARGUS_HIP_F16: return dispatch_dim<_Float16>(ctx, p, D, a->batch, want_scores, stream);
     case ARGUS_HIP_F32: return dispatch_dim<float>(ctx, p, D, a->batch, want_scores, stream);
-    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: kv dtype %d", a->kv_dtype);
+    case kKvDesc: return dispatch_dim<DescRow>(ctx, p, D, a->batch, want_scores, stream);
+    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: kv dtype %d", kv_dtype);
   }
+}
+
+ARGUS_API int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *a) {
+  if (!ctx || !a) return ARGUS_HIP_ERR_INVALID;
+  return attention_gen_impl(ctx, a, a->kv_dtype, nullptr, 0);
+}
+
+// attention_gen over a cache whose rows are blocks of any descriptor the generic floor decodes
+// (PerBlockF16 / PerBlockF16WithMin x Nibble / Byte / Quad, block_elems a multiple of 8 up to 64 that
+// divides head_dim).  The four named 32-element formats go to the matrix-core block kernel; every
+// other one is attended by the vector-ALU kernel, each lane decoding the 8 channels of its piece from
+// the row's blocks.  Anything else is declined with ARGUS_HIP_ERR_UNSUPPORTED (nothing launched), which
+// is the caller's cue to take the floor: decode the cache with argus_hip_kv_decode_descriptor (or on
+// the CPU) and attend the F16 / F32 copy.
+ARGUS_API int argus_hip_attention_gen_desc(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *a, const argus_hip_kv_layout_desc *d) {
+  if (!ctx || !a || !d) return ARGUS_HIP_ERR_INVALID;
+  int q;
+  switch (d->packing) {
+    case 1: q = (int)d->block_elems / 2; break;
+    case 2: q = (int)d->block_elems; break;
+    case 3: q = (int)d->block_elems / 4; break;
+    default: return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_desc: declined, packing %u has no block form", d->packing);
+  }
+  if (d->scale_layout != 1 && d->scale_layout != 2)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_desc: declined, scale layout %u", d->scale_layout);
+  const bool bits_ok = (d->packing == 1 && d->bits >= 2 && d->bits <= 4) || (d->packing == 2 && d->bits == 8) || (d->packing == 3 && d->bits == 2);
+  if (!bits_ok || d->block_elems == 0 || d->block_elems > 64 || d->block_elems % 8 || (d->packing == 3 && d->scale_layout != 2))
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_desc: declined, block_elems %u bits %u", d->block_elems, (unsigned)d->bits);
+  if (a->head_dim <= 0 || a->head_dim % (int)d->block_elems)
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen_desc: declined, head_dim %d is not whole blocks of %u", a->head_dim, d->block_elems);
+  if (d->block_elems == 32) {
+    int named = -1;
+    if (d->packing == 1 && d->bits == 4) named = d->scale_layout == 1 ? ARGUS_HIP_Q4_0 : ARGUS_HIP_Q4_1;
+    else if (d->packing == 2 && d->scale_layout == 1) named = ARGUS_HIP_Q8_0;
+    else if (d->packing == 3) named = ARGUS_HIP_Q2_0;
+    if (named >= 0) {
+      const int rc = attention_gen_impl(ctx, a, named, nullptr, 0);
+      if (rc != ARGUS_HIP_ERR_UNSUPPORTED) return rc;  // shapes the block kernel refuses (wide GQA groups, unaligned rows) go on below
+    }
+  }
+  return attention_gen_impl(ctx, a, kKvDesc, d, q + (d->scale_layout == 1 ? 2 : 4));
 }

@@ -31,7 +31,47 @@ struct DecodeParams {
   int32_t slot_bound;  // slots an index list may name (the cache capacity)
   int32_t head_chunks; // vector-ALU kernel: workgroups per KV head (GQA groups wider than its head tile)
   int32_t stage_scores;  // matrix-core kernels: the chunk's logits wait in LDS and are written after the token loop
+  // Descriptor-driven rows (vector-ALU kernel only): KVLayoutDesc of the cache and its block size in bytes.
+  int32_t desc_block_elems, desc_bits, desc_scale_layout, desc_packing, desc_block_bytes;
 };
+
+// Tag type of a cache whose rows are blocks described by a KVLayoutDesc (any PerBlockF16[WithMin] x
+// Nibble / Byte / Quad descriptor, engine/src/format/dtype_layout.rs:102-166).
+struct DescRow {};
+
+// Elements w0 .. w0+7 (w0 a multiple of 8) of the block at `blk`, decoded like
+// unpack_block_via_descriptor: nibble packing keeps element i < n/2 in the low nibble of byte i and
+// element n/2 + i in the high nibble; signed with zero point 2^(bits-1) when the block has no
+// minimum, else code * scale + min; byte packing is a signed i8; quad packing holds elements
+// 4i .. 4i+3 of byte i at bit offsets 0/2/4/6.  Blocks are only 2-byte aligned.
+__device__ __forceinline__ void desc_decode8(const DecodeParams &p, const uint8_t *blk, int w0, float (&out)[8]) {
+  const float scale = (float)*(const _Float16 *)blk;
+  const bool has_min = p.desc_scale_layout == 2;
+  const float mn = has_min ? (float)*(const _Float16 *)(blk + 2) : 0.0f;
+  const uint8_t *q = blk + (has_min ? 4 : 2);
+  if (p.desc_packing == 1) {
+    const int half = p.desc_block_elems / 2, zp = 1 << (p.desc_bits - 1);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int i = w0 + e;
+      const int b = (int)q[i < half ? i : i - half];
+      const int code = i < half ? (b & 0x0f) : (b >> 4);
+      out[e] = has_min ? __fadd_rn(__fmul_rn((float)code, scale), mn) : __fmul_rn((float)(code - zp), scale);
+    }
+  } else if (p.desc_packing == 2) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = __fmul_rn((float)(int)(int8_t)q[w0 + e], scale);
+  } else {
+    const uint32_t w = (uint32_t)q[w0 / 4] | ((uint32_t)q[w0 / 4 + 1] << 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = __fadd_rn(__fmul_rn((float)((w >> (2 * e)) & 3u), scale), mn);
+  }
+}
+// Byte offset of the block that holds element `elem` (a multiple of the block size apart from the
+// position inside the block) of a cache addressed in elements.
+__device__ __forceinline__ int64_t desc_block_offset(const DecodeParams &p, int64_t elem) {
+  return elem / p.desc_block_elems * p.desc_block_bytes;
+}
 
 // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1); the argument is clamped where
 // tanh is 1 to f32 precision so exp cannot overflow.  The caller handles NaN.
@@ -57,6 +97,29 @@ __device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
       acc += u * (float)vb[slot * p.row_stride + c];
     }
     p.out[(int64_t)b * p.out_bs + (int64_t)h * D + c] = acc;
+  }
+  if (p.scores) {
+    float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
+    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = u;
+  }
+}
+
+template <>
+__device__ inline void uniform_fallback<DescRow>(const DecodeParams &p, int b, int h, int D) {
+  const int kvh = h / p.group;
+  const uint8_t *vb = (const uint8_t *)p.v;
+  const int32_t *idx = p.kv_index ? p.kv_index + (int64_t)b * p.index_bs : nullptr;
+  const float u = 1.0f / (float)p.len;
+  for (int c8 = threadIdx.x; c8 < D / 8; c8 += blockDim.x) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int t = 0; t < p.len; ++t) {
+      const int64_t slot = idx ? (int64_t)min((uint32_t)idx[t], (uint32_t)(p.slot_bound - 1)) : (p.kv_start + t);
+      const int64_t elem = (int64_t)b * p.kv_bs + (int64_t)kvh * p.head_stride + slot * p.row_stride + 8 * c8;
+      float v[8];
+      desc_decode8(p, vb + desc_block_offset(p, elem), (int)(elem % p.desc_block_elems), v);
+      for (int e = 0; e < 8; ++e) acc[e] += u * v[e];
+    }
+    for (int e = 0; e < 8; ++e) p.out[(int64_t)b * p.out_bs + (int64_t)h * D + 8 * c8 + e] = acc[e];
   }
   if (p.scores) {
     float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;

@@ -402,6 +402,18 @@ int argus_hip_kv_decode_descriptor(argus_hip_ctx *ctx, void *stream, const argus
                                    void *dst, int32_t dst_dtype, int64_t n_elems);
 int argus_hip_kv_encode_descriptor(argus_hip_ctx *ctx, void *stream, const argus_hip_kv_layout_desc *desc, const void *src,
                                    void *dst, int64_t n_elems);
+/* Backend::attention_gen over a cache whose rows are blocks of `desc`: what StandardFormat computes for
+ * an opaque --kv-format cache after decoding it whole (engine/src/kv/standard_format.rs:538-643 with
+ * engine/src/format/dtype_layout.rs:102-166), without the decoded copy.  `args` as for
+ * argus_hip_attention_gen (kv_dtype ignored; capacity, kv_start and strides in elements, whole blocks;
+ * caches 2-byte aligned).  Any PerBlockF16 / PerBlockF16WithMin x Nibble / Byte / Quad descriptor whose
+ * block_elems is a multiple of 8, at most 64 and divides head_dim is attended in-kernel: q4_0 / q4_1 /
+ * q8_0 / q2_0 on the matrix cores, every other one by the vector-ALU kernel (each lane decodes its 8
+ * channels from the row's blocks), any GQA ratio.  Every other descriptor (Dense packing, no scale,
+ * shared exponents, codebooks, ...) is DECLINED: ARGUS_HIP_ERR_UNSUPPORTED, nothing launched, and the
+ * caller takes the floor (argus_hip_kv_decode_descriptor or its CPU decode, then the F16 / F32 call). */
+int argus_hip_attention_gen_desc(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args,
+                                 const argus_hip_kv_layout_desc *desc);
 
 /* ---- (a-4) attention-score reduce for H2O / D2O --------------------------------------------- */
 /* Field-for-field twin of CudaScoreReduceArgs, crates/argus-extension-api/src/lib.rs:2909-2933;

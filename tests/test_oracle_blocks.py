@@ -56,3 +56,54 @@ def test_q4_0_unpack_matches_the_descriptor_decode_bit_for_bit():
     raw = blocks(O.DESC_Q4_0, 64, 5)
     got = O.decode_via_descriptor(O.DESC_Q4_0, raw, 64 * 32)
     assert np.array_equal(got, unpack(O.DESC_Q4_0, raw, 64 * 32).astype(np.float32))
+
+
+def unpack_any(desc, raw, n_elems):
+    """Any PerBlockF16[WithMin] x Nibble / Byte / Quad descriptor, written from the doc comments of
+    unpack_block_via_descriptor (engine/src/format/dtype_layout.rs:88-101): nibble packing keeps element
+    i < n/2 in the low nibble of byte i and element n/2 + i in the high nibble, signed around 2^(bits-1)
+    without a minimum, code*scale + min with one; byte packing is i8 * scale; quad packing puts element
+    4i + k at bits 2k of byte i."""
+    be, bits, scale_layout, packing = desc
+    bb = O.desc_block_bytes(desc)
+    blk = np.asarray(raw, np.uint8).reshape(-1, bb)
+    d = blk[:, 0:2].copy().view(np.float16).astype(np.float64)
+    has_min = scale_layout == O.SCALE_F16_MIN
+    m = blk[:, 2:4].copy().view(np.float16).astype(np.float64) if has_min else 0.0
+    codes = blk[:, 4 if has_min else 2:]
+    if packing == O.PACK_BYTE:
+        x = d * codes.view(np.int8).astype(np.float64)
+    elif packing == O.PACK_QUAD:
+        n = np.stack([(codes >> (2 * k)) & 3 for k in range(4)], axis=2).reshape(len(blk), be).astype(np.float64)
+        x = d * n + m
+    else:
+        n = np.concatenate([codes & 15, codes >> 4], axis=1).astype(np.float64)
+        x = d * n + m if has_min else d * (n - float(1 << (bits - 1)))
+    return x.reshape(-1)[:n_elems]
+
+
+@pytest.mark.parametrize("desc", [(16, 4, O.SCALE_F16, O.PACK_NIBBLE), (8, 4, O.SCALE_F16_MIN, O.PACK_NIBBLE),
+                                  (16, 3, O.SCALE_F16, O.PACK_NIBBLE), (64, 4, O.SCALE_F16_MIN, O.PACK_NIBBLE),
+                                  (64, 8, O.SCALE_F16, O.PACK_BYTE), (8, 8, O.SCALE_F16, O.PACK_BYTE),
+                                  (16, 2, O.SCALE_F16_MIN, O.PACK_QUAD), (64, 2, O.SCALE_F16_MIN, O.PACK_QUAD),
+                                  (32, 3, O.SCALE_F16_MIN, O.PACK_NIBBLE)])
+def test_descriptors_beyond_the_named_formats(desc):
+    # the decode floor and the attention composed on it, for descriptors no named format uses
+    hq, hkv, d, L, cap = 8, 2, 64, 150, 160
+    n = hkv * cap * d
+    rng = np.random.default_rng(sum(desc))
+    bb = O.desc_block_bytes(desc)
+    raw = rng.integers(0, 256, size=(n // desc[0], bb), dtype=np.uint8)
+    raw[:, 0:2] = rng.uniform(0.05, 0.3, n // desc[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    if desc[2] == O.SCALE_F16_MIN:
+        raw[:, 2:4] = rng.uniform(-1.5, 0.0, n // desc[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    raw = raw.reshape(-1)
+    want = unpack_any(desc, raw, n)
+    got = O.decode_via_descriptor(desc, raw, n)
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+    q = rng.standard_normal((hq, d)).astype(np.float32)
+    out, p = O.attention_gen_blocks(q, raw, raw, desc, hkv, L, cap, scores=True)
+    kf = want.reshape(hkv, cap, d)
+    ref_out, ref_p = T.decode_attention(q, kf, kf, hkv, L)
+    assert np.abs(out - ref_out).max() < 1e-5 * (1.0 + np.abs(ref_out).max())  # f32 sums against f64
+    assert np.allclose(p, ref_p, rtol=1e-4, atol=1e-9)
