@@ -120,6 +120,25 @@ class HipBackend {
                        size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
                        float *scores_out, size_t scores_len);
 
+  // ---- attention over an opaque --kv-format cache ----------------------------------------------
+  // What StandardFormat::attention_into does in its opaque arm (engine/src/kv/standard_format.rs:
+  // 538-643): the cache rows are blocks of the format plugin's KVLayoutDesc.  Ok(true): attended on
+  // the device without a decoded copy.  Ok(false): the descriptor is outside what the kernels decode
+  // -- the caller takes the floor (decode_via_descriptor, then attention_gen on the F32 copy), as it
+  // does for every backend today.  `capacity`: rows per KV head of the HeadMajor cache.
+  Result<bool> attention_gen_opaque(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out, const argus_hip_kv_layout_desc &desc,
+                                    size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len, size_t capacity) {
+    if (!q.device || !k_cache.device || !v_cache.device || !out.device) return Result<bool>::Ok(false);
+    argus_hip_attention_gen_args a{};
+    a.q = (const float *)q.ptr; a.k_cache = k_cache.ptr; a.v_cache = v_cache.ptr; a.out = (float *)out.ptr;
+    a.num_heads_q = (int32_t)num_heads_q; a.num_heads_kv = (int32_t)num_heads_kv; a.head_dim = (int32_t)head_dim;
+    a.cache_seq_len = (int32_t)cache_seq_len; a.capacity = (int32_t)capacity; a.layout = ARGUS_HIP_HEAD_MAJOR; a.batch = 1;
+    const int rc = argus_hip_attention_gen_desc(ctx_, &a, &desc);
+    if (rc == ARGUS_HIP_ERR_UNSUPPORTED) return Result<bool>::Ok(false);
+    if (rc != ARGUS_HIP_OK) return Result<bool>::Err("attention_gen_desc failed: " + last_error());
+    return Result<bool>::Ok(true);
+  }
+
   // ---- Backend::flash_attention_prefill (engine/src/backend.rs:1011-1027) --------------------
   // Ok(true) = dispatched, Ok(false) = not handled, caller uses its CPU path.
   Result<bool> flash_attention_prefill(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,

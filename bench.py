@@ -531,6 +531,9 @@ def main():
         add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
             bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=8),
             "scores emitted; 8 KV and score buffer sets rotated (537 MB of attended rows)")
+        add("cfg5_gemma2_L2048_cap4096_b64_scores_softcap50",
+            bench_decode(ctx, 8, 4, 256, 2048, 64, es, ew, capacity=4096, scores=True, softcap=50.0),
+            "the same shape with 64 sequences per call (542 MB): the kernel's rate once the call is not latency-bound")
         add("cfg4_kivi_q4_L8192_res128_f32", bench_kivi(ctx, 4, es, ew), "8 block sets rotated; single launch, 11.4 MB")
         add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")
         add("cfg4_kivi_q4_L8192_res128_f16", bench_kivi(ctx, 4, es, ew, res_f16=True), "F16 residual window")

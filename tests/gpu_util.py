@@ -14,6 +14,27 @@ def ctx():
     return _ctx
 
 
+_env_ctx = {}
+
+
+def env_ctx(name, value):
+    """A context created under the environment switch `name=value` (switches are read at creation)."""
+    key = (name, value)
+    if key not in _env_ctx:
+        import os
+        import argus_hip
+        old = os.environ.get(name)
+        os.environ[name] = value
+        try:
+            _env_ctx[key] = argus_hip.Context(0)
+        finally:
+            if old is None:
+                del os.environ[name]
+            else:
+                os.environ[name] = old
+    return _env_ctx[key]
+
+
 _direct_ctx = None
 
 
