@@ -351,7 +351,7 @@ def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
 # scaled by what the same counters read for a plain 1 GiB copy (x2.000 and x1.000).  Counters cannot
 # be read from inside this process, so the figure is the one of the profile run named beside it in
 # the output (`traffic_source`), not a measurement of this run.
-DECODE_TRAFFIC_BYTES = 2_153_496_471
+DECODE_TRAFFIC_BYTES = 2_161_544_418
 DECODE_TRAFFIC_SOURCE = "profiles/decode_mfma_cfg3_L32768_b16_hbm_traffic.md"
 
 
@@ -426,7 +426,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
                     choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1",
-                             "q8_0", "copy_calib", "aux", "layers"],
+                             "q8_0", "copy_calib", "aux", "layers", "primary_scores", "cfg5_b64"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -456,6 +456,10 @@ def main():
             res = bench_aux(ctx, args.steps, args.warmup)
         elif w == "layers":
             res = bench_layer_loop(ctx, args.steps, args.warmup)
+        elif w == "primary_scores":
+            res = bench_decode(ctx, 32, 8, 128, 32768, 16, args.steps, args.warmup, scores=True)
+        elif w == "cfg5_b64":
+            res = bench_decode(ctx, 8, 4, 256, 2048, 64, args.steps, args.warmup, capacity=4096, scores=True, softcap=50.0)
         elif w == "decode_b1":
             res = bench_decode(ctx, 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=4)
         elif w == "prefill":
