@@ -53,7 +53,7 @@ def test_reference_matrix(nq, nkv, layout, window):
 @pytest.mark.parametrize("k_f16", [False, True])
 @pytest.mark.parametrize("nq,nkv,d,seq_len,prefix,q_start,q_window,window",
                          [(32, 8, 128, 64, 1024, 960, 32, None), (8, 4, 256, 40, 300, 260, 64, 128),
-                          (14, 2, 64, 128, 128, 0, 16, None)])
+                          (14, 2, 64, 128, 128, 0, 16, None), (16, 2, 128, 48, 333, 285, 32, None)])
 def test_model_shapes_head_major(k_f16, nq, nkv, d, seq_len, prefix, q_start, q_window, window):
     # HeadMajor cache [kv_heads, capacity, d], chunked prefill (q_start_pos > 0), accumulation into a
     # non-zero sum buffer, F16 K compared with the oracle fed the f16-rounded K.
@@ -73,6 +73,30 @@ def test_model_shapes_head_major(k_f16, nq, nkv, d, seq_len, prefix, q_start, q_
     close(got_s, ref_s)
     close(got_m, ref_m)
     assert np.abs((got_s - init).sum(1) - qw).max() < 1e-3  # each row adds a distribution
+
+
+@pytest.mark.parametrize("k_f16", [False, True])
+def test_seq_major_per_head_rows_sum_to_sum_out(k_f16):
+    # SeqMajor cache [capacity, kv_heads, d] (key stride = kv_heads * d) on the matrix-core logits path,
+    # per-head per-row layout: adding a head's rows in order reproduces sum_out bit for bit.
+    nq, nkv, d, seq_len, prefix, q_start, q_window = 12, 4, 128, 40, 700, 660, 24
+    cap = prefix + 5
+    rng = np.random.default_rng(77)
+    q = rng.standard_normal((seq_len, nq, d)).astype(np.float32)
+    k = rng.standard_normal((cap, nkv, d)).astype(np.float32)
+    k_ref = k.astype(np.float16).astype(np.float32) if k_f16 else k
+    ref_s = np.zeros((nq, prefix), np.float32)
+    ref_r = np.zeros((q_window, nq, prefix), np.float32)
+    O.prefill_attention_scores(q, k_ref.reshape(-1), nq, nkv, d, seq_len, prefix, nkv * d, d, q_start, q_window, None,
+                               sum_out=ref_s, per_row=ref_r, per_head=True)
+    got_s, got_r = run_dev(q, k.reshape(-1), nq, nkv, d, seq_len, prefix, nkv * d, d, q_start, q_window, None, True,
+                           (q_window, nq, prefix), True, k_f16=k_f16)
+    close(got_s, ref_s)
+    close(got_r, ref_r)
+    acc = np.zeros((nq, prefix), np.float32)
+    for step in range(q_window):
+        acc = acc + got_r[step]
+    assert (acc.view(np.uint32) == got_s.view(np.uint32)).all()
 
 
 def test_nothing_armed_and_errors():
