@@ -28,6 +28,13 @@ int oracle_decode_via_descriptor(int block_elems, int bits, int scale_layout, in
                                  int64_t n_elems);
 int oracle_encode_via_descriptor(int block_elems, int bits, int scale_layout, int packing, const float *src, uint8_t *dst,
                                  int64_t n_elems);
+int oracle_kivi_build(const float *k_in, const float *v_in, int n_tokens, int kv_heads, int head_dim, int res_cap, int bits, uint8_t *qk,
+                      uint8_t *qv, float *res_k, float *res_v, int *q_tokens_out, int *res_tokens_out);
+int oracle_kivi_assemble_view(const uint8_t *qk, const uint8_t *qv, const float *res_k, const float *res_v, int q_tokens, int res_tokens,
+                              int kv_heads, int head_dim, int res_cap, int bits, float *attn_k, float *attn_v);
+int oracle_kivi_attention(const float *q, const uint8_t *qk, const uint8_t *qv, const float *res_k, const float *res_v, float *out,
+                          float *scores, int64_t score_stride, int num_heads_q, int num_heads_kv, int head_dim, int q_tokens, int res_tokens,
+                          int res_cap, float scale, int bits);
 void oracle_kv_scatter(const float *k_src, const float *v_src, void *k_dst, void *v_dst, int kv_heads, int head_dim,
                        int capacity, int write_pos_start, int seq_len, int dst_f16);
 }
@@ -309,6 +316,111 @@ static void test_quant_attn(HipBackend &be) {
   printf("[kivi] degraded handle, gather_update, residual-only attention + host score read-back ok\n");
 }
 
+// The KIVI container in GPU mode, driven the way the layer loop drives it: a multi-token prefill
+// update that crosses a flush, then one token per step; at checkpoints the device blocks must be
+// the CPU container's bit for bit, the fused attention and its host scores must match the oracle's
+// attention over that container, and the F16 view must be the dequantised cache.
+static float f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000) << 16, exp = (h >> 10) & 31, man = h & 1023;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) bits = sign;
+    else {
+      int e = -1;
+      uint32_t m = man;
+      do { ++e; m <<= 1; } while (!(m & 1024));
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((m & 1023) << 13);
+    }
+  } else if (exp == 31) bits = sign | 0x7f800000u | (man << 13);
+  else bits = sign | ((exp + 112) << 23) | (man << 13);
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+static void test_quant_window_cache(HipBackend &be) {
+  const size_t hq = 8, hkv = 2, hd = 128, res_cap = 64, max_seq = 320, total = 3 * res_cap + 37;
+  std::vector<float> k(total * hkv * hd), v(k.size()), q(hq * hd);
+  oracle_gen_data(k.data(), k.size(), 501); oracle_gen_data(v.data(), v.size(), 502); oracle_gen_data(q.data(), q.size(), 503);
+  for (size_t t = 0; t < total; ++t) k[(t * hkv + 1) * hd + 7] *= 12.0f;  // an outlier channel
+  DevBuf dk(&be, k.size() * 4, k.data()), dv(&be, v.size() * 4, v.data()), dq(&be, q.size() * 4, q.data()), dout(&be, q.size() * 4);
+  CHECK(!HipQuantWindowCache::new_gpu(&be, hkv, hd, max_seq, 48, 4).ok(), "residual_size must be a multiple of 32");
+  CHECK(!HipQuantWindowCache::new_gpu(&be, hkv, hd, max_seq, res_cap, 3).ok(), "bits 3 refused");
+  for (int bits : {2, 4, 8}) {
+    auto made = HipQuantWindowCache::new_gpu(&be, hkv, hd, max_seq, res_cap, (uint8_t)bits);
+    CHECK(made.ok(), "new_gpu bits %d: %s", bits, made.error().c_str());
+    if (!made.ok()) return;
+    HipQuantWindowCache &c = *made.value();
+    const size_t bb = 4 + 32 * bits / 8;
+    auto tokens = [&](void *base, size_t first, size_t n) {
+      return Tensor{(char *)base + first * hkv * hd * 4, DType::F32, {1, n, hkv, hd}, true};
+    };
+    auto check_at = [&](size_t n) {
+      CHECK(c.current_pos() == n, "current_pos %zu != %zu", c.current_pos(), n);
+      const size_t max_blocks = (n / res_cap + 1) * hkv * res_cap * hd / 32;
+      std::vector<uint8_t> rqk(max_blocks * bb, 0), rqv(max_blocks * bb, 0);
+      std::vector<float> rrk(hkv * res_cap * hd, 0.0f), rrv(rrk.size(), 0.0f);
+      int qt = 0, rt = 0;
+      CHECK(oracle_kivi_build(k.data(), v.data(), (int)n, hkv, hd, res_cap, bits, rqk.data(), rqv.data(), rrk.data(), rrv.data(), &qt, &rt) == 0, "oracle build");
+      const QuantWindowRawBuffers raw = c.get_raw_gpu_buffers();
+      CHECK(raw.q_tokens == (size_t)qt && raw.res_tokens == (size_t)rt && raw.bits == bits, "q_tokens %zu/%d res_tokens %zu/%d", raw.q_tokens, qt, raw.res_tokens, rt);
+      const size_t used = (size_t)qt * hkv * hd / 32 * bb;
+      std::vector<uint8_t> gk(used), gv(used);
+      if (used) {
+        be.read_buffer(gk.data(), raw.qk_buf, used);
+        be.read_buffer(gv.data(), raw.qv_buf, used);
+        CHECK(memcmp(gk.data(), rqk.data(), used) == 0, "bits %d n %zu: key blocks differ from the CPU container", bits, n);
+        CHECK(memcmp(gv.data(), rqv.data(), used) == 0, "bits %d n %zu: value blocks differ from the CPU container", bits, n);
+      }
+      std::vector<float> grk(rrk.size());
+      be.read_buffer(grk.data(), raw.res_k, grk.size() * 4);
+      bool same = true;
+      for (size_t h = 0; h < hkv; ++h)
+        for (size_t i = 0; i < (size_t)rt * hd; ++i) same = same && grk[h * res_cap * hd + i] == rrk[h * res_cap * hd + i];
+      CHECK(same, "bits %d n %zu: residual ring differs", bits, n);
+      // fused attention + host scores
+      std::vector<float> ref(hq * hd), ref_sc(hq * n), got(hq * hd), sc(hq * n, -1.0f);
+      const float scale = 1.0f / sqrtf((float)hd);
+      oracle_kivi_attention(q.data(), rqk.data(), rqv.data(), rrk.data(), rrv.data(), ref.data(), ref_sc.data(), (int64_t)n, hq, hkv, hd, qt, rt, res_cap, scale, bits);
+      Tensor tq{dq.p, DType::F32, {hq, hd}, true}, tout{dout.p, DType::F32, {hq, hd}, true};
+      auto st = c.attention_native(tq, tout, hq, sc.data(), sc.size());
+      CHECK(st.ok(), "attention_native: %s", st.error().c_str());
+      be.read_buffer(got.data(), dout.p, got.size() * 4);
+      CHECK(max_abs_diff(got, ref) < 2e-3f, "bits %d n %zu: attention out diff %g", bits, n, max_abs_diff(got, ref));
+      float worst = 0;
+      for (size_t i = 0; i < sc.size(); ++i) worst = fmaxf(worst, fabsf(sc[i] - ref_sc[i]) / fmaxf(ref_sc[i], 1e-30f));
+      CHECK(worst < 1e-4f, "bits %d n %zu: scores rel diff %g", bits, n, worst);
+      // F16 view = dequantised blocks + residual rows
+      std::vector<float> vk(n * hkv * hd), vv(vk.size());
+      oracle_kivi_assemble_view(rqk.data(), rqv.data(), rrk.data(), rrv.data(), qt, rt, hkv, hd, res_cap, bits, vk.data(), vv.data());
+      auto view = c.get_view_gpu();
+      CHECK(view.ok(), "get_view_gpu: %s", view.error().c_str());
+      if (!view.ok()) return;
+      std::vector<uint16_t> hk(vk.size()), hv(vk.size());
+      be.read_buffer(hk.data(), view.value().first.ptr, hk.size() * 2);
+      be.read_buffer(hv.data(), view.value().second.ptr, hv.size() * 2);
+      float wk = 0, wv = 0;
+      for (size_t i = 0; i < vk.size(); ++i) {
+        wk = fmaxf(wk, fabsf(f16_bits_to_f32(hk[i]) - vk[i]) / (1.0f + fabsf(vk[i])));
+        wv = fmaxf(wv, fabsf(f16_bits_to_f32(hv[i]) - vv[i]) / (1.0f + fabsf(vv[i])));
+      }
+      CHECK(wk < 1e-3f && wv < 1e-3f, "bits %d n %zu: F16 view differs (%g, %g)", bits, n, wk, wv);
+    };
+    // prefill of 100 tokens: fills the ring, flushes 64, leaves 36
+    CHECK(c.update(tokens(dk.p, 0, 100), tokens(dv.p, 0, 100)).ok(), "prefill update");
+    check_at(100);
+    for (size_t t = 100; t < total; ++t) {
+      auto st = c.update(tokens(dk.p, t, 1), tokens(dv.p, t, 1));
+      CHECK(st.ok(), "update token %zu: %s", t, st.error().c_str());
+      if (t + 1 == 128 || t + 1 == 129 || t + 1 == 3 * res_cap) check_at(t + 1);
+    }
+    check_at(total);
+    CHECK(!c.update(tokens(dk.p, 0, max_seq), tokens(dv.p, 0, max_seq)).ok(), "overflow refused");
+    c.reset();
+    CHECK(c.current_pos() == 0, "reset");
+  }
+  printf("[kivi] quant-window container on the device: update / flush / raw buffers / fused attention / F16 view ok (bits 2, 4, 8)\n");
+}
+
 // A committed keep-list on a device cache: compaction through overlapping buffer_shift runs must
 // equal the gather cache[:, keep] (engine/src/kv/naive_reference.rs), per layer and per head; then
 // write_buffer_range into the freed tail.
@@ -374,6 +486,7 @@ int main() {
   test_accumulator_binding(be);
   test_prefill_and_scatter(be);
   test_quant_attn(be);
+  test_quant_window_cache(be);
   test_compaction_and_memory(be);
   if (g_fail) {
     printf("%d check(s) FAILED\n", g_fail);
