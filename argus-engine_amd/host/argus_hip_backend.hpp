@@ -120,7 +120,52 @@ class HipBackend {
   // export instead of failing (cuda_pc.rs:1776-1779).
   Status attention_gen(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,
                        size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
-                       float *scores_out, size_t scores_len);
+                       float *scores_out, size_t scores_len) {
+    return attention_gen_indexed(q, k_cache, v_cache, out, num_heads_q, num_heads_kv, head_dim, cache_seq_len, nullptr, scores_out, scores_len);
+  }
+
+  // ---- SelectiveRead::attention_into_selected (engine/src/kv/standard_format.rs:2043-2184) ------
+  // Attention over the selected cache positions only, the softmax normalised over that subset.
+  // `page_size` 0 = ReadGranularity::Token (select holds positions), else ::Page (select holds page
+  // indices, expanded by page_indices_to_positions, standard_format.rs:1924-1938, clamped to
+  // current_pos).  An empty cache or selection zeroes `out`.  The reference gathers the rows on the
+  // host (for a device cache: snapshot, CPU attention, upload); here the positions go to the device
+  // as an index list and the decode kernel reads the rows in place.  scores_out[h * stride + i] is
+  // the weight of the i-th selected position.
+  Status attention_into_selected(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out, size_t num_heads_q,
+                                 size_t num_heads_kv, size_t head_dim, size_t current_pos, const std::vector<size_t> &select,
+                                 size_t page_size, float *scores_out, size_t scores_len) {
+    std::vector<int32_t> positions;
+    if (current_pos != 0) {
+      if (page_size == 0) {
+        positions.assign(select.begin(), select.end());
+      } else {
+        for (size_t pi : select)
+          for (size_t pos = pi * page_size, end = std::min(pi * page_size + page_size, current_pos); pos < end; ++pos) positions.push_back((int32_t)pos);
+      }
+    }
+    if (positions.empty()) {
+      const std::vector<float> zeros(num_heads_q * head_dim, 0.0f);
+      return write_buffer(out.ptr, zeros.data(), zeros.size() * sizeof(float));
+    }
+    const std::vector<size_t> &kd = k_cache.dims;
+    const bool head_major = kd.size() >= 3 && kd[1] == num_heads_kv && kd[1] != kd[2];
+    const size_t slots = kd.size() >= 3 ? (head_major ? kd[2] : kd[1]) : 0;
+    for (int32_t pos : positions)
+      if (pos < 0 || (size_t)pos >= slots) return Status::Err("attention_into_selected: position " + std::to_string(pos) + " outside the cache (" + std::to_string(slots) + " slots)");
+    const size_t need = positions.size() * sizeof(int32_t);
+    if (need > index_tmp_bytes_) {
+      if (index_tmp_) argus_hip_free(ctx_, index_tmp_);
+      index_tmp_ = nullptr;
+      index_tmp_bytes_ = 0;
+      if (argus_hip_malloc(ctx_, need, &index_tmp_) != ARGUS_HIP_OK) return Status::Err("index list: " + last_error());
+      index_tmp_bytes_ = need;
+    }
+    Status st = write_buffer(index_tmp_, positions.data(), need);
+    if (!st.ok()) return st;
+    return attention_gen_indexed(q, k_cache, v_cache, out, num_heads_q, num_heads_kv, head_dim, positions.size(), (const int32_t *)index_tmp_, scores_out,
+                                 scores_len);
+  }
 
   // ---- attention over an opaque --kv-format cache ----------------------------------------------
   // What StandardFormat::attention_into does in its opaque arm (engine/src/kv/standard_format.rs:
@@ -205,8 +250,12 @@ class HipBackend {
  private:
   explicit HipBackend(argus_hip_ctx *ctx) : ctx_(ctx) {}
   argus_hip_ctx *ctx_;
+  Status attention_gen_indexed(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out, size_t num_heads_q, size_t num_heads_kv,
+                               size_t head_dim, size_t cache_seq_len, const int32_t *kv_index_dev, float *scores_out, size_t scores_len);
   void *score_tmp_ = nullptr;  // reusable device score scratch (cuda_pc.rs `score_tmp_buf`)
   size_t score_tmp_bytes_ = 0;
+  void *index_tmp_ = nullptr;  // reusable device index list of attention_into_selected
+  size_t index_tmp_bytes_ = 0;
   std::unique_ptr<HipGpuScoreAccumulator> acc_;
 };
 
@@ -593,6 +642,7 @@ class HipGpuScoreAccumulator {
 inline HipBackend::~HipBackend() {
   acc_.reset();
   if (score_tmp_) argus_hip_free(ctx_, score_tmp_);
+  if (index_tmp_) argus_hip_free(ctx_, index_tmp_);
   argus_hip_destroy(ctx_);
 }
 
@@ -603,9 +653,9 @@ inline Status HipBackend::init_gpu_score_acc(size_t n_layers, size_t n_heads_q, 
   return OkStatus();
 }
 
-inline Status HipBackend::attention_gen(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,
-                                        size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
-                                        float *scores_out, size_t scores_len) {
+inline Status HipBackend::attention_gen_indexed(const Tensor &q, const Tensor &k_cache, const Tensor &v_cache, Tensor &out,
+                                                size_t num_heads_q, size_t num_heads_kv, size_t head_dim, size_t cache_seq_len,
+                                                const int32_t *kv_index_dev, float *scores_out, size_t scores_len) {
   // The reference falls back to its CPU companion for non-device buffers and Q4_0 KV
   // (cuda_pc.rs:1716-1729); this mirror has no CPU companion, so it reports the former.  Q4_0
   // caches are attended on the device (BlockQ4_0 rows, common.rs:676-850).
@@ -618,10 +668,11 @@ inline Status HipBackend::attention_gen(const Tensor &q, const Tensor &k_cache, 
   a.q = (const float *)q.ptr; a.k_cache = k_cache.ptr; a.v_cache = v_cache.ptr; a.out = (float *)out.ptr;
   a.num_heads_q = (int32_t)num_heads_q; a.num_heads_kv = (int32_t)num_heads_kv; a.head_dim = (int32_t)head_dim;
   a.cache_seq_len = (int32_t)cache_seq_len;
-  a.capacity = head_major ? (int32_t)kd[2] : 0;
+  a.capacity = head_major ? (int32_t)kd[2] : (kv_index_dev && kd.size() >= 3 ? (int32_t)kd[1] : 0);
   a.layout = head_major ? ARGUS_HIP_HEAD_MAJOR : ARGUS_HIP_SEQ_MAJOR;
   a.kv_dtype = (int32_t)k_cache.dtype;
   a.batch = 1;
+  a.kv_index = kv_index_dev;
 
   size_t stride = 0;
   bool copy_back = false;

@@ -141,6 +141,35 @@ static void test_attention_gen(HipBackend &be) {
     std::vector<float> small(hq * 4, -7.0f);
     CHECK(be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, small.data(), small.size()).ok(), "malformed slice");
     for (float x : small) CHECK(x == -7.0f, "malformed slice untouched");
+    // SelectiveRead (standard_format.rs:2043-2184): a token selection, the same as pages, an empty one
+    {
+      const std::vector<size_t> sel = {0, 1, 2, 3, 6, 9, 10, 11, (size_t)len - 2, (size_t)len - 1};
+      std::vector<int32_t> idx(sel.begin(), sel.end());
+      std::vector<float> ssc(hq * sel.size(), -7.0f), sref(hq * d), sref_sc(hq * sel.size(), -7.0f);
+      CHECK(be.attention_into_selected(tq, tk, tv, tout, hq, hkv, d, len, sel, 0, ssc.data(), ssc.size()).ok(), "attention_into_selected");
+      be.read_buffer(got.data(), dout.p, got.size() * 4);
+      oracle_attention_gen_scalar(q.data(), kp, vp, sref.data(), hq, hkv, d, (int)sel.size(), cap, 1, f16, sref_sc.data(), (int64_t)sel.size(), 0.0f, idx.data());
+      CHECK(max_abs_diff(got, sref) < (f16 ? 1e-3f : 1e-4f), "selected out diff %g", max_abs_diff(got, sref));
+      CHECK(max_abs_diff(ssc, sref_sc) < 1e-5f, "selected scores diff %g", max_abs_diff(ssc, sref_sc));
+      // pages of 4: page 0 = positions 0..3, the last page clamped to current_pos
+      const std::vector<size_t> pages = {0, (size_t)(len - 1) / 4};
+      std::vector<int32_t> pidx = {0, 1, 2, 3};
+      for (int pos = (len - 1) / 4 * 4; pos < len; ++pos) pidx.push_back(pos);
+      CHECK(be.attention_into_selected(tq, tk, tv, tout, hq, hkv, d, len, pages, 4, nullptr, 0).ok(), "attention_into_selected pages");
+      be.read_buffer(got.data(), dout.p, got.size() * 4);
+      oracle_attention_gen_scalar(q.data(), kp, vp, sref.data(), hq, hkv, d, (int)pidx.size(), cap, 1, f16, nullptr, 0, 0.0f, pidx.data());
+      CHECK(max_abs_diff(got, sref) < (f16 ? 1e-3f : 1e-4f), "paged out diff %g", max_abs_diff(got, sref));
+      // select = every position: the full read
+      std::vector<size_t> all(len);
+      for (int t = 0; t < len; ++t) all[t] = t;
+      CHECK(be.attention_into_selected(tq, tk, tv, tout, hq, hkv, d, len, all, 0, nullptr, 0).ok(), "select all");
+      be.read_buffer(got.data(), dout.p, got.size() * 4);
+      CHECK(max_abs_diff(got, ref) < (f16 ? 1e-3f : 1e-4f), "select-all equals the full read (%g)", max_abs_diff(got, ref));
+      CHECK(be.attention_into_selected(tq, tk, tv, tout, hq, hkv, d, len, {}, 0, nullptr, 0).ok(), "empty selection");
+      be.read_buffer(got.data(), dout.p, got.size() * 4);
+      for (float x : got) CHECK(x == 0.0f, "empty selection zeroes out");
+      CHECK(!be.attention_into_selected(tq, tk, tv, tout, hq, hkv, d, len, {(size_t)cap + 3}, 0, nullptr, 0).ok(), "position outside the cache refused");
+    }
     // SeqMajor-shaped tensor ([len, hkv, d]) is detected from the shape
     Tensor host_q = tq;
     host_q.device = false;
@@ -168,7 +197,7 @@ static void test_attention_gen(HipBackend &be) {
     for (size_t i = 0; i < sc.size(); ++i) worst = fmaxf(worst, fabsf(sc[i] - ref_sc[i]) / ref_sc[i]);
     CHECK(worst < 1e-4f, "q4_0 scores rel diff %g", worst);
   }
-  printf("[attention_gen] unit shape f32/f16/q4_0 + host score slice ok\n");
+  printf("[attention_gen] unit shape f32/f16/q4_0 + host score slice + selective read (tokens, pages, all, none) ok\n");
 }
 
 static void test_accumulator_binding(HipBackend &be) {
