@@ -594,6 +594,33 @@ class HipGpuScoreAccumulator {
     return OkStatus();
   }
 
+  // seed_prefill_importance[_dual] (engine/src/inference/attention_scores.rs:249-322) without the
+  // host fold: `pfa_dev` holds the per-layer column sums of prefill_attention_scores on the device,
+  // [n_layers, n_heads_q, prefix_len] F32, and one synthetic step folds them into the cumulative
+  // buffers exactly as the reference's accumulate_layer_gqa + end_step does on the host
+  // (importance += layer-MAX of the head sums, head_importance += GQA average), with the PFA layout's
+  // stride = cache_seq_len = prefix_len.  The reference folds on the CPU and uploads the result
+  // through seed_cumulative, because its PFA runs on the host.
+  Status seed_prefill_importance_device(void *stream, const void *pfa_dev, size_t prefix_len) {
+    if (!active_ || prefix_len == 0 || n_heads_q_ == 0) return OkStatus();
+    if (prefix_len > max_seq_len_) return Status::Err("seed_prefill_importance: prefix_len exceeds max_seq_len");
+    argus_hip_score_reduce_args a{};
+    a.stream = stream;
+    a.score_buf = (uint64_t)pfa_dev; a.importance = (uint64_t)importance_; a.head_importance = (uint64_t)head_importance_;
+    a.decay_factor = decay_factor_; a.n_layers = n_layers_; a.n_heads_q = n_heads_q_; a.n_kv_heads = n_kv_heads_;
+    a.cache_seq_len = prefix_len; a.score_stride = prefix_len; a.max_seq_len = max_seq_len_;
+    a.layer_flat_importance = (uint64_t)layer_flat_;
+    HipScoreReduceBackend reducer(be_->ctx());
+    int ret = reducer.reduce(a);
+    if (ret != 0) return Status::Err("attn_score HIP prefill seed failed: code " + std::to_string(ret));
+    if (per_layer_flat_) {
+      ret = reducer.reduce_per_layer(a);
+      if (ret != 0) return Status::Err("attn_score HIP per-layer prefill seed failed: code " + std::to_string(ret));
+    }
+    steps_ += 1;
+    return OkStatus();
+  }
+
   Result<std::pair<std::vector<float>, std::vector<float>>> sync_to_cpu() const {
     using R = Result<std::pair<std::vector<float>, std::vector<float>>>;
     std::vector<float> flat(max_seq_len_), head(n_kv_heads_ * max_seq_len_);

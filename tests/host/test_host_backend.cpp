@@ -35,6 +35,9 @@ int oracle_kivi_assemble_view(const uint8_t *qk, const uint8_t *qv, const float 
 int oracle_kivi_attention(const float *q, const uint8_t *qk, const uint8_t *qv, const float *res_k, const float *res_v, float *out,
                           float *scores, int64_t score_stride, int num_heads_q, int num_heads_kv, int head_dim, int q_tokens, int res_tokens,
                           int res_cap, float scale, int bits);
+int oracle_prefill_attention_scores(const float *q, const float *k, int n_heads_q, int n_heads_kv, int head_dim, int seq_len, int cache_seq_len,
+                                    int64_t k_pos_stride, int64_t kv_head_stride, int q_start_pos, int q_window, int window, float *sum_out,
+                                    float *per_row_out, int per_row_per_head);
 void oracle_kv_scatter(const float *k_src, const float *v_src, void *k_dst, void *v_dst, int kv_heads, int head_dim,
                        int capacity, int write_pos_start, int seq_len, int dst_f16);
 }
@@ -345,6 +348,46 @@ static void test_quant_attn(HipBackend &be) {
   printf("[kivi] degraded handle, gather_update, residual-only attention + host score read-back ok\n");
 }
 
+// Faithful-H2O seed on the device: the PFA column sums of every layer are produced on the device
+// into one [n_layers, n_heads_q, prefix] buffer and folded into the cumulative importance by one
+// synthetic reduce step (attention_scores.rs:249-276), with no host round trip.  Expected values:
+// the oracle's PFA per layer folded by the oracle's reduce.
+static void test_prefill_seed(HipBackend &be) {
+  const size_t n_layers = 3, hq = 8, hkv = 2, hd = 64, prefix = 96, seq = 40, qwin = 16, max_seq = 128;
+  CHECK(be.init_gpu_score_acc(n_layers, hq, hkv, max_seq, 0.0f).ok(), "init");
+  be.gpu_score_acc()->set_active(true);
+  std::vector<float> ref_pfa(n_layers * hq * prefix, 0.0f);
+  DevBuf dpfa(&be, ref_pfa.size() * 4, ref_pfa.data());  // zeroed: the side channel accumulates
+  for (size_t l = 0; l < n_layers; ++l) {
+    std::vector<float> q(seq * hq * hd), k(hkv * prefix * hd);
+    oracle_gen_data(q.data(), q.size(), 700 + l); oracle_gen_data(k.data(), k.size(), 800 + l);
+    DevBuf dq(&be, q.size() * 4, q.data()), dk(&be, k.size() * 4, k.data());
+    Tensor tq{dq.p, DType::F32, {seq, hq, hd}, true}, tk{dk.p, DType::F32, {1, hkv, prefix, hd}, true};
+    // HeadMajor K: key stride hd, head stride prefix * hd; chunked prefill: q_start_pos = prefix - seq
+    CHECK(be.prefill_attention_scores(tq, tk, hq, hkv, hd, seq, prefix, hd, prefix * hd, prefix - seq, qwin, false, 0,
+                                      (float *)dpfa.p + l * hq * prefix, nullptr, false).ok(), "pfa layer %zu", l);
+    oracle_prefill_attention_scores(q.data(), k.data(), hq, hkv, hd, seq, prefix, hd, prefix * hd, prefix - seq, qwin, -1,
+                                    ref_pfa.data() + l * hq * prefix, nullptr, 0);
+  }
+  CHECK(be.gpu_score_acc()->seed_prefill_importance_device(nullptr, dpfa.p, prefix).ok(), "seed");
+  std::vector<float> imp(max_seq, 0.0f), himp(hkv * max_seq, 0.0f);
+  oracle_score_fused_reduce(ref_pfa.data(), imp.data(), himp.data(), 1.0f, n_layers, hq, hkv, prefix, prefix, max_seq);
+  auto got = be.gpu_score_acc()->sync_to_cpu();
+  CHECK(got.ok(), "sync");
+  float worst = 0, total = 0;
+  for (size_t t = 0; t < prefix; ++t) {
+    worst = fmaxf(worst, fabsf(got.value().first[t] - imp[t]) / fmaxf(imp[t], 1e-30f));
+    total += got.value().first[t];
+  }
+  for (size_t i = 0; i < himp.size(); ++i)
+    if (i % max_seq < prefix) worst = fmaxf(worst, fabsf(got.value().second[i] - himp[i]) / fmaxf(himp[i], 1e-30f));
+  CHECK(worst < 1e-4f, "seeded importance rel diff %g", worst);
+  for (size_t t = prefix; t < max_seq; ++t) CHECK(got.value().first[t] == 0.0f, "positions past the prefix untouched");
+  CHECK(total > 0.0f, "seed is not empty");
+  CHECK(be.gpu_score_acc()->steps_accumulated() == 1, "one synthetic step");
+  printf("[score] PFA on the device -> one-step prefill seed of the cumulative importance ok (rel %.3g)\n", worst);
+}
+
 // The KIVI container in GPU mode, driven the way the layer loop drives it: a multi-token prefill
 // update that crosses a flush, then one token per step; at checkpoints the device blocks must be
 // the CPU container's bit for bit, the fused attention and its host scores must match the oracle's
@@ -514,6 +557,7 @@ int main() {
   test_attention_gen(be);
   test_accumulator_binding(be);
   test_prefill_and_scatter(be);
+  test_prefill_seed(be);
   test_quant_attn(be);
   test_quant_window_cache(be);
   test_compaction_and_memory(be);
