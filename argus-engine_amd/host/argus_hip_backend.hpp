@@ -641,6 +641,17 @@ class HipGpuScoreAccumulator {
     if (!s.ok()) return s;
     return be_->write_buffer(head_importance_, head.data(), head.size() * 4);
   }
+  // gpu_score.rs:340-363
+  Status seed_layer_flat_cumulative(const std::vector<float> &layer_flat) {
+    if (layer_flat.size() != n_layers_ * max_seq_len_)
+      return Status::Err("seed_layer_flat_cumulative: layer_flat.len()=" + std::to_string(layer_flat.size()) + " != n_layers*max_seq_len=" +
+                         std::to_string(n_layers_ * max_seq_len_));
+    return be_->write_buffer(layer_flat_, layer_flat.data(), layer_flat.size() * 4);
+  }
+  Status reset_layer_flat() {
+    const std::vector<float> z(n_layers_ * max_seq_len_, 0.0f);
+    return be_->write_buffer(layer_flat_, z.data(), z.size() * 4);
+  }
   Status reset() {
     std::vector<float> z(n_layers_ * max_seq_len_ > n_kv_heads_ * max_seq_len_ ? n_layers_ * max_seq_len_ : n_kv_heads_ * max_seq_len_, 0.0f);
     Status s = be_->write_buffer(importance_, z.data(), max_seq_len_ * 4);

@@ -110,6 +110,16 @@ static void test_score_accumulator(HipBackend &be) {
   auto r3 = be.gpu_score_acc()->sync_to_cpu();
   CHECK(r3.value().first == sf && r3.value().second == sh, "case3 seed round trip");
   CHECK(!be.gpu_score_acc()->seed_cumulative(std::vector<float>(3), sh).ok(), "seed length check");
+  // per-layer flat cumulative: seed, read back, clear alone (gpu_score.rs:329-363)
+  std::vector<float> lf(n_layers * max_seq);
+  for (size_t i = 0; i < lf.size(); ++i) lf[i] = 0.5f * (float)i;
+  CHECK(be.gpu_score_acc()->seed_layer_flat_cumulative(lf).ok(), "seed_layer_flat_cumulative");
+  CHECK(!be.gpu_score_acc()->seed_layer_flat_cumulative(std::vector<float>(5)).ok(), "layer_flat length check");
+  CHECK(be.gpu_score_acc()->sync_layer_flat_to_cpu().value() == lf, "layer_flat round trip");
+  CHECK(be.gpu_score_acc()->reset_layer_flat().ok(), "reset_layer_flat");
+  auto cleared = be.gpu_score_acc()->sync_layer_flat_to_cpu();
+  for (float x : cleared.value()) CHECK(x == 0.0f, "reset_layer_flat clears");
+  CHECK(be.gpu_score_acc()->sync_to_cpu().value().first == sf, "reset_layer_flat leaves the collapsed buffers");
   CHECK(be.gpu_score_acc()->reset().ok(), "reset");
   auto r4 = be.gpu_score_acc()->sync_to_cpu();
   for (float x : r4.value().first) CHECK(x == 0.0f, "reset clears");
