@@ -41,6 +41,9 @@ struct PrefillParams {
   int32_t seq_len, cache_len, q_start, capacity, batch, window;
   int32_t n_qtiles, group_chunks;  // grid decomposition
   int32_t q_f16, out_f16;
+  // F32 caches take two passes over the same kernel: V rounded to f16 first, then (v_residual) the
+  // rounding's remainder v - f16(v), whose output is added to the first pass's (accumulate).
+  int32_t v_residual, accumulate;
   float scale_log2e;
 };
 
@@ -57,21 +60,25 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 // 8 consecutive K or V elements as f16, read through a bounds-checked buffer descriptor
 // (byte offsets: per-lane `voff`, wave-uniform `soff`); out-of-range chunks read as zero.
+// `residual` (F32 rows only): what the f16 rounding leaves, x - f16(x), itself as f16.
 template <typename KV_T>
-__device__ __forceinline__ half8_t load_kv_chunk(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff);
+__device__ __forceinline__ half8_t load_kv_chunk(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, bool residual);
 template <>
-__device__ __forceinline__ half8_t load_kv_chunk<_Float16>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+__device__ __forceinline__ half8_t load_kv_chunk<_Float16>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, bool) {
   return __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0));
 }
 template <>
-__device__ __forceinline__ half8_t load_kv_chunk<float>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+__device__ __forceinline__ half8_t load_kv_chunk<float>(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, bool residual) {
   const float4_t a = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0));
   const float4_t b = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + 16, soff, 0));
   half8_t h;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    h[e] = (_Float16)a[e];
-    h[4 + e] = (_Float16)b[e];
+  for (int e = 0; e < 8; ++e) {
+    const float x = e < 4 ? a[e] : b[e - 4];
+    const _Float16 hi = (_Float16)x;
+    // an infinite or NaN element keeps its value in the first pass and adds nothing in the second
+    const float rest = x - (float)hi;
+    h[e] = residual ? ((rest == rest && __builtin_fabsf(rest) < 65504.0f) ? (_Float16)rest : (_Float16)0.0f) : hi;
   }
   return h;
 }
@@ -193,14 +200,14 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   const uint32_t kv_bytes = (uint32_t)kv_end * D * sizeof(KV_T);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)kbase, 0, kv_bytes, kBufferFlags);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)vbase, 0, kv_bytes, kBufferFlags);
-  auto fetch_tiles = [&](__amdgpu_buffer_rsrc_t rsrc, int it, half8_t(&pre)[CH]) {
+  auto fetch_tiles = [&](__amdgpu_buffer_rsrc_t rsrc, int it, half8_t(&pre)[CH], bool residual) {
     const uint32_t tile_off = (uint32_t)((kt_begin + it * NG) * BN) * (D * sizeof(KV_T));
 #pragma unroll
     for (int c = 0; c < CH; ++c)
-      pre[c] = load_kv_chunk<KV_T>(rsrc, (uint32_t)(threadIdx.x + NT * c) * (8 * sizeof(KV_T)), tile_off);
+      pre[c] = load_kv_chunk<KV_T>(rsrc, (uint32_t)(threadIdx.x + NT * c) * (8 * sizeof(KV_T)), tile_off, residual);
   };
-  auto fetch_k = [&](int it, auto set_c) { fetch_tiles(k_rsrc, it, kpre[decltype(set_c)::value]); };
-  auto fetch_v = [&](int it, auto set_c) { fetch_tiles(v_rsrc, it, vpre[decltype(set_c)::value]); };
+  auto fetch_k = [&](int it, auto set_c) { fetch_tiles(k_rsrc, it, kpre[decltype(set_c)::value], false); };
+  auto fetch_v = [&](int it, auto set_c) { fetch_tiles(v_rsrc, it, vpre[decltype(set_c)::value], p.v_residual != 0); };
   auto stage_k = [&](int buf, auto set_c) {
     constexpr int SET = decltype(set_c)::value;
 #pragma unroll
@@ -472,7 +479,9 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
         half4_t oh = {(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
         *(half4_t *)((_Float16 *)p.out + ooff + d0) = oh;
       } else {
-        *(float4_t *)((float *)p.out + ooff + d0) = o;
+        float4_t *dst = (float4_t *)((float *)p.out + ooff + d0);
+        if (p.accumulate) o += *dst;
+        *dst = o;
       }
     }
   }
@@ -580,6 +589,15 @@ ARGUS_API int argus_hip_flash_attention_prefill(argus_hip_ctx *ctx, const argus_
   p.out_f16 = a->out_dtype == ARGUS_HIP_F16;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)a->head_dim);
   hipStream_t stream = (hipStream_t)a->stream;
-  return a->kv_dtype == ARGUS_HIP_F16 ? dispatch_dim<_Float16>(ctx, p, a->head_dim, stream)
-                                      : dispatch_dim<float>(ctx, p, a->head_dim, stream);
+  if (a->kv_dtype == ARGUS_HIP_F16) return dispatch_dim<_Float16>(ctx, p, a->head_dim, stream);
+  // F32 cache: the matrix cores take f16 operands.  Rounding K moves a logit by ~1e-4 (nothing at the
+  // 2e-3 output bar), but rounding V moves an output that one key dominates by up to 2^-12 |v|, 2e-3
+  // for |v| >= 4: over the bar in a few rows per thousand random cases.  A second pass over the same
+  // logits with V's rounding remainder restores the f32 values (F32 outputs; an F16 output rounds by
+  // more than that itself).
+  const int rc = dispatch_dim<float>(ctx, p, a->head_dim, stream);
+  if (rc != 1 || p.out_f16) return rc;
+  p.v_residual = 1;
+  p.accumulate = 1;
+  return dispatch_dim<float>(ctx, p, a->head_dim, stream);
 }

@@ -94,7 +94,9 @@ def test_kivi_attention_random(case):
     check_scores(sc, p, what)
 
 
-@pytest.mark.parametrize("case", range(40))
+# the cases past 40 are F32-cache draws in which one key dominates a row with |v| near 4: they fail
+# the 2e-3 bar when V is rounded to f16 without its remainder
+@pytest.mark.parametrize("case", list(range(40)) + [1428, 2005, 2925, 3625, 3862, 3950])
 def test_prefill_random(case):
     from test_gpu_prefill import f16, run_prefill
     rng = np.random.default_rng(9_000_000 + case)
