@@ -53,7 +53,8 @@ def test_reference_matrix(nq, nkv, layout, window):
 @pytest.mark.parametrize("k_f16", [False, True])
 @pytest.mark.parametrize("nq,nkv,d,seq_len,prefix,q_start,q_window,window",
                          [(32, 8, 128, 64, 1024, 960, 32, None), (8, 4, 256, 40, 300, 260, 64, 128),
-                          (14, 2, 64, 128, 128, 0, 16, None), (16, 2, 128, 48, 333, 285, 32, None)])
+                          (14, 2, 64, 128, 128, 0, 16, None), (16, 2, 128, 48, 333, 285, 32, None),
+                          (8, 2, 64, 16, 9300, 9284, 8, None)])  # rows longer than the 8192 keys a workgroup holds in registers
 def test_model_shapes_head_major(k_f16, nq, nkv, d, seq_len, prefix, q_start, q_window, window):
     # HeadMajor cache [kv_heads, capacity, d], chunked prefill (q_start_pos > 0), accumulation into a
     # non-zero sum buffer, F16 K compared with the oracle fed the f16-rounded K.
