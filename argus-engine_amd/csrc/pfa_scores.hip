@@ -280,7 +280,8 @@ __device__ __forceinline__ float prob_at(const PfaParams &p, int h, int r, int s
 // sum_out[h][key] += p over the rows in order; per-head per-row slots are written on the way.
 // The stored exponentials are fetched kBatch rows at a time so the loads overlap; the additions keep
 // their order.
-constexpr int kBatch = 8;
+constexpr int kBatch = 32;     // window rows fetched together by the sum pass (12.9 us; 8: 16.0 us)
+constexpr int kHeadBatch = 8;  // heads fetched together by the head-mean pass, 1 MB apart (13.1 us; 32: 16.4 us)
 template <typename K_T>
 __global__ __launch_bounds__(256) void pfa_sum_kernel(const PfaParams p) {
   const int key = blockIdx.x * 256 + threadIdx.x, h = blockIdx.y;
@@ -330,12 +331,12 @@ __global__ __launch_bounds__(256) void pfa_headmean_kernel(const PfaParams p) {
   if (p.exp_stored) {
     const float *base = p.logits + (int64_t)step * p.prefix_len + key;
     const float *st = p.stats + (int64_t)step * 2;
-    for (int h0 = 0; h0 < p.n_heads_q; h0 += kBatch) {
-      float e[kBatch];
+    for (int h0 = 0; h0 < p.n_heads_q; h0 += kHeadBatch) {
+      float e[kHeadBatch];
 #pragma unroll
-      for (int j = 0; j < kBatch; ++j) e[j] = h0 + j < p.n_heads_q ? base[(int64_t)(h0 + j) * p.qwin * p.prefix_len] : 0.0f;
+      for (int j = 0; j < kHeadBatch; ++j) e[j] = h0 + j < p.n_heads_q ? base[(int64_t)(h0 + j) * p.qwin * p.prefix_len] : 0.0f;
 #pragma unroll
-      for (int j = 0; j < kBatch; ++j)
+      for (int j = 0; j < kHeadBatch; ++j)
         if (h0 + j < p.n_heads_q)
           acc = __fadd_rn(acc, __fmul_rn(__fdiv_rn(e[j], st[(int64_t)(h0 + j) * p.qwin * 2 + 1]), p.inv_heads));
     }
