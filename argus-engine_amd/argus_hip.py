@@ -38,7 +38,12 @@ EXPORTED_SYMBOLS = [
     "argus_hip_score_reduce", "argus_hip_score_reduce_per_layer",
     "argus_hip_kv_scatter_f32_to_f16", "argus_hip_kv_scatter_f32_to_f16_batch",
     "argus_hip_kv_scatter_f32_batch", "argus_hip_kv_decode_descriptor", "argus_hip_kv_encode_descriptor",
-    "argus_hip_attention_gen_desc",
+    "argus_hip_attention_gen_desc", "argus_hip_quant_requant",
+    "argus_hip_quant_cache_make", "argus_hip_quant_cache_drop", "argus_hip_quant_cache_current_pos",
+    "argus_hip_quant_cache_capacity", "argus_hip_quant_cache_current_bits", "argus_hip_quant_cache_update",
+    "argus_hip_quant_cache_flush_if_full", "argus_hip_quant_cache_assemble_view",
+    "argus_hip_quant_cache_get_raw_buffers", "argus_hip_quant_cache_transition_bits",
+    "argus_hip_quant_cache_get_vtable",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -139,6 +144,35 @@ class QuantDequantFlushArgs(C.Structure):
                 ("is_key", C.c_uint8)]
 
 
+class QuantRequantArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("src_mem", C.c_uint64), ("dst_mem", C.c_uint64),
+                ("n_blocks", C.c_size_t), ("old_bits", C.c_uint8), ("new_bits", C.c_uint8)]
+
+
+class QuantCacheMakeArgs(C.Structure):
+    _fields_ = [("ctx", C.c_void_p), ("device", C.c_void_p), ("stream", C.c_void_p), ("build_opts", C.c_char_p),
+                ("kv_heads", C.c_size_t), ("head_dim", C.c_size_t), ("max_seq_len", C.c_size_t),
+                ("residual_size", C.c_size_t), ("bits", C.c_uint8)]
+
+
+class QuantCacheUpdateArgs(C.Structure):
+    _fields_ = [("stream", C.c_void_p), ("k_in_mem", C.c_void_p), ("v_in_mem", C.c_void_p), ("seq_len", C.c_size_t)]
+
+
+class QuantCacheViewOut(C.Structure):
+    _fields_ = [("k_mem", C.c_void_p), ("v_mem", C.c_void_p), ("tokens", C.c_size_t), ("layout", C.c_uint32)]
+
+
+class QuantCacheRawBuffersOut(C.Structure):
+    _fields_ = [("qk_mem", C.c_void_p), ("qv_mem", C.c_void_p), ("res_k_mem", C.c_void_p), ("res_v_mem", C.c_void_p),
+                ("q_tokens", C.c_size_t), ("res_tokens", C.c_size_t), ("res_cap", C.c_size_t), ("bits", C.c_uint8)]
+
+
+class QuantCacheVTable(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("make", "current_pos", "capacity", "current_bits", "update", "flush_if_full",
+                                          "assemble_view", "get_raw_buffers", "transition_bits", "drop")]
+
+
 class QuantScatterResidualArgs(C.Structure):
     _fields_ = [("stream", C.c_void_p), ("res_mem", C.c_uint64), ("attn_mem", C.c_uint64),
                 ("kv_heads", C.c_size_t), ("res_cap", C.c_size_t), ("head_dim", C.c_size_t),
@@ -200,12 +234,75 @@ def _bind():
     lib.argus_hip_kv_scatter_f32_to_f16.argtypes = sc16
     lib.argus_hip_kv_scatter_f32_to_f16_batch.argtypes = sc16 + [i32]
     lib.argus_hip_kv_scatter_f32_batch.argtypes = sc16 + [i32]
+    lib.argus_hip_quant_requant.argtypes = [vp, C.POINTER(QuantRequantArgs)]
+    lib.argus_hip_quant_cache_make.argtypes = [C.POINTER(QuantCacheMakeArgs)]
+    for name in ("current_pos", "capacity", "current_bits", "flush_if_full", "drop"):
+        getattr(lib, "argus_hip_quant_cache_" + name).argtypes = [vp]
+    lib.argus_hip_quant_cache_update.argtypes = [vp, C.POINTER(QuantCacheUpdateArgs)]
+    lib.argus_hip_quant_cache_assemble_view.argtypes = [vp, C.POINTER(QuantCacheViewOut)]
+    lib.argus_hip_quant_cache_get_raw_buffers.argtypes = [vp, C.POINTER(QuantCacheRawBuffersOut)]
+    lib.argus_hip_quant_cache_transition_bits.argtypes = [vp, C.c_uint8]
+    lib.argus_hip_quant_cache_get_vtable.argtypes = []
     for name in EXPORTED_SYMBOLS:
         if name != "argus_hip_last_error":
             getattr(lib, name).restype = C.c_int
+    lib.argus_hip_quant_cache_make.restype = vp
+    lib.argus_hip_quant_cache_get_vtable.restype = C.POINTER(QuantCacheVTable)
+    lib.argus_hip_quant_cache_current_pos.restype = C.c_size_t
+    lib.argus_hip_quant_cache_capacity.restype = C.c_size_t
+    lib.argus_hip_quant_cache_current_bits.restype = C.c_uint8
+    lib.argus_hip_quant_cache_get_raw_buffers.restype = C.c_bool
+    lib.argus_hip_quant_cache_drop.restype = None
 
 
 _bind()
+
+
+class QuantCache:
+    """Handle of argus_hip_quant_cache_* (QuantCacheBackend, crates/argus-extension-api/src/lib.rs:2017-2035)."""
+
+    def __init__(self, ctx, handle):
+        self.ctx, self.handle = ctx, C.c_void_p(handle)
+
+    def close(self):
+        if self.handle:
+            lib.argus_hip_quant_cache_drop(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def current_pos(self):
+        return lib.argus_hip_quant_cache_current_pos(self.handle)
+
+    def capacity(self):
+        return lib.argus_hip_quant_cache_capacity(self.handle)
+
+    def current_bits(self):
+        return lib.argus_hip_quant_cache_current_bits(self.handle)
+
+    def update(self, k, v, check=True):
+        """k, v: device F32 [seq_len, kv_heads, head_dim]."""
+        a = QuantCacheUpdateArgs(stream=_stream(), k_in_mem=_ptr(k), v_in_mem=_ptr(v), seq_len=k.shape[0])
+        return self.ctx._check(lib.argus_hip_quant_cache_update(self.handle, C.byref(a)), check)
+
+    def flush_if_full(self, check=True):
+        return self.ctx._check(lib.argus_hip_quant_cache_flush_if_full(self.handle), check)
+
+    def assemble_view(self):
+        out = QuantCacheViewOut()
+        self.ctx._check(lib.argus_hip_quant_cache_assemble_view(self.handle, C.byref(out)))
+        return out
+
+    def get_raw_buffers(self):
+        out = QuantCacheRawBuffersOut()
+        return out if lib.argus_hip_quant_cache_get_raw_buffers(self.handle, C.byref(out)) else None
+
+    def transition_bits(self, bits, check=True):
+        return self.ctx._check(lib.argus_hip_quant_cache_transition_bits(self.handle, bits), check)
 
 
 class ArgusHipError(RuntimeError):
@@ -404,6 +501,18 @@ class Context:
                            head_dim=head_dim, flush_tokens=flush_tokens,
                            k_block_start=k_block_start, v_block_start=v_block_start, bits=bits)
         return self._check(lib.argus_hip_quant_flush(self.handle, C.byref(a)), check)
+
+    def quant_requant(self, src, dst, n_blocks, old_bits, new_bits, check=True):
+        a = QuantRequantArgs(stream=_stream(), src_mem=_ptr(src), dst_mem=_ptr(dst), n_blocks=n_blocks,
+                             old_bits=old_bits, new_bits=new_bits)
+        return self._check(lib.argus_hip_quant_requant(self.handle, C.byref(a)), check)
+
+    def quant_cache(self, kv_heads, head_dim, max_seq_len, residual_size, bits):
+        """The KIVI container behind the CACHE-category vtable; None when `make` refuses."""
+        a = QuantCacheMakeArgs(ctx=self.handle, device=None, stream=_stream(), build_opts=None, kv_heads=kv_heads,
+                               head_dim=head_dim, max_seq_len=max_seq_len, residual_size=residual_size, bits=bits)
+        h = lib.argus_hip_quant_cache_make(C.byref(a))
+        return QuantCache(self, h) if h else None
 
     def quant_dequant_flush(self, blocks, attn, kv_heads, head_dim, n_groups_or_tokens, tok_base,
                             block_start, bits, is_key, check=True):

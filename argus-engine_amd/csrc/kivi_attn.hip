@@ -309,6 +309,33 @@ __global__ __launch_bounds__(128) void kivi_flush_v_kernel(const float *__restri
   quantize_block<BITS>(x, qv + (block_start + i) * BB);
 }
 
+// ---- bit-width transition ------------------------------------------------------------------------
+// QuantizedRecentWindowCache::transition_bits between two quantised widths
+// (engine/src/kv/quant_window_cache.rs:1308-1372): every block is dequantised to 32 f32 values
+// (`q * d + m`, crates/argus-kv-codec/src/lib.rs:61-72: the product of a code and an f16 scale is
+// exact in f32, so the sum rounds once) and quantised again at the new width; block count and order
+// stay.  One thread per block.
+template <int OLD, int NEW>
+__global__ __launch_bounds__(128) void kivi_requant_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t n_blocks) {
+  constexpr int OB = 4 + 32 * OLD / 8, NB = 4 + 32 * NEW / 8;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_blocks) return;
+  const uint32_t *w = (const uint32_t *)(src + i * OB);  // block sizes are multiples of 4
+  uint32_t words[OB / 4];
+#pragma unroll
+  for (int k = 0; k < OB / 4; ++k) words[k] = w[k];
+  const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(words[0] & 0xffffu));
+  const float m = (float)__builtin_bit_cast(_Float16, (uint16_t)(words[0] >> 16));
+  float x[32];
+#pragma unroll
+  for (int e = 0; e < 32; ++e) {
+    const int bit = e * OLD;
+    const uint32_t c = (words[1 + bit / 32] >> (bit % 32)) & ((1u << OLD) - 1u);
+    x[e] = __fadd_rn(__fmul_rn((float)c, d), m);
+  }
+  quantize_block<NEW>(x, dst + i * NB);
+}
+
 template <int BITS>
 int launch_kivi(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   // ARGUS_HIP_KIVI=valu (read when the context is created) keeps the vector-ALU kernel for A/B measurements.
@@ -502,6 +529,38 @@ ARGUS_API int argus_hip_quant_flush(argus_hip_ctx *ctx, const argus_hip_quant_fl
     default: ARGUS_FLUSH(8); break;
   }
 #undef ARGUS_FLUSH
+  ARGUS_HIP_CHECK(ctx, hipGetLastError());
+  return ARGUS_HIP_OK;
+}
+
+ARGUS_API int argus_hip_quant_requant(argus_hip_ctx *ctx, const argus_hip_quant_requant_args *a) {
+  if (!ctx || !a) return ARGUS_HIP_ERR_INVALID;
+  if (!bits_ok(a->old_bits) || !bits_ok(a->new_bits))
+    return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "quant_requant: bits %d -> %d", (int)a->old_bits, (int)a->new_bits);
+  if (a->n_blocks == 0) return ARGUS_HIP_OK;
+  if (!a->src_mem || !a->dst_mem || ((a->src_mem | a->dst_mem) & 3))
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "quant_requant: null or misaligned block stream");
+  const uint64_t ob = 4 + 32 * (uint64_t)a->old_bits / 8, nb = 4 + 32 * (uint64_t)a->new_bits / 8;
+  if (a->src_mem < a->dst_mem + a->n_blocks * nb && a->dst_mem < a->src_mem + a->n_blocks * ob)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "quant_requant: source and destination streams overlap");
+  hipStream_t stream = (hipStream_t)a->stream;
+  const dim3 grid((unsigned)((a->n_blocks + 127) / 128));
+  const uint8_t *src = (const uint8_t *)a->src_mem;
+  uint8_t *dst = (uint8_t *)a->dst_mem;
+  const int64_t n = (int64_t)a->n_blocks;
+#define ARGUS_REQUANT(O, N) hipLaunchKernelGGL((kivi_requant_kernel<O, N>), grid, dim3(128), 0, stream, src, dst, n)
+  switch (a->old_bits * 16 + a->new_bits) {
+    case 2 * 16 + 2: ARGUS_REQUANT(2, 2); break;
+    case 2 * 16 + 4: ARGUS_REQUANT(2, 4); break;
+    case 2 * 16 + 8: ARGUS_REQUANT(2, 8); break;
+    case 4 * 16 + 2: ARGUS_REQUANT(4, 2); break;
+    case 4 * 16 + 4: ARGUS_REQUANT(4, 4); break;
+    case 4 * 16 + 8: ARGUS_REQUANT(4, 8); break;
+    case 8 * 16 + 2: ARGUS_REQUANT(8, 2); break;
+    case 8 * 16 + 4: ARGUS_REQUANT(8, 4); break;
+    default: ARGUS_REQUANT(8, 8); break;
+  }
+#undef ARGUS_REQUANT
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   return ARGUS_HIP_OK;
 }

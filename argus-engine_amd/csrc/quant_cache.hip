@@ -1,0 +1,247 @@
+// The KIVI container as a C ABI: the CACHE-category capability of the reference's plugin interface
+// (QuantCacheBackend / QuantCacheVTable, crates/argus-extension-api/src/lib.rs:1932-2090) served by the
+// GPU mode of QuantizedRecentWindowCache (engine/src/kv/quant_window_cache.rs:380-586 new_gpu,
+// 2518-2562 update, 1563-1686 update_gpu, 1688-1848 flush_residual_gpu, 741-760 get_raw_gpu_buffers,
+// 2248-2475 assemble_view_gpu, 1308-1448 transition_bits between quantised widths) with every step on
+// the device: append = the gather kernel, flush = quantise-at-flush, the tokens a flush leaves behind
+// move down with the overlap-safe shift, a width transition requantises both block streams in place
+// of the reference's read-back / CPU loop / upload.  Host code only; the kernels are those of
+// kivi_attn.hip and kivi_view.hip behind their own entry points.
+#include "argus_hip_internal.hpp"
+
+#include <algorithm>
+#include <new>
+
+namespace {
+
+constexpr size_t kGroup = 32;  // QKKV: tokens per key block, channels per value block
+
+struct QuantCache {
+  argus_hip_ctx *ctx = nullptr;
+  void *stream = nullptr;
+  size_t kv_heads = 0, head_dim = 0, max_seq_len = 0, res_cap = 0;
+  uint8_t bits = 0;
+  size_t q_tokens = 0, res_pos = 0, deq_tokens = 0;
+  void *res_k = nullptr, *res_v = nullptr, *qk = nullptr, *qv = nullptr, *attn_k = nullptr, *attn_v = nullptr;
+
+  size_t block_bytes(uint8_t b) const { return 4 + kGroup * b / 8; }
+  // blocks one stream can come to hold: whole groups of max_seq_len tokens
+  size_t stream_blocks() const { return (max_seq_len / kGroup + 1) * kv_heads * head_dim; }
+  size_t blocks_held() const { return q_tokens * kv_heads * head_dim / kGroup; }
+  void release() {
+    for (void **p : {&res_k, &res_v, &qk, &qv, &attn_k, &attn_v}) {
+      if (*p) argus_hip_free(ctx, *p);
+      *p = nullptr;
+    }
+  }
+};
+
+// flush_residual_gpu: whole groups of the ring become blocks, the remainder moves to the ring's start.
+int flush_residual(QuantCache *c, void *stream) {
+  const size_t flush_tokens = c->res_pos / kGroup * kGroup;
+  if (flush_tokens == 0) return ARGUS_HIP_OK;
+  argus_hip_quant_flush_args f{};
+  f.stream = stream;
+  f.res_k_mem = (uint64_t)c->res_k; f.res_v_mem = (uint64_t)c->res_v;
+  f.qk_mem = (uint64_t)c->qk; f.qv_mem = (uint64_t)c->qv;
+  f.kv_heads = c->kv_heads; f.res_cap = c->res_cap; f.head_dim = c->head_dim; f.flush_tokens = flush_tokens;
+  f.k_block_start = f.v_block_start = c->blocks_held();
+  f.bits = c->bits;
+  int rc = argus_hip_quant_flush(c->ctx, &f);
+  if (rc != ARGUS_HIP_OK) return rc;
+  c->q_tokens += flush_tokens;
+  const size_t remaining = c->res_pos - flush_tokens;
+  if (remaining > 0) {
+    for (void *ring : {c->res_k, c->res_v})
+      for (size_t h = 0; h < c->kv_heads; ++h) {
+        float *base = (float *)ring + h * c->res_cap * c->head_dim;
+        rc = argus_hip_buffer_shift(c->ctx, stream, base, base + flush_tokens * c->head_dim, remaining * c->head_dim * sizeof(float));
+        if (rc != ARGUS_HIP_OK) return rc;
+      }
+  }
+  c->res_pos = remaining;
+  return ARGUS_HIP_OK;
+}
+
+}  // namespace
+
+ARGUS_API void *argus_hip_quant_cache_make(const argus_hip_quant_cache_make_args *a) {
+  if (!a || !a->ctx) return nullptr;
+  argus_hip_ctx *ctx = (argus_hip_ctx *)a->ctx;
+  // the reference asserts these (quant_window_cache.rs:283-295); bits 16 (the unquantised fallback) has
+  // no device form here
+  if (a->bits != 2 && a->bits != 4 && a->bits != 8) {
+    argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "quant_cache_make: bits %d (2, 4 or 8)", (int)a->bits);
+    return nullptr;
+  }
+  if (a->kv_heads == 0 || a->head_dim == 0 || a->head_dim % kGroup || a->residual_size == 0 || a->residual_size % kGroup ||
+      a->max_seq_len == 0) {
+    argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "quant_cache_make: kv_heads %zu head_dim %zu residual_size %zu max_seq_len %zu", a->kv_heads,
+               a->head_dim, a->residual_size, a->max_seq_len);
+    return nullptr;
+  }
+  QuantCache *c = new (std::nothrow) QuantCache();
+  if (!c) return nullptr;
+  c->ctx = ctx; c->stream = a->stream;
+  c->kv_heads = a->kv_heads; c->head_dim = a->head_dim; c->max_seq_len = a->max_seq_len; c->res_cap = a->residual_size; c->bits = a->bits;
+  const size_t res_bytes = c->kv_heads * c->res_cap * c->head_dim * sizeof(float);
+  const size_t stream_bytes = c->stream_blocks() * c->block_bytes(c->bits);
+  if (argus_hip_malloc(ctx, res_bytes, &c->res_k) != ARGUS_HIP_OK || argus_hip_malloc(ctx, res_bytes, &c->res_v) != ARGUS_HIP_OK ||
+      argus_hip_malloc(ctx, stream_bytes, &c->qk) != ARGUS_HIP_OK || argus_hip_malloc(ctx, stream_bytes, &c->qv) != ARGUS_HIP_OK) {
+    c->release();
+    delete c;
+    return nullptr;
+  }
+  return c;
+}
+
+ARGUS_API void argus_hip_quant_cache_drop(void *handle) {
+  QuantCache *c = (QuantCache *)handle;
+  if (!c) return;
+  c->release();
+  delete c;
+}
+
+ARGUS_API size_t argus_hip_quant_cache_current_pos(void *handle) {
+  const QuantCache *c = (const QuantCache *)handle;
+  return c ? c->q_tokens + c->res_pos : 0;
+}
+ARGUS_API size_t argus_hip_quant_cache_capacity(void *handle) {
+  const QuantCache *c = (const QuantCache *)handle;
+  return c ? c->max_seq_len : 0;
+}
+ARGUS_API uint8_t argus_hip_quant_cache_current_bits(void *handle) {
+  const QuantCache *c = (const QuantCache *)handle;
+  return c ? c->bits : 0;
+}
+
+ARGUS_API int32_t argus_hip_quant_cache_update(void *handle, const argus_hip_quant_cache_update_args *a) {
+  QuantCache *c = (QuantCache *)handle;
+  if (!c || !a) return ARGUS_HIP_ERR_INVALID;
+  if (a->seq_len == 0) return ARGUS_HIP_OK;
+  if (!a->k_in_mem || !a->v_in_mem) return argus_fail(c->ctx, ARGUS_HIP_ERR_INVALID, "quant_cache_update: null input");
+  if (c->q_tokens + c->res_pos + a->seq_len > c->max_seq_len)
+    return argus_fail(c->ctx, ARGUS_HIP_ERR_INVALID, "QuantWindowCache overflow: %zu + %zu > %zu", c->q_tokens + c->res_pos, a->seq_len,
+                      c->max_seq_len);
+  void *stream = a->stream ? a->stream : c->stream;
+  size_t written = 0;
+  while (written < a->seq_len) {
+    if (c->res_pos >= c->res_cap) {
+      const int rc = flush_residual(c, stream);
+      if (rc != ARGUS_HIP_OK) return rc;
+    }
+    const size_t batch = std::min(a->seq_len - written, c->res_cap - c->res_pos);
+    const size_t off = written * c->kv_heads * c->head_dim * sizeof(float);
+    for (int which = 0; which < 2; ++which) {
+      argus_hip_quant_gather_args g{stream, (uint64_t)((const char *)(which ? a->v_in_mem : a->k_in_mem) + off),
+                                    (uint64_t)(which ? c->res_v : c->res_k), c->kv_heads, c->res_cap, c->head_dim, batch, c->res_pos};
+      const int rc = argus_hip_gather_update_quant(c->ctx, &g);
+      if (rc != ARGUS_HIP_OK) return rc;
+    }
+    c->res_pos += batch;
+    written += batch;
+  }
+  return ARGUS_HIP_OK;
+}
+
+ARGUS_API int32_t argus_hip_quant_cache_flush_if_full(void *handle) {
+  QuantCache *c = (QuantCache *)handle;
+  if (!c) return ARGUS_HIP_ERR_INVALID;
+  if (c->res_pos < c->res_cap) return ARGUS_HIP_OK;
+  return flush_residual(c, c->stream);
+}
+
+ARGUS_API int32_t argus_hip_quant_cache_assemble_view(void *handle, argus_hip_quant_cache_view_out *out) {
+  QuantCache *c = (QuantCache *)handle;
+  if (!c || !out) return ARGUS_HIP_ERR_INVALID;
+  // the view is allocated once, at max_seq_len, the first time it is asked for
+  const size_t view_bytes = c->max_seq_len * c->kv_heads * c->head_dim * 2;
+  for (void **p : {&c->attn_k, &c->attn_v})
+    if (!*p) {
+      const int rc = argus_hip_malloc(c->ctx, view_bytes, p);
+      if (rc != ARGUS_HIP_OK) return rc;
+    }
+  while (c->deq_tokens < c->q_tokens) {
+    // one flush of the streams at a time: key blocks are grouped per flush
+    const size_t flush_tokens = std::min(c->res_cap, c->q_tokens - c->deq_tokens);
+    const size_t block_start = c->deq_tokens * c->kv_heads * c->head_dim / kGroup;
+    argus_hip_quant_dequant_flush_args dk{c->stream, (uint64_t)c->qk, (uint64_t)c->attn_k, c->kv_heads, c->head_dim, flush_tokens / kGroup,
+                                          c->deq_tokens, block_start, c->bits, 1};
+    argus_hip_quant_dequant_flush_args dv{c->stream, (uint64_t)c->qv, (uint64_t)c->attn_v, c->kv_heads, c->head_dim, flush_tokens,
+                                          c->deq_tokens, block_start, c->bits, 0};
+    int rc = argus_hip_quant_dequant_flush(c->ctx, &dk);
+    if (rc == ARGUS_HIP_OK) rc = argus_hip_quant_dequant_flush(c->ctx, &dv);
+    if (rc != ARGUS_HIP_OK) return rc;
+    c->deq_tokens += flush_tokens;
+  }
+  if (c->res_pos > 0) {
+    argus_hip_quant_scatter_residual_args sk{c->stream, (uint64_t)c->res_k, (uint64_t)c->attn_k, c->kv_heads, c->res_cap, c->head_dim,
+                                             c->res_pos, c->q_tokens};
+    argus_hip_quant_scatter_residual_args sv = sk;
+    sv.res_mem = (uint64_t)c->res_v;
+    sv.attn_mem = (uint64_t)c->attn_v;
+    int rc = argus_hip_quant_scatter_residual(c->ctx, &sk);
+    if (rc == ARGUS_HIP_OK) rc = argus_hip_quant_scatter_residual(c->ctx, &sv);
+    if (rc != ARGUS_HIP_OK) return rc;
+  }
+  out->k_mem = c->attn_k;
+  out->v_mem = c->attn_v;
+  out->tokens = c->q_tokens + c->res_pos;
+  out->layout = ARGUS_HIP_VIEW_TOKENS_HEADS_DIM;
+  return ARGUS_HIP_OK;
+}
+
+ARGUS_API bool argus_hip_quant_cache_get_raw_buffers(void *handle, argus_hip_quant_cache_raw_buffers_out *out) {
+  const QuantCache *c = (const QuantCache *)handle;
+  if (!c || !out || c->q_tokens + c->res_pos == 0) return false;  // no native-consumable set on an empty cache
+  out->qk_mem = c->qk; out->qv_mem = c->qv; out->res_k_mem = c->res_k; out->res_v_mem = c->res_v;
+  out->q_tokens = c->q_tokens; out->res_tokens = c->res_pos; out->res_cap = c->res_cap; out->bits = c->bits;
+  return true;
+}
+
+ARGUS_API int32_t argus_hip_quant_cache_transition_bits(void *handle, uint8_t target_bits) {
+  QuantCache *c = (QuantCache *)handle;
+  if (!c) return ARGUS_HIP_ERR_INVALID;
+  if (target_bits == c->bits) return ARGUS_HIP_OK;
+  if (target_bits != 2 && target_bits != 4 && target_bits != 8)
+    return argus_fail(c->ctx, ARGUS_HIP_ERR_UNSUPPORTED, "quant_cache_transition_bits: %d -> %d (quantised widths 2, 4, 8 only)", (int)c->bits,
+                      (int)target_bits);
+  // Both streams are rewritten at the new block size into fresh buffers (the one allocation this
+  // handle makes after `make`; a transition is a rare, policy-driven event), then the old ones go.
+  const size_t new_bytes = c->stream_blocks() * c->block_bytes(target_bits);
+  void *nk = nullptr, *nv = nullptr;
+  int rc = argus_hip_malloc(c->ctx, new_bytes, &nk);
+  if (rc == ARGUS_HIP_OK) rc = argus_hip_malloc(c->ctx, new_bytes, &nv);
+  if (rc == ARGUS_HIP_OK && c->q_tokens > 0) {
+    argus_hip_quant_requant_args r{c->stream, (uint64_t)c->qk, (uint64_t)nk, c->blocks_held(), c->bits, target_bits};
+    rc = argus_hip_quant_requant(c->ctx, &r);
+    if (rc == ARGUS_HIP_OK) {
+      r.src_mem = (uint64_t)c->qv;
+      r.dst_mem = (uint64_t)nv;
+      rc = argus_hip_quant_requant(c->ctx, &r);
+    }
+    // the old streams are freed below: every kernel that reads them must have finished
+    if (rc == ARGUS_HIP_OK) rc = argus_hip_synchronize(c->ctx, c->stream);
+  }
+  if (rc != ARGUS_HIP_OK) {
+    if (nk) argus_hip_free(c->ctx, nk);
+    if (nv) argus_hip_free(c->ctx, nv);
+    return rc;
+  }
+  argus_hip_free(c->ctx, c->qk);
+  argus_hip_free(c->ctx, c->qv);
+  c->qk = nk;
+  c->qv = nv;
+  c->bits = target_bits;
+  c->deq_tokens = 0;  // the F16 view is rebuilt from the new blocks
+  return ARGUS_HIP_OK;
+}
+
+ARGUS_API const argus_hip_quant_cache_vtable *argus_hip_quant_cache_get_vtable(void) {
+  static const argus_hip_quant_cache_vtable vt = {
+      argus_hip_quant_cache_make,          argus_hip_quant_cache_current_pos,   argus_hip_quant_cache_capacity,
+      argus_hip_quant_cache_current_bits,  argus_hip_quant_cache_update,        argus_hip_quant_cache_flush_if_full,
+      argus_hip_quant_cache_assemble_view, argus_hip_quant_cache_get_raw_buffers, argus_hip_quant_cache_transition_bits,
+      argus_hip_quant_cache_drop};
+  return &vt;
+}

@@ -358,61 +358,37 @@ struct QuantWindowRawBuffers {
 };
 
 // The GPU mode of QuantizedRecentWindowCache (engine/src/kv/quant_window_cache.rs:380-586 new_gpu,
-// 2518-2562 update, 1563-1686 update_gpu, 1688-1848 flush_residual_gpu, 741-760
-// get_raw_gpu_buffers, 2248-2475 assemble_view_gpu / get_view_gpu, 810-843 reset) for one layer:
-// an F32 residual ring [kv_heads, res_cap, head_dim] that new tokens are appended to, and the two
-// block streams (keys per channel, values per token, flush after flush) it is quantised into when
-// full.  Every step stays on the device: append = gather_update_quant, flush = quant_flush (the
-// reference reads the ring back, quantises on the CPU and uploads the blocks; the blocks are bit
-// for bit the same), the tokens a flush leaves behind move down with buffer_shift.  The F16
-// attention view (blocks dequantised + residual rows) is assembled on request for callers that
-// do not take the fused kernel.  Flush metrics (QCF / AWQE proxies) and transition_bits are host
-// bookkeeping of the reference with no device part and are not mirrored.
+// 2518-2562 update, 1688-1848 flush_residual_gpu, 741-760 get_raw_gpu_buffers, 2248-2475
+// get_view_gpu, 973-1448 transition_bits, 810-843 reset) for one layer, over the library's
+// CACHE-category handle (argus_hip_quant_cache_*, the C form of QuantCacheBackend,
+// crates/argus-extension-api/src/lib.rs:2017-2035): an F32 residual ring that new tokens are
+// appended to and the two block streams it is quantised into when full, every step on the device.
+// Flush metrics (QCF / AWQE proxies) and the unquantised bits = 16 mode are host bookkeeping of
+// the reference with no device part and are not mirrored.
 class HipQuantWindowCache {
  public:
-  static constexpr size_t kGroup = 32;  // QKKV, tokens per key block group
   static Result<std::unique_ptr<HipQuantWindowCache>> new_gpu(HipBackend *be, size_t kv_heads, size_t head_dim, size_t max_seq_len,
                                                               size_t residual_size, uint8_t bits) {
     using R = Result<std::unique_ptr<HipQuantWindowCache>>;
     if (!be) return R::Err("quant-window GPU mode needs a backend");
-    if (bits != 2 && bits != 4 && bits != 8) return R::Err("quant-window bits must be 2, 4 or 8");
-    if (kv_heads == 0 || head_dim == 0 || head_dim % kGroup) return R::Err("head_dim must be a positive multiple of 32");
-    // the reference asserts the same (quant_window_cache.rs:283-290)
-    if (residual_size == 0 || residual_size % kGroup) return R::Err("residual_size must be a positive multiple of 32");
-    const size_t res_cap = residual_size;
+    argus_hip_quant_cache_make_args a{};
+    a.ctx = be->ctx(); a.kv_heads = kv_heads; a.head_dim = head_dim; a.max_seq_len = max_seq_len; a.residual_size = residual_size; a.bits = bits;
+    void *h = argus_hip_quant_cache_make(&a);
+    if (!h) return R::Err("quant-window cache: " + be->last_error());
     std::unique_ptr<HipQuantWindowCache> c(new HipQuantWindowCache());
-    c->be_ = be;
-    c->cap_ = HipQuantAttnBackend(be->ctx());
-    c->kv_heads_ = kv_heads; c->head_dim_ = head_dim; c->max_seq_len_ = max_seq_len; c->res_cap_ = res_cap; c->bits_ = bits;
-    const size_t block_bytes = 4 + kGroup * bits / 8;
-    const size_t max_blocks = (max_seq_len / kGroup + 1) * kv_heads * head_dim;  // per stream, whole flushes only
-    const size_t res_bytes = kv_heads * res_cap * head_dim * sizeof(float);
-    for (void **p : {&c->res_k_, &c->res_v_}) {
-      auto a = be->alloc(res_bytes);
-      if (!a.ok()) return R::Err(a.error());
-      *p = a.value();
-    }
-    for (void **p : {&c->qk_, &c->qv_}) {
-      auto a = be->alloc(max_blocks * block_bytes);
-      if (!a.ok()) return R::Err(a.error());
-      *p = a.value();
-    }
+    c->be_ = be; c->h_ = h; c->kv_heads_ = kv_heads; c->head_dim_ = head_dim; c->max_seq_len_ = max_seq_len; c->res_cap_ = residual_size;
     return R::Ok(std::move(c));
   }
-  ~HipQuantWindowCache() {
-    for (void *p : {res_k_, res_v_, qk_, qv_, attn_k_, attn_v_})
-      if (p) be_->free(p);
-  }
+  ~HipQuantWindowCache() { argus_hip_quant_cache_drop(h_); }
   HipQuantWindowCache(const HipQuantWindowCache &) = delete;
   HipQuantWindowCache &operator=(const HipQuantWindowCache &) = delete;
 
   bool is_gpu() const { return true; }
-  uint8_t bits() const { return bits_; }
-  size_t current_pos() const { return q_tokens_ + res_pos_; }
-  size_t capacity() const { return max_seq_len_; }
+  uint8_t bits() const { return argus_hip_quant_cache_current_bits(h_); }
+  size_t current_pos() const { return argus_hip_quant_cache_current_pos(h_); }
+  size_t capacity() const { return argus_hip_quant_cache_capacity(h_); }
   size_t kv_heads() const { return kv_heads_; }
   size_t head_dim() const { return head_dim_; }
-  size_t res_cap() const { return res_cap_; }
 
   // update(new_k, new_v): device F32 [1, seq_len, kv_heads, head_dim]; flushes whenever the ring is full.
   Status update(const Tensor &new_k, const Tensor &new_v) {
@@ -420,65 +396,27 @@ class HipQuantWindowCache {
       return Status::Err("QuantWindowCache update: expected [1, seq_len, kv_heads, head_dim]");
     if (new_k.dtype != DType::F32 || new_v.dtype != DType::F32 || !new_k.device || !new_v.device)
       return Status::Err("QuantWindowCache update: device F32 tensors expected");
-    const size_t seq_len = new_k.dims[1];
-    if (current_pos() + seq_len > max_seq_len_)
-      return Status::Err("QuantWindowCache overflow: " + std::to_string(current_pos()) + " + " + std::to_string(seq_len) + " > " +
-                         std::to_string(max_seq_len_));
-    size_t written = 0;
-    while (written < seq_len) {
-      if (res_pos_ >= res_cap_) {
-        Status st = flush_residual_gpu();
-        if (!st.ok()) return st;
-      }
-      const size_t batch = std::min(seq_len - written, res_cap_ - res_pos_);
-      const size_t off = written * kv_heads_ * head_dim_ * sizeof(float);
-      for (int which = 0; which < 2; ++which) {
-        argus_hip_quant_gather_args g{nullptr, (uint64_t)((const char *)(which ? new_v.ptr : new_k.ptr) + off),
-                                      (uint64_t)(which ? res_v_ : res_k_), kv_heads_, res_cap_, head_dim_, batch, res_pos_};
-        const int rc = cap_.gather_update_quant(g);
-        if (rc != 0) return Status::Err("quant-window gather_update_quant (" + std::string(which ? "V" : "K") + ") failed (rc=" + std::to_string(rc) + ")");
-      }
-      res_pos_ += batch;
-      written += batch;
-    }
-    return OkStatus();
+    argus_hip_quant_cache_update_args a{nullptr, new_k.ptr, new_v.ptr, new_k.dims[1]};
+    return wrap(argus_hip_quant_cache_update(h_, &a));
   }
+  Status flush_if_full() { return wrap(argus_hip_quant_cache_flush_if_full(h_)); }
+  Status transition_bits(uint8_t new_bits) { return wrap(argus_hip_quant_cache_transition_bits(h_, new_bits)); }
 
-  // Quantise the whole groups of the ring into blocks and move what is left to its start.
-  Status flush_residual_gpu() {
-    const size_t n_groups = res_pos_ / kGroup, flush_tokens = n_groups * kGroup;
-    if (flush_tokens == 0) return OkStatus();
-    argus_hip_quant_flush_args f{};
-    f.res_k_mem = (uint64_t)res_k_; f.res_v_mem = (uint64_t)res_v_; f.qk_mem = (uint64_t)qk_; f.qv_mem = (uint64_t)qv_;
-    f.kv_heads = kv_heads_; f.res_cap = res_cap_; f.head_dim = head_dim_; f.flush_tokens = flush_tokens;
-    // both streams hold q_tokens * kv_heads * head_dim / 32 blocks so far
-    f.k_block_start = f.v_block_start = q_tokens_ * kv_heads_ * head_dim_ / kGroup;
-    f.bits = bits_;
-    const int rc = argus_hip_quant_flush(be_->ctx(), &f);
-    if (rc != 0) return Status::Err("quant-window flush failed (rc=" + std::to_string(rc) + "): " + be_->last_error());
-    q_tokens_ += flush_tokens;
-    const size_t remaining = res_pos_ - flush_tokens;
-    if (remaining > 0) {
-      for (void *ring : {res_k_, res_v_}) {
-        Tensor t{ring, DType::F32, {kv_heads_, res_cap_, head_dim_}, true};
-        for (size_t h = 0; h < kv_heads_; ++h) {
-          const size_t base = h * res_cap_ * head_dim_;
-          Status st = be_->buffer_shift(t, base + flush_tokens * head_dim_, base, remaining * head_dim_);
-          if (!st.ok()) return st;
-        }
-      }
-    }
-    res_pos_ = remaining;
-    return OkStatus();
+  // None (ok() false) for an empty cache, like the reference for a cache with no native set.
+  Result<QuantWindowRawBuffers> get_raw_gpu_buffers() const {
+    argus_hip_quant_cache_raw_buffers_out o{};
+    if (!argus_hip_quant_cache_get_raw_buffers(h_, &o)) return Result<QuantWindowRawBuffers>::Err("no raw buffers");
+    return Result<QuantWindowRawBuffers>::Ok(QuantWindowRawBuffers{o.qk_mem, o.qv_mem, o.res_k_mem, o.res_v_mem, o.q_tokens, o.res_tokens, o.res_cap, o.bits});
   }
-
-  QuantWindowRawBuffers get_raw_gpu_buffers() const { return QuantWindowRawBuffers{qk_, qv_, res_k_, res_v_, q_tokens_, res_pos_, res_cap_, bits_}; }
 
   // QuantWindowFormat::attention_native (engine/src/kv/quant_window_format.rs:258-330): fused
   // dequant + attention over the raw buffers; `scores` (host, [n_heads_q, current_pos]) optional.
   Status attention_native(const Tensor &q, Tensor &out, size_t n_heads_q, float *scores, size_t scores_len) const {
-    const QuantWindowRawBuffers raw = get_raw_gpu_buffers();
-    if (!cap_.has_quant_attn_kernel(raw.bits)) return Status::Err("no fused kernel for these bits");
+    auto got = get_raw_gpu_buffers();
+    if (!got.ok()) return Status::Err("attention_native: empty cache");
+    const QuantWindowRawBuffers &raw = got.value();
+    HipQuantAttnBackend cap(be_->ctx());
+    if (!cap.has_quant_attn_kernel(raw.bits)) return Status::Err("no fused kernel for these bits");
     argus_hip_quant_attn_args a{};
     a.q_mem = (uint64_t)q.ptr; a.qk_mem = (uint64_t)raw.qk_buf; a.qv_mem = (uint64_t)raw.qv_buf;
     a.res_k_mem = (uint64_t)raw.res_k; a.res_v_mem = (uint64_t)raw.res_v; a.out_mem = (uint64_t)out.ptr;
@@ -486,51 +424,39 @@ class HipQuantWindowCache {
     a.num_heads_q = n_heads_q; a.num_heads_kv = kv_heads_; a.head_dim = head_dim_;
     a.q_tokens = raw.q_tokens; a.res_tokens = raw.res_tokens; a.res_cap = raw.res_cap;
     a.scale = 1.0f / std::sqrt((float)head_dim_); a.bits = raw.bits;
-    const int rc = cap_.attention_gen_quant(a);
+    const int rc = cap.attention_gen_quant(a);
     return rc == 0 ? OkStatus() : Status::Err("attention_gen_quant failed (rc=" + std::to_string(rc) + "): " + be_->last_error());
   }
 
-  // get_view_gpu: F16 [max_seq_len, kv_heads, head_dim] views covering [0, current_pos); blocks
-  // flushed since the last call are dequantised, the residual rows copied behind them.
+  // get_view_gpu: F16 [max_seq_len, kv_heads, head_dim] views covering [0, current_pos).
   Result<std::pair<Tensor, Tensor>> get_view_gpu() {
     using R = Result<std::pair<Tensor, Tensor>>;
-    const size_t view_bytes = max_seq_len_ * kv_heads_ * head_dim_ * 2;
-    for (void **p : {&attn_k_, &attn_v_})
-      if (!*p) {
-        auto a = be_->alloc(view_bytes);
-        if (!a.ok()) return R::Err(a.error());
-        *p = a.value();
-      }
-    while (deq_tokens_ < q_tokens_) {
-      // one flush of the stream at a time: key blocks are grouped per flush
-      const size_t flush_tokens = std::min(res_cap_, q_tokens_ - deq_tokens_);
-      const size_t block_start = deq_tokens_ * kv_heads_ * head_dim_ / kGroup;
-      argus_hip_quant_dequant_flush_args dk{nullptr, (uint64_t)qk_, (uint64_t)attn_k_, kv_heads_, head_dim_, flush_tokens / kGroup, deq_tokens_, block_start, bits_, 1};
-      argus_hip_quant_dequant_flush_args dv{nullptr, (uint64_t)qv_, (uint64_t)attn_v_, kv_heads_, head_dim_, flush_tokens, deq_tokens_, block_start, bits_, 0};
-      if (cap_.dequant_flush(dk) != 0 || cap_.dequant_flush(dv) != 0) return R::Err("dequant_flush failed: " + be_->last_error());
-      deq_tokens_ += flush_tokens;
-    }
-    if (res_pos_ > 0) {
-      argus_hip_quant_scatter_residual_args sk{nullptr, (uint64_t)res_k_, (uint64_t)attn_k_, kv_heads_, res_cap_, head_dim_, res_pos_, q_tokens_};
-      argus_hip_quant_scatter_residual_args sv = sk;
-      sv.res_mem = (uint64_t)res_v_; sv.attn_mem = (uint64_t)attn_v_;
-      if (cap_.scatter_residual(sk) != 0 || cap_.scatter_residual(sv) != 0) return R::Err("scatter_residual failed: " + be_->last_error());
-    }
-    Tensor tk{attn_k_, DType::F16, {1, max_seq_len_, kv_heads_, head_dim_}, true}, tv = tk;
-    tv.ptr = attn_v_;
+    argus_hip_quant_cache_view_out o{};
+    const int rc = argus_hip_quant_cache_assemble_view(h_, &o);
+    if (rc != 0) return R::Err("assemble_view failed (rc=" + std::to_string(rc) + "): " + be_->last_error());
+    Tensor tk{o.k_mem, DType::F16, {1, max_seq_len_, kv_heads_, head_dim_}, true}, tv = tk;
+    tv.ptr = o.v_mem;
     return R::Ok(std::make_pair(tk, tv));
   }
 
-  void reset() { q_tokens_ = res_pos_ = deq_tokens_ = 0; }
+  // reset(): a fresh handle of the same geometry and width (the reference keeps its buffers and
+  // zeroes its counters; the vtable has no such call)
+  Status reset() {
+    argus_hip_quant_cache_make_args a{};
+    a.ctx = be_->ctx(); a.kv_heads = kv_heads_; a.head_dim = head_dim_; a.max_seq_len = max_seq_len_; a.residual_size = res_cap_; a.bits = bits();
+    void *h = argus_hip_quant_cache_make(&a);
+    if (!h) return Status::Err("quant-window cache: " + be_->last_error());
+    argus_hip_quant_cache_drop(h_);
+    h_ = h;
+    return OkStatus();
+  }
 
  private:
-  HipQuantWindowCache() : cap_(nullptr) {}
+  HipQuantWindowCache() = default;
+  Status wrap(int rc) const { return rc == 0 ? OkStatus() : Status::Err(be_->last_error() + " (code " + std::to_string(rc) + ")"); }
   HipBackend *be_ = nullptr;
-  HipQuantAttnBackend cap_;
+  void *h_ = nullptr;
   size_t kv_heads_ = 0, head_dim_ = 0, max_seq_len_ = 0, res_cap_ = 0;
-  uint8_t bits_ = 2;
-  size_t q_tokens_ = 0, res_pos_ = 0, deq_tokens_ = 0;
-  void *res_k_ = nullptr, *res_v_ = nullptr, *qk_ = nullptr, *qv_ = nullptr, *attn_k_ = nullptr, *attn_v_ = nullptr;
 };
 
 // CudaGpuScoreAccumulator twin (engine/src/backend/cuda_pc/gpu_score.rs:72-403): persistent device

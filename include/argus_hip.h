@@ -18,6 +18,7 @@
 #ifndef ARGUS_HIP_H
 #define ARGUS_HIP_H
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -315,6 +316,21 @@ typedef struct argus_hip_quant_flush_args {
 } argus_hip_quant_flush_args;
 int argus_hip_quant_flush(argus_hip_ctx *ctx, const argus_hip_quant_flush_args *args);
 
+/* Bit-width transition of a block stream on the device: the block loop of
+ * QuantizedRecentWindowCache::transition_bits between two quantised widths,
+ * engine/src/kv/quant_window_cache.rs:1308-1372 (each block dequantised to f32 and quantised again
+ * at the new width; the reference reads the streams back, does it on the CPU and uploads the result).
+ * Same blocks bit for bit.  `n_blocks` blocks from src_mem to dst_mem, which must not overlap. */
+typedef struct argus_hip_quant_requant_args {
+  void *stream;
+  uint64_t src_mem;
+  uint64_t dst_mem;
+  size_t n_blocks;
+  uint8_t old_bits; /* 2, 4 or 8 */
+  uint8_t new_bits;
+} argus_hip_quant_requant_args;
+int argus_hip_quant_requant(argus_hip_ctx *ctx, const argus_hip_quant_requant_args *args);
+
 /* Dequantise flushed blocks into the F16 attention view [max_seq, kv_heads, head_dim] (sequence
  * major).  Field-for-field twin of CudaQuantDequantFlushArgs,
  * crates/argus-extension-api/src/lib.rs:3045-3063; CudaQuantAttnBackend::dequant_flush 3096-3099;
@@ -350,6 +366,80 @@ typedef struct argus_hip_quant_scatter_residual_args {
   size_t tok_base;
 } argus_hip_quant_scatter_residual_args;
 int argus_hip_quant_scatter_residual(argus_hip_ctx *ctx, const argus_hip_quant_scatter_residual_args *args);
+
+/* ---- CACHE-category capability: the KIVI container behind the reference's plugin vtable ------
+ * QuantCacheBackend / QuantCacheVTable, crates/argus-extension-api/src/lib.rs:1932-2090: a stateful
+ * per-layer quantised cache (F32 residual ring + the two block streams) with `make`, `current_pos`,
+ * `capacity`, `current_bits`, `update`, `flush_if_full`, `assemble_view`, `get_raw_buffers`,
+ * `transition_bits`, `drop`.  The structs are field-for-field twins of QuantCacheMakeArgs (1932-1955),
+ * QuantCacheUpdateArgs (1957-1970), QuantCacheViewOut (1972-1986) and QuantCacheRawBuffersOut
+ * (1988-2012) with the OpenCL handles replaced by their HIP counterparts, and
+ * argus_hip_quant_cache_vtable lists the functions in QuantCacheVTable's order (2068-2090), so the Rust
+ * side registers `argus_hip_quant_cache_get_vtable()` as the vtable of a BACKEND_CAP_CATEGORY_CACHE
+ * entry.  Behaviour is the GPU mode of QuantizedRecentWindowCache
+ * (engine/src/kv/quant_window_cache.rs:1563-1848, 2518-2562, 741-760, 2248-2475, 1308-1448), every
+ * step on the device.  A handle allocates its ring and streams at `make` (sized for max_seq_len),
+ * the F16 view at the first assemble_view, and new streams at a width transition; nothing else.
+ * Work functions return 0 or a negative ARGUS_HIP_ERR_* (text in argus_hip_last_error of the context
+ * given at make).  Widths 2, 4 and 8; bits = 16 (the unquantised fallback) is refused. */
+#define ARGUS_HIP_VIEW_TOKENS_HEADS_DIM 0u /* ViewLayoutTag::HeadMajor of lib.rs:1917-1926: [tokens, kv_heads, head_dim] */
+typedef struct argus_hip_quant_cache_make_args {
+  void *ctx;              /* cl_ctx slot: the argus_hip_ctx the cache allocates from and launches on */
+  void *device;           /* cl_device_id slot: unused */
+  void *stream;           /* cl_queue slot: the stream of every call of the handle (NULL = default) */
+  const char *build_opts; /* unused */
+  size_t kv_heads;
+  size_t head_dim;      /* multiple of 32 */
+  size_t max_seq_len;
+  size_t residual_size; /* positive multiple of 32 */
+  uint8_t bits;         /* 2, 4 or 8 */
+} argus_hip_quant_cache_make_args;
+typedef struct argus_hip_quant_cache_update_args {
+  void *stream;   /* may be NULL: the handle's stream */
+  void *k_in_mem; /* device F32 [seq_len, kv_heads, head_dim] */
+  void *v_in_mem;
+  size_t seq_len; /* 1 = decode, > 1 = prefill batch */
+} argus_hip_quant_cache_update_args;
+typedef struct argus_hip_quant_cache_view_out {
+  void *k_mem; /* F16 [max_seq_len, kv_heads, head_dim], rows [0, tokens) valid */
+  void *v_mem;
+  size_t tokens;
+  uint32_t layout; /* ARGUS_HIP_VIEW_TOKENS_HEADS_DIM */
+} argus_hip_quant_cache_view_out;
+typedef struct argus_hip_quant_cache_raw_buffers_out {
+  void *qk_mem;
+  void *qv_mem;
+  void *res_k_mem;
+  void *res_v_mem;
+  size_t q_tokens;
+  size_t res_tokens;
+  size_t res_cap;
+  uint8_t bits;
+} argus_hip_quant_cache_raw_buffers_out;
+void *argus_hip_quant_cache_make(const argus_hip_quant_cache_make_args *args); /* NULL on failure */
+size_t argus_hip_quant_cache_current_pos(void *handle);
+size_t argus_hip_quant_cache_capacity(void *handle);
+uint8_t argus_hip_quant_cache_current_bits(void *handle);
+int32_t argus_hip_quant_cache_update(void *handle, const argus_hip_quant_cache_update_args *args);
+int32_t argus_hip_quant_cache_flush_if_full(void *handle);
+int32_t argus_hip_quant_cache_assemble_view(void *handle, argus_hip_quant_cache_view_out *out);
+/* false (out untouched) when there is no native-consumable set: an empty cache. */
+bool argus_hip_quant_cache_get_raw_buffers(void *handle, argus_hip_quant_cache_raw_buffers_out *out);
+int32_t argus_hip_quant_cache_transition_bits(void *handle, uint8_t target_bits);
+void argus_hip_quant_cache_drop(void *handle);
+typedef struct argus_hip_quant_cache_vtable {
+  void *(*make)(const argus_hip_quant_cache_make_args *);
+  size_t (*current_pos)(void *);
+  size_t (*capacity)(void *);
+  uint8_t (*current_bits)(void *);
+  int32_t (*update)(void *, const argus_hip_quant_cache_update_args *);
+  int32_t (*flush_if_full)(void *);
+  int32_t (*assemble_view)(void *, argus_hip_quant_cache_view_out *);
+  bool (*get_raw_buffers)(void *, argus_hip_quant_cache_raw_buffers_out *);
+  int32_t (*transition_bits)(void *, uint8_t);
+  void (*drop)(void *);
+} argus_hip_quant_cache_vtable;
+const argus_hip_quant_cache_vtable *argus_hip_quant_cache_get_vtable(void);
 
 /* ---- (a-6) PFA side channel: prefill attention scores on the device --------------------------
  * Stands in for the host mirror prefill_attention_scores, engine/src/kv/standard_format.rs:

@@ -540,6 +540,19 @@ ORACLE_API int oracle_kivi_dequantize_block(const uint8_t *blk, int bits, float 
   return 0;
 }
 
+/* transition_bits between two quantised widths, quant_window_cache.rs:1350-1362 / 1421-1432:
+ * dequantize_block then push_quantized per block, block order unchanged. */
+ORACLE_API int oracle_kivi_requant(const uint8_t *src, uint8_t *dst, int64_t n_blocks, int old_bits, int new_bits) {
+  if ((old_bits != 2 && old_bits != 4 && old_bits != 8) || (new_bits != 2 && new_bits != 4 && new_bits != 8)) return -1;
+  const int ob = kivi_block_bytes(old_bits), nb = kivi_block_bytes(new_bits);
+  float buf[32];
+  for (int64_t i = 0; i < n_blocks; ++i) {
+    oracle_kivi_dequantize_block(src + i * ob, old_bits, buf);
+    oracle_kivi_quantize_block(buf, new_bits, dst + i * nb);
+  }
+  return 0;
+}
+
 /* ------------------------------------------------------------------------- */
 /* a-3 KIVI container: QuantizedRecentWindowCache CPU path                    */
 /*   update() engine/src/kv/quant_window_cache.rs:2518-2562 (lazy flush: when */

@@ -66,6 +66,7 @@ _prefill = _sig("oracle_prefill_attention", C.c_int, [
     C.c_int, C.c_int, C.c_int, C.c_int])
 _kq = _sig("oracle_kivi_quantize_block", C.c_int, [_f32p, C.c_int, _u8p])
 _kdq = _sig("oracle_kivi_dequantize_block", C.c_int, [_u8p, C.c_int, _f32p])
+_krequant = _sig("oracle_kivi_requant", C.c_int, [_u8p, _u8p, C.c_int64, C.c_int, C.c_int])
 _kbuild = _sig("oracle_kivi_build", C.c_int, [
     _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _u8p, _u8p, _f32p, _f32p,
     C.POINTER(C.c_int), C.POINTER(C.c_int)])
@@ -185,6 +186,17 @@ def kivi_dequantize_block(blk, bits):
     blk = np.ascontiguousarray(blk, np.uint8)
     out = np.zeros(32, np.float32)
     assert _kdq(_p(blk, _u8p), bits, _p(out, _f32p)) == 0
+    return out
+
+
+def kivi_requant(blocks, old_bits, new_bits):
+    """transition_bits between two quantised widths on a uint8 block stream: every block dequantised
+    and quantised again at the new width, order kept (quant_window_cache.rs:1350-1362)."""
+    blocks = np.ascontiguousarray(blocks, np.uint8)
+    n = blocks.size // kivi_block_bytes(old_bits)
+    out = np.zeros(n * kivi_block_bytes(new_bits), np.uint8)
+    if _krequant(_p(blocks, _u8p), _p(out, _u8p), n, old_bits, new_bits) != 0:
+        raise ValueError("oracle kivi_requant: bits %d -> %d" % (old_bits, new_bits))
     return out
 
 

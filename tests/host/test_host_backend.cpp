@@ -443,7 +443,10 @@ static void test_quant_window_cache(HipBackend &be) {
       std::vector<float> rrk(hkv * res_cap * hd, 0.0f), rrv(rrk.size(), 0.0f);
       int qt = 0, rt = 0;
       CHECK(oracle_kivi_build(k.data(), v.data(), (int)n, hkv, hd, res_cap, bits, rqk.data(), rqv.data(), rrk.data(), rrv.data(), &qt, &rt) == 0, "oracle build");
-      const QuantWindowRawBuffers raw = c.get_raw_gpu_buffers();
+      auto raw_r = c.get_raw_gpu_buffers();
+      CHECK(raw_r.ok(), "raw buffers");
+      if (!raw_r.ok()) return;
+      const QuantWindowRawBuffers raw = raw_r.value();
       CHECK(raw.q_tokens == (size_t)qt && raw.res_tokens == (size_t)rt && raw.bits == bits, "q_tokens %zu/%d res_tokens %zu/%d", raw.q_tokens, qt, raw.res_tokens, rt);
       const size_t used = (size_t)qt * hkv * hd / 32 * bb;
       std::vector<uint8_t> gk(used), gv(used);
@@ -497,8 +500,20 @@ static void test_quant_window_cache(HipBackend &be) {
     }
     check_at(total);
     CHECK(!c.update(tokens(dk.p, 0, max_seq), tokens(dv.p, 0, max_seq)).ok(), "overflow refused");
-    c.reset();
-    CHECK(c.current_pos() == 0, "reset");
+    // a width transition keeps the token count and serves attention at the new width
+    const uint8_t other = bits == 4 ? 8 : 4;
+    CHECK(c.transition_bits(other).ok() && c.bits() == other && c.current_pos() == total, "transition_bits");
+    {
+      std::vector<float> got(hq * hd);
+      Tensor tq{dq.p, DType::F32, {hq, hd}, true}, tout{dout.p, DType::F32, {hq, hd}, true};
+      CHECK(c.attention_native(tq, tout, hq, nullptr, 0).ok(), "attention after the transition");
+      be.read_buffer(got.data(), dout.p, got.size() * 4);
+      bool finite = true;
+      for (float x : got) finite = finite && std::isfinite(x);
+      CHECK(finite, "attention after the transition is finite");
+    }
+    CHECK(!c.transition_bits(16).ok(), "bits 16 refused");
+    CHECK(c.reset().ok() && c.current_pos() == 0 && !c.get_raw_gpu_buffers().ok(), "reset");
   }
   printf("[kivi] quant-window container on the device: update / flush / raw buffers / fused attention / F16 view ok (bits 2, 4, 8)\n");
 }

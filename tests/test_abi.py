@@ -37,7 +37,12 @@ def test_struct_layouts_match_header_field_order():
              "argus_hip_quant_dequant_flush_args": A.QuantDequantFlushArgs,
              "argus_hip_quant_scatter_residual_args": A.QuantScatterResidualArgs,
              "argus_hip_score_reduce_args": A.ScoreReduceArgs, "argus_hip_device_info": A.DeviceInfo,
-             "argus_hip_create_opts": A.CreateOpts, "argus_hip_decode_plan": A.DecodePlan}
+             "argus_hip_create_opts": A.CreateOpts, "argus_hip_decode_plan": A.DecodePlan,
+             "argus_hip_quant_requant_args": A.QuantRequantArgs,
+             "argus_hip_quant_cache_make_args": A.QuantCacheMakeArgs,
+             "argus_hip_quant_cache_update_args": A.QuantCacheUpdateArgs,
+             "argus_hip_quant_cache_view_out": A.QuantCacheViewOut,
+             "argus_hip_quant_cache_raw_buffers_out": A.QuantCacheRawBuffersOut}
     for cname, cls in pairs.items():
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), text, re.S).group(1)
         fields = []
@@ -48,6 +53,27 @@ def test_struct_layouts_match_header_field_order():
             for part in decl.split(","):
                 fields.append(re.findall(r"([A-Za-z_][A-Za-z0-9_]*)\s*(?:\[\d+\])?\s*$", part.strip())[0])
         assert fields == [f[0] for f in cls._fields_], cname
+
+
+def test_quant_cache_vtable_lists_the_exports_in_the_reference_order():
+    # QuantCacheVTable, crates/argus-extension-api/src/lib.rs:2068-2090: make, current_pos, capacity,
+    # current_bits, update, flush_if_full, assemble_view, get_raw_buffers, transition_bits, drop
+    import argus_hip as A
+    vt = A.lib.argus_hip_quant_cache_get_vtable().contents
+    order = ["make", "current_pos", "capacity", "current_bits", "update", "flush_if_full", "assemble_view",
+             "get_raw_buffers", "transition_bits", "drop"]
+    assert [f[0] for f in A.QuantCacheVTable._fields_] == order
+    for name in order:
+        fn = getattr(A.lib, "argus_hip_quant_cache_" + name)
+        assert getattr(vt, name) == C.cast(fn, C.c_void_p).value, name
+    # a null handle never crashes
+    null = C.c_void_p()
+    assert A.lib.argus_hip_quant_cache_current_pos(null) == 0 and A.lib.argus_hip_quant_cache_capacity(null) == 0
+    assert A.lib.argus_hip_quant_cache_update(null, None) < 0 and A.lib.argus_hip_quant_cache_flush_if_full(null) < 0
+    assert A.lib.argus_hip_quant_cache_transition_bits(null, 4) < 0
+    assert not A.lib.argus_hip_quant_cache_get_raw_buffers(null, None)
+    assert not A.lib.argus_hip_quant_cache_make(None)
+    A.lib.argus_hip_quant_cache_drop(null)
 
 
 def test_degraded_without_device_or_context():

@@ -308,3 +308,121 @@ def test_f16_view_dequant_flush_and_scatter_bit_exact(bits, hkv, d, R, n):
     assert ctx().quant_scatter_residual(rk, dev_k, hkv, R, d, 0, 0) == 0
     assert ctx().quant_dequant_flush(qk, dev_k, hkv, d, 1, 0, 0, 3, True, check=False) == A.ERR_UNSUPPORTED
     assert ctx().quant_scatter_residual(rk, dev_k, hkv, R, d, R + 1, 0, check=False) == A.ERR_INVALID
+
+
+@pytest.mark.parametrize("old,new", [(8, 4), (4, 2), (8, 2), (2, 4), (2, 8), (4, 8), (8, 8)])
+def test_requant_bit_exact(old, new):
+    # transition_bits between quantised widths on the device (quant_window_cache.rs:1350-1362):
+    # the new stream is the CPU loop's, byte for byte.
+    import torch
+    rng = np.random.default_rng(500 + 10 * old + new)
+    n = 4099
+    src = rng.standard_normal((n, 32)).astype(np.float32)
+    src[::13, 3] *= 30.0
+    src[5] = -1.5                                   # constant block
+    src[6] = np.round(src[6] * 2) / 2               # rounding ties
+    blocks = np.concatenate([O.kivi_quantize_block(src[i], old) for i in range(n)])
+    dst = torch.zeros(n * O.kivi_block_bytes(new), dtype=torch.uint8, device="cuda")
+    ctx().quant_requant(dev(blocks), dst, n, old, new)
+    assert np.array_equal(host(dst), O.kivi_requant(blocks, old, new))
+
+
+def test_requant_argument_errors():
+    import argus_hip as A
+    import torch
+    buf = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    assert ctx().quant_requant(buf, buf[2048:], 10, 3, 4, check=False) == A.ERR_UNSUPPORTED
+    assert ctx().quant_requant(buf, buf[36:], 10, 8, 4, check=False) == A.ERR_INVALID      # overlapping streams
+    assert ctx().quant_requant(buf, buf[2:], 0, 8, 4, check=False) == A.OK                  # nothing to do
+    assert ctx().quant_requant(buf, buf[2050:], 10, 8, 4, check=False) == A.ERR_INVALID     # misaligned
+
+
+class _Raw:
+    """A raw device pointer dressed as a tensor for the ctypes wrappers."""
+
+    def __init__(self, ptr, dtype):
+        self.ptr, self.dtype = ptr, dtype
+
+    def data_ptr(self):
+        return self.ptr or 0
+
+
+def _read_dev(ptr, nbytes):
+    import argus_hip as A
+    out = np.zeros(nbytes, np.uint8)
+    assert A.lib.argus_hip_read_buffer(ctx().handle, None, out.ctypes.data, ptr, nbytes) == 0
+    return out
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_quant_cache_capability_through_the_c_abi(bits):
+    # The container behind the CACHE-category vtable (extension-api lib.rs:1932-2090) driven as the
+    # layer loop drives it: a prefill update that crosses a flush, then a token per step.  Blocks and
+    # residual ring against the CPU container bit for bit; fused attention over the raw buffers and the
+    # F16 view against the oracle; a width transition against the oracle's requantised streams.
+    import argus_hip as A
+    import torch
+    hq, hkv, d, R, max_seq = 8, 2, 128, 64, 400
+    rng = np.random.default_rng(900 + bits)
+    total = 3 * R + 21
+    k = rng.standard_normal((total, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((total, hkv, d)).astype(np.float32)
+    k[:, 1, 9] *= 15.0
+    q = rng.standard_normal((hq, d)).astype(np.float32)
+    kd, vd, qd = dev(k), dev(v), dev(q)
+    assert ctx().quant_cache(hkv, d, max_seq, R, 16) is None           # the unquantised fallback is refused
+    assert ctx().quant_cache(hkv, d, max_seq, 48, bits) is None        # residual_size must be a multiple of 32
+    c = ctx().quant_cache(hkv, d, max_seq, R, bits)
+    assert c is not None and c.current_pos() == 0 and c.capacity() == max_seq and c.current_bits() == bits
+    assert c.get_raw_buffers() is None                                  # empty cache: no native set
+    bb = O.kivi_block_bytes(bits)
+
+    def check_at(n, cur_bits, ref=None):
+        ref = ref or O.kivi_build(k[:n], v[:n], R, cur_bits)
+        assert c.current_pos() == n
+        raw = c.get_raw_buffers()
+        assert raw is not None and (raw.q_tokens, raw.res_tokens, raw.res_cap, raw.bits) == (ref["q_tokens"], ref["res_tokens"], R, cur_bits)
+        used = ref["q_tokens"] * hkv * d // 32 * O.kivi_block_bytes(cur_bits)
+        if used:
+            assert np.array_equal(_read_dev(raw.qk_mem, used), ref["qk"][:used]), "key blocks (n %d)" % n
+            assert np.array_equal(_read_dev(raw.qv_mem, used), ref["qv"][:used]), "value blocks (n %d)" % n
+        ring = _read_dev(raw.res_k_mem, hkv * R * d * 4).view(np.float32).reshape(hkv, R, d)
+        assert np.array_equal(ring[:, :ref["res_tokens"]], ref["res_k"][:, :ref["res_tokens"]])
+        out = torch.empty((hq, d), device="cuda")
+        sh = np.full((hq, n), -1.0, np.float32)
+        ctx().attention_gen_quant(qd, _Raw(raw.qk_mem, torch.uint8), _Raw(raw.qv_mem, torch.uint8), _Raw(raw.res_k_mem, torch.float32),
+                                  _Raw(raw.res_v_mem, torch.float32), out, hkv, raw.q_tokens, raw.res_tokens, raw.res_cap,
+                                  1.0 / np.sqrt(d), cur_bits, scores_host=sh)
+        ro, rs = O.kivi_attention(q, ref, 1.0 / np.sqrt(d), scores=True)
+        check_attention_out(host(out), ro)
+        check_scores(sh, rs)
+        view = c.assemble_view()
+        assert view.tokens == n and view.layout == 0
+        gk = _read_dev(view.k_mem, n * hkv * d * 2).view(np.float16).reshape(n, hkv, d).astype(np.float32)
+        gv = _read_dev(view.v_mem, n * hkv * d * 2).view(np.float16).reshape(n, hkv, d).astype(np.float32)
+        ak, av = O.kivi_assemble_view(ref)
+        assert np.array_equal(gk, ak.astype(np.float16).astype(np.float32)) and np.array_equal(gv, av.astype(np.float16).astype(np.float32))
+        return ref
+
+    c.update(kd[:100], vd[:100])                    # fills the ring, flushes 64, leaves 36
+    check_at(100, bits)
+    for t in range(100, total):
+        c.update(kd[t:t + 1], vd[t:t + 1])
+        if t + 1 in (128, 129, 3 * R):
+            check_at(t + 1, bits)
+    ref = check_at(total, bits)
+    # a full ring is flushed on request, a partly filled one is left alone
+    assert c.flush_if_full() == 0 and c.current_pos() == total and c.get_raw_buffers().res_tokens == ref["res_tokens"]
+    # width transitions: same blocks as the CPU loop, and the cache keeps working at the new width
+    for nb in [b for b in (4, 2, 8) if b != bits]:
+        old = c.current_bits()
+        assert c.transition_bits(nb) == 0 and c.current_bits() == nb
+        ref = dict(ref, qk=O.kivi_requant(ref["qk"], old, nb), qv=O.kivi_requant(ref["qv"], old, nb), bits=nb)
+        check_at(total, nb, ref)
+    assert c.transition_bits(c.current_bits()) == 0                     # no-op
+    assert c.transition_bits(16, check=False) == A.ERR_UNSUPPORTED
+    assert c.update(dev(np.zeros((max_seq, hkv, d), np.float32)), dev(np.zeros((max_seq, hkv, d), np.float32)), check=False) == A.ERR_INVALID
+    c.close()
+    e = ctx().quant_cache(hkv, d, max_seq, R, 8)                        # test_kivi_transition_empty: no tokens, just the format
+    assert e.transition_bits(2) == 0 and e.current_bits() == 2 and e.current_pos() == 0
+    e.close()

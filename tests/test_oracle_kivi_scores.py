@@ -62,6 +62,50 @@ def test_codec_bit_exact_vs_independent_numpy_restatement(bits):
         assert err <= d * 0.5 + (1 << bits) * d * 2 ** -10 + np.abs(src).max() * 2 ** -10 + 1e-6
 
 
+@pytest.mark.parametrize("old,new", [(8, 4), (4, 2), (8, 2), (2, 4), (2, 8), (4, 8), (4, 4)])
+def test_requant_vs_independent_numpy_composition(old, new):
+    # transition_bits between quantised widths (quant_window_cache.rs:1350-1362): dequantise each
+    # block, quantise it again.  Against the independent numpy codec, block by block.
+    rng = np.random.default_rng(40 + 10 * old + new)
+    n = 300
+    src = rng.standard_normal((n, 32)).astype(np.float32)
+    src[::9, 5] *= 20.0
+    src[7] = 3.25                      # constant block: d == 0 survives the transition
+    blocks = np.concatenate([O.kivi_quantize_block(src[i], old) for i in range(n)])
+    got = O.kivi_requant(blocks, old, new)
+    bo, bn = O.kivi_block_bytes(old), O.kivi_block_bytes(new)
+    assert got.size == n * bn
+    for i in range(n):
+        ref = T.kivi_quantize_block(T.kivi_dequantize_block(blocks[i * bo:(i + 1) * bo], old), new)
+        assert np.array_equal(got[i * bn:(i + 1) * bn], ref), i
+    c = got[7 * bn:8 * bn]
+    assert not c[4:].any() and np.all(O.kivi_dequantize_block(c, new) == 3.25)
+    if new >= old:  # widening keeps every value to within the f16 rounding of the new scale and minimum
+        for i in range(0, n, 17):
+            a = O.kivi_dequantize_block(blocks[i * bo:(i + 1) * bo], old)
+            b = O.kivi_dequantize_block(got[i * bn:(i + 1) * bn], new)
+            d = float(got[i * bn:i * bn + 2].view(np.float16)[0])
+            assert np.abs(a - b).max() <= 0.5 * d + (1 << new) * d * 2.0 ** -10 + np.abs(a).max() * 2.0 ** -10 + 1e-6
+
+
+def test_requant_reference_transition_case():
+    # test_kivi_transition_bits_8_to_4_to_2 (quant_window_cache.rs:3325-3389): 64 tokens of
+    # make_input_tensor ramps; Q4 stays close to Q8, Q2 loses more than Q4 did.
+    kv_heads, d = 2, 64
+    ramp = (np.arange(kv_heads * d, dtype=np.float32) * np.float32(0.01)).reshape(kv_heads, d)  # make_input_tensor, :2682-2692
+    k = np.stack([np.float32(i * 0.03) + ramp for i in range(65)])
+    c8 = O.kivi_build(k, k + 10.0, 32, 8)
+    assert c8["q_tokens"] == 64
+    v8, _ = O.kivi_assemble_view(c8)
+    c4 = dict(c8, qk=O.kivi_requant(c8["qk"], 8, 4), qv=O.kivi_requant(c8["qv"], 8, 4), bits=4)
+    v4, _ = O.kivi_assemble_view(c4)
+    c2 = dict(c4, qk=O.kivi_requant(c4["qk"], 4, 2), qv=O.kivi_requant(c4["qv"], 4, 2), bits=2)
+    v2, _ = O.kivi_assemble_view(c2)
+    mse84 = float(np.mean((v8[:64] - v4[:64]) ** 2))
+    mse42 = float(np.mean((v4[:64] - v2[:64]) ** 2))
+    assert mse84 < 1.0 and mse42 < 5.0 and mse42 > mse84
+
+
 def test_codec_round_trip_reference_tolerances():
     # :350-366 KVQ4 i*0.1, max_err range/30+0.02; :399-415 KVQ8 (i-16)*0.5, range/510+0.02;
     # :211-231 Q2 range/6+0.01.
