@@ -44,6 +44,10 @@ EXPORTED_SYMBOLS = [
     "argus_hip_quant_cache_flush_if_full", "argus_hip_quant_cache_assemble_view",
     "argus_hip_quant_cache_get_raw_buffers", "argus_hip_quant_cache_transition_bits",
     "argus_hip_quant_cache_get_vtable",
+    "argus_hip_quant_attn_cap_make", "argus_hip_quant_attn_cap_drop", "argus_hip_quant_attn_cap_has_kernel",
+    "argus_hip_quant_attn_cap_is_nosub_device", "argus_hip_quant_attn_cap_attention_gen_quant",
+    "argus_hip_quant_attn_cap_gather_update_quant", "argus_hip_quant_attn_cap_dequant_flush",
+    "argus_hip_quant_attn_cap_scatter_residual", "argus_hip_quant_attn_get_vtable",
 ]
 
 if not os.path.exists(LIB_PATH):
@@ -173,6 +177,23 @@ class QuantCacheVTable(C.Structure):
                                           "assemble_view", "get_raw_buffers", "transition_bits", "drop")]
 
 
+class QuantAttnMakeArgs(C.Structure):
+    _fields_ = [("cl_ctx", C.c_void_p), ("device", C.c_void_p), ("build_opts", C.c_char_p)]
+
+
+class QuantAttnVTable(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("make", "has_quant_attn_kernel", "is_nosub_device", "attention_gen_quant",
+                                          "gather_update_quant", "dequant_flush", "scatter_residual", "drop")]
+
+
+class BackendCapVTableAbi(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("category", C.c_uint32), ("vtable", C.c_void_p)]
+
+
+class BackendCapExportAbi(C.Structure):
+    _fields_ = [("abi_version", C.c_uint32), ("count", C.c_size_t), ("vtables", C.POINTER(BackendCapVTableAbi))]
+
+
 class QuantScatterResidualArgs(C.Structure):
     _fields_ = [("stream", C.c_void_p), ("res_mem", C.c_uint64), ("attn_mem", C.c_uint64),
                 ("kv_heads", C.c_size_t), ("res_cap", C.c_size_t), ("head_dim", C.c_size_t),
@@ -246,6 +267,22 @@ def _bind():
     for name in EXPORTED_SYMBOLS:
         if name != "argus_hip_last_error":
             getattr(lib, name).restype = C.c_int
+    lib.argus_hip_quant_attn_cap_make.argtypes = [C.POINTER(QuantAttnMakeArgs)]
+    lib.argus_hip_quant_attn_cap_make.restype = vp
+    lib.argus_hip_quant_attn_cap_drop.argtypes = [vp]
+    lib.argus_hip_quant_attn_cap_drop.restype = None
+    lib.argus_hip_quant_attn_cap_has_kernel.argtypes = [vp, C.c_uint8]
+    lib.argus_hip_quant_attn_cap_has_kernel.restype = C.c_bool
+    lib.argus_hip_quant_attn_cap_is_nosub_device.argtypes = [vp]
+    lib.argus_hip_quant_attn_cap_is_nosub_device.restype = C.c_bool
+    lib.argus_hip_quant_attn_cap_attention_gen_quant.argtypes = [vp, C.POINTER(QuantAttnArgs)]
+    lib.argus_hip_quant_attn_cap_gather_update_quant.argtypes = [vp, C.POINTER(QuantGatherArgs)]
+    lib.argus_hip_quant_attn_cap_dequant_flush.argtypes = [vp, C.POINTER(QuantDequantFlushArgs)]
+    lib.argus_hip_quant_attn_cap_scatter_residual.argtypes = [vp, C.POINTER(QuantScatterResidualArgs)]
+    lib.argus_hip_quant_attn_get_vtable.argtypes = []
+    lib.argus_hip_quant_attn_get_vtable.restype = C.POINTER(QuantAttnVTable)
+    lib.register_backend_caps_v2.argtypes = []
+    lib.register_backend_caps_v2.restype = BackendCapExportAbi
     lib.argus_hip_quant_cache_make.restype = vp
     lib.argus_hip_quant_cache_get_vtable.restype = C.POINTER(QuantCacheVTable)
     lib.argus_hip_quant_cache_current_pos.restype = C.c_size_t

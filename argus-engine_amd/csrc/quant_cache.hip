@@ -18,6 +18,7 @@ constexpr size_t kGroup = 32;  // QKKV: tokens per key block, channels per value
 
 struct QuantCache {
   argus_hip_ctx *ctx = nullptr;
+  bool owns_ctx = false;  // made without a context: one of its own, destroyed with the handle
   void *stream = nullptr;
   size_t kv_heads = 0, head_dim = 0, max_seq_len = 0, res_cap = 0;
   uint8_t bits = 0;
@@ -66,8 +67,24 @@ int flush_residual(QuantCache *c, void *stream) {
 }  // namespace
 
 ARGUS_API void *argus_hip_quant_cache_make(const argus_hip_quant_cache_make_args *a) {
-  if (!a || !a->ctx) return nullptr;
+  if (!a) return nullptr;
   argus_hip_ctx *ctx = (argus_hip_ctx *)a->ctx;
+  const bool owns_ctx = ctx == nullptr;
+  if (owns_ctx) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    if (argus_hip_create(device, &ctx) != ARGUS_HIP_OK) return nullptr;
+  }
+  struct CtxGuard {  // a refused make gives the context back
+    argus_hip_ctx *ctx;
+    bool armed;
+    ~CtxGuard() {
+      if (armed) argus_hip_destroy(ctx);
+    }
+  } guard{ctx, owns_ctx};
   // the reference asserts these (quant_window_cache.rs:283-295); bits 16 (the unquantised fallback) has
   // no device form here
   if (a->bits != 2 && a->bits != 4 && a->bits != 8) {
@@ -81,8 +98,8 @@ ARGUS_API void *argus_hip_quant_cache_make(const argus_hip_quant_cache_make_args
     return nullptr;
   }
   QuantCache *c = new (std::nothrow) QuantCache();
-  if (!c) return nullptr;
-  c->ctx = ctx; c->stream = a->stream;
+  if (!c) return nullptr;  // (the guard returns an owned context)
+  c->ctx = ctx; c->owns_ctx = owns_ctx; c->stream = a->stream;
   c->kv_heads = a->kv_heads; c->head_dim = a->head_dim; c->max_seq_len = a->max_seq_len; c->res_cap = a->residual_size; c->bits = a->bits;
   const size_t res_bytes = c->kv_heads * c->res_cap * c->head_dim * sizeof(float);
   const size_t stream_bytes = c->stream_blocks() * c->block_bytes(c->bits);
@@ -92,6 +109,7 @@ ARGUS_API void *argus_hip_quant_cache_make(const argus_hip_quant_cache_make_args
     delete c;
     return nullptr;
   }
+  guard.armed = false;
   return c;
 }
 
@@ -99,6 +117,7 @@ ARGUS_API void argus_hip_quant_cache_drop(void *handle) {
   QuantCache *c = (QuantCache *)handle;
   if (!c) return;
   c->release();
+  if (c->owns_ctx) argus_hip_destroy(c->ctx);
   delete c;
 }
 

@@ -384,7 +384,8 @@ int argus_hip_quant_scatter_residual(argus_hip_ctx *ctx, const argus_hip_quant_s
  * given at make).  Widths 2, 4 and 8; bits = 16 (the unquantised fallback) is refused. */
 #define ARGUS_HIP_VIEW_TOKENS_HEADS_DIM 0u /* ViewLayoutTag::HeadMajor of lib.rs:1917-1926: [tokens, kv_heads, head_dim] */
 typedef struct argus_hip_quant_cache_make_args {
-  void *ctx;              /* cl_ctx slot: the argus_hip_ctx the cache allocates from and launches on */
+  void *ctx;              /* cl_ctx slot: the argus_hip_ctx the cache allocates from and launches on; NULL: a
+                             context of its own on the current device, destroyed with the handle */
   void *device;           /* cl_device_id slot: unused */
   void *stream;           /* cl_queue slot: the stream of every call of the handle (NULL = default) */
   const char *build_opts; /* unused */
@@ -440,6 +441,60 @@ typedef struct argus_hip_quant_cache_vtable {
   void (*drop)(void *);
 } argus_hip_quant_cache_vtable;
 const argus_hip_quant_cache_vtable *argus_hip_quant_cache_get_vtable(void);
+
+/* ---- the reference's dlopen plugin protocol -----------------------------------------------------
+ * A capability plugin is a shared library that exports `register_backend_caps_v2`, returning by
+ * value the envelope BackendCapExportAbi { abi_version, count, vtables } of entries
+ * BackendCapVTableAbi { name, category, vtable } (crates/argus-extension-api/src/lib.rs:1752-1782,
+ * BACKEND_CAP_ABI_VERSION = 2 at 1574, categories ATTENTION = 1 at 1578 and CACHE = 2 at 1914; loaded by
+ * engine/src/capability/dynamic_backend_registry.rs:50-160 and resolved by `--backend-cap <name>`).
+ * This library is such a plugin: it registers the fused dequant + attention capability as
+ * "kivi_hip" (QuantAttnVTable, lib.rs:1726-1746: make, has_quant_attn_kernel, is_nosub_device,
+ * attention_gen_quant, gather_update_quant, dequant_flush, scatter_residual, drop) and the container
+ * above as "kivi_cache_hip".  The ATTENTION handle owns a context on the device that is current when
+ * `make` is called and ignores the OpenCL handles of QuantAttnMakeArgs (lib.rs:1583-1592); the `*_mem`
+ * slots of the argument structs carry HIP device pointers and the `cl_queue` slot the HIP stream, as
+ * in the entry points of the same names above.  A CACHE `make` with a NULL `ctx` slot does the same. */
+#define ARGUS_BACKEND_CAP_ABI_VERSION 2u
+#define ARGUS_BACKEND_CAP_CATEGORY_ATTENTION 1u
+#define ARGUS_BACKEND_CAP_CATEGORY_CACHE 2u
+#define ARGUS_HIP_CAP_NAME_ATTENTION "kivi_hip"
+#define ARGUS_HIP_CAP_NAME_CACHE "kivi_cache_hip"
+typedef struct argus_hip_quant_attn_make_args {
+  void *cl_ctx;
+  void *device;
+  const char *build_opts;
+} argus_hip_quant_attn_make_args;
+typedef struct argus_hip_quant_attn_vtable {
+  void *(*make)(const argus_hip_quant_attn_make_args *);
+  bool (*has_quant_attn_kernel)(void *, uint8_t);
+  bool (*is_nosub_device)(void *);
+  int32_t (*attention_gen_quant)(void *, const argus_hip_quant_attn_args *);
+  int32_t (*gather_update_quant)(void *, const argus_hip_quant_gather_args *);
+  int32_t (*dequant_flush)(void *, const argus_hip_quant_dequant_flush_args *);
+  int32_t (*scatter_residual)(void *, const argus_hip_quant_scatter_residual_args *);
+  void (*drop)(void *);
+} argus_hip_quant_attn_vtable;
+void *argus_hip_quant_attn_cap_make(const argus_hip_quant_attn_make_args *args); /* NULL on failure */
+bool argus_hip_quant_attn_cap_has_kernel(void *handle, uint8_t bits);
+bool argus_hip_quant_attn_cap_is_nosub_device(void *handle);
+int32_t argus_hip_quant_attn_cap_attention_gen_quant(void *handle, const argus_hip_quant_attn_args *args);
+int32_t argus_hip_quant_attn_cap_gather_update_quant(void *handle, const argus_hip_quant_gather_args *args);
+int32_t argus_hip_quant_attn_cap_dequant_flush(void *handle, const argus_hip_quant_dequant_flush_args *args);
+int32_t argus_hip_quant_attn_cap_scatter_residual(void *handle, const argus_hip_quant_scatter_residual_args *args);
+void argus_hip_quant_attn_cap_drop(void *handle);
+const argus_hip_quant_attn_vtable *argus_hip_quant_attn_get_vtable(void);
+typedef struct argus_backend_cap_vtable_abi {
+  const char *name;
+  uint32_t category;
+  const void *vtable;
+} argus_backend_cap_vtable_abi;
+typedef struct argus_backend_cap_export_abi {
+  uint32_t abi_version;
+  size_t count;
+  const argus_backend_cap_vtable_abi *vtables;
+} argus_backend_cap_export_abi;
+argus_backend_cap_export_abi register_backend_caps_v2(void);
 
 /* ---- (a-6) PFA side channel: prefill attention scores on the device --------------------------
  * Stands in for the host mirror prefill_attention_scores, engine/src/kv/standard_format.rs:

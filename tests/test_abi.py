@@ -38,7 +38,8 @@ def test_struct_layouts_match_header_field_order():
              "argus_hip_quant_scatter_residual_args": A.QuantScatterResidualArgs,
              "argus_hip_score_reduce_args": A.ScoreReduceArgs, "argus_hip_device_info": A.DeviceInfo,
              "argus_hip_create_opts": A.CreateOpts, "argus_hip_decode_plan": A.DecodePlan,
-             "argus_hip_quant_requant_args": A.QuantRequantArgs,
+             "argus_hip_quant_requant_args": A.QuantRequantArgs, "argus_hip_quant_attn_make_args": A.QuantAttnMakeArgs,
+             "argus_backend_cap_vtable_abi": A.BackendCapVTableAbi, "argus_backend_cap_export_abi": A.BackendCapExportAbi,
              "argus_hip_quant_cache_make_args": A.QuantCacheMakeArgs,
              "argus_hip_quant_cache_update_args": A.QuantCacheUpdateArgs,
              "argus_hip_quant_cache_view_out": A.QuantCacheViewOut,
@@ -74,6 +75,36 @@ def test_quant_cache_vtable_lists_the_exports_in_the_reference_order():
     assert not A.lib.argus_hip_quant_cache_get_raw_buffers(null, None)
     assert not A.lib.argus_hip_quant_cache_make(None)
     A.lib.argus_hip_quant_cache_drop(null)
+
+
+def test_plugin_envelope_follows_the_reference_dlopen_protocol():
+    # register_backend_caps_v2 -> BackendCapExportAbi { abi_version 2, count, vtables } of
+    # BackendCapVTableAbi { name, category, vtable } (crates/argus-extension-api/src/lib.rs:1569-1578,
+    # 1752-1782; loader engine/src/capability/dynamic_backend_registry.rs:50-160: version check, non-null
+    # vtables, known categories, unique names).
+    import argus_hip as A
+    env = A.lib.register_backend_caps_v2()
+    assert env.abi_version == 2 and env.count == 2 and bool(env.vtables)
+    entries = [env.vtables[i] for i in range(env.count)]
+    assert [(e.name, e.category) for e in entries] == [(b"kivi_hip", 1), (b"kivi_cache_hip", 2)]
+    assert entries[0].vtable == C.cast(A.lib.argus_hip_quant_attn_get_vtable(), C.c_void_p).value
+    assert entries[1].vtable == C.cast(A.lib.argus_hip_quant_cache_get_vtable(), C.c_void_p).value
+    # QuantAttnVTable order, lib.rs:1726-1746
+    vt = A.lib.argus_hip_quant_attn_get_vtable().contents
+    names = {"make": "make", "has_quant_attn_kernel": "has_kernel", "is_nosub_device": "is_nosub_device",
+             "attention_gen_quant": "attention_gen_quant", "gather_update_quant": "gather_update_quant",
+             "dequant_flush": "dequant_flush", "scatter_residual": "scatter_residual", "drop": "drop"}
+    assert [f[0] for f in A.QuantAttnVTable._fields_] == list(names)
+    for field, sym in names.items():
+        assert getattr(vt, field) == C.cast(getattr(A.lib, "argus_hip_quant_attn_cap_" + sym), C.c_void_p).value, field
+    # a degraded (null) handle answers -1 / false without crashing (engine/tests/gate_c_kivi_backend_cap.rs:90-146)
+    null = C.c_void_p()
+    assert not A.lib.argus_hip_quant_attn_cap_has_kernel(null, 2)
+    assert A.lib.argus_hip_quant_attn_cap_attention_gen_quant(null, None) == -1
+    assert A.lib.argus_hip_quant_attn_cap_gather_update_quant(null, None) == -1
+    assert A.lib.argus_hip_quant_attn_cap_dequant_flush(null, None) == -1
+    assert A.lib.argus_hip_quant_attn_cap_scatter_residual(null, None) == -1
+    A.lib.argus_hip_quant_attn_cap_drop(null)
 
 
 def test_degraded_without_device_or_context():

@@ -1,4 +1,6 @@
 """GPU parity: KIVI fused dequant decode, residual append and on-device quantise-at-flush."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -426,3 +428,57 @@ def test_quant_cache_capability_through_the_c_abi(bits):
     e = ctx().quant_cache(hkv, d, max_seq, R, 8)                        # test_kivi_transition_empty: no tokens, just the format
     assert e.transition_bits(2) == 0 and e.current_bits() == 2 and e.current_pos() == 0
     e.close()
+
+
+def test_plugin_protocol_end_to_end():
+    # What engine/src/capability/dynamic_backend_registry.rs does with a capability plugin: dlopen,
+    # register_backend_caps_v2, pick the entries by name, call through the vtables only.  The CACHE
+    # handle builds a cache from tokens on the device, the ATTENTION handle attends over its raw buffers.
+    import argus_hip as A
+    import torch
+    env = A.lib.register_backend_caps_v2()
+    by_name = {env.vtables[i].name: env.vtables[i] for i in range(env.count)}
+    attn = C.cast(by_name[b"kivi_hip"].vtable, C.POINTER(A.QuantAttnVTable)).contents
+    cache = C.cast(by_name[b"kivi_cache_hip"].vtable, C.POINTER(A.QuantCacheVTable)).contents
+    vp = C.c_void_p
+    a_make = C.CFUNCTYPE(vp, C.POINTER(A.QuantAttnMakeArgs))(attn.make)
+    a_has = C.CFUNCTYPE(C.c_bool, vp, C.c_uint8)(attn.has_quant_attn_kernel)
+    a_nosub = C.CFUNCTYPE(C.c_bool, vp)(attn.is_nosub_device)
+    a_attn = C.CFUNCTYPE(C.c_int32, vp, C.POINTER(A.QuantAttnArgs))(attn.attention_gen_quant)
+    a_drop = C.CFUNCTYPE(None, vp)(attn.drop)
+    c_make = C.CFUNCTYPE(vp, C.POINTER(A.QuantCacheMakeArgs))(cache.make)
+    c_update = C.CFUNCTYPE(C.c_int32, vp, C.POINTER(A.QuantCacheUpdateArgs))(cache.update)
+    c_pos = C.CFUNCTYPE(C.c_size_t, vp)(cache.current_pos)
+    c_raw = C.CFUNCTYPE(C.c_bool, vp, C.POINTER(A.QuantCacheRawBuffersOut))(cache.get_raw_buffers)
+    c_drop = C.CFUNCTYPE(None, vp)(cache.drop)
+
+    hq, hkv, d, R, n, bits = 8, 2, 128, 32, 75, 4
+    rng = np.random.default_rng(4242)
+    k = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((n, hkv, d)).astype(np.float32)
+    q = rng.standard_normal((hq, d)).astype(np.float32)
+    kd, vd, qd = dev(k), dev(v), dev(q)
+    stream = torch.cuda.current_stream().cuda_stream
+    ah = a_make(C.byref(A.QuantAttnMakeArgs()))          # the OpenCL handles of the reference are not used
+    assert ah and a_has(ah, 2) and a_has(ah, 4) and a_has(ah, 8) and not a_has(ah, 3) and a_nosub(ah)
+    ch = c_make(C.byref(A.QuantCacheMakeArgs(ctx=None, stream=stream, kv_heads=hkv, head_dim=d, max_seq_len=128, residual_size=R, bits=bits)))
+    assert ch
+    assert c_update(ch, C.byref(A.QuantCacheUpdateArgs(stream=stream, k_in_mem=kd.data_ptr(), v_in_mem=vd.data_ptr(), seq_len=n))) == 0
+    assert c_pos(ch) == n
+    raw = A.QuantCacheRawBuffersOut()
+    assert c_raw(ch, C.byref(raw)) and (raw.q_tokens, raw.res_tokens, raw.bits) == (64, 11, bits)
+    out = torch.empty((hq, d), device="cuda")
+    sh = np.zeros((hq, n), np.float32)
+    args = A.QuantAttnArgs(stream=stream, q_mem=qd.data_ptr(), qk_mem=raw.qk_mem, qv_mem=raw.qv_mem, res_k_mem=raw.res_k_mem,
+                           res_v_mem=raw.res_v_mem, out_mem=out.data_ptr(), scores_out=sh.ctypes.data, scores_len=sh.size,
+                           num_heads_q=hq, num_heads_kv=hkv, head_dim=d, q_tokens=raw.q_tokens, res_tokens=raw.res_tokens,
+                           res_cap=raw.res_cap, scale=1.0 / np.sqrt(d), bits=bits)
+    assert a_attn(ah, C.byref(args)) == 0
+    ref = O.kivi_build(k, v, R, bits)
+    ro, rs = O.kivi_attention(q, ref, 1.0 / np.sqrt(d), scores=True)
+    check_attention_out(host(out), ro)
+    check_scores(sh, rs)
+    args.bits = 3
+    assert a_attn(ah, C.byref(args)) < 0
+    c_drop(ch)
+    a_drop(ah)
