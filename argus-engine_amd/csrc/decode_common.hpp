@@ -417,7 +417,12 @@ inline dim3 combine_grid(const DecodeParams &p, int batch) {
 // step with the device full: rounds x (tile steps per workgroup + 0.75 for set-up, merge and
 // partial write-out).  Sets p.nsplit and p.chunk (a multiple of tile_rows).
 // `max_chunk` > 0: no chunk longer than that many tokens, when the split limit allows it.
-inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slots, int max_chunk = 0) {
+// `second_launch`: what the combine pass costs a plan with more than one split, in the same unit,
+// for launchers whose single-split plan needs no combine (it writes the output itself).  Measured
+// on rows of up to 1024 tokens, one to four sequences: a tile step of a lone workgroup takes about
+// 1 us and the second launch 3.2 us, so rows of up to four tile steps are better served by one
+// workgroup per KV head and a single launch (512 tokens x 4 sequences: 9.4 against 11.8 us per call).
+inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slots, int max_chunk = 0, float second_launch = 0.0f) {
   const int max_splits = std::min((p.len + tile_rows - 1) / tile_rows, kMaxSplits);
   int nsplit = 1, chunk = (p.len + tile_rows - 1) / tile_rows * tile_rows;
   float best = 3.0e38f;
@@ -426,7 +431,7 @@ inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slo
     if (max_chunk > 0 && c > max_chunk && n < max_splits) continue;
     const int ns = (p.len + c - 1) / c;
     const int64_t rounds = ((int64_t)pairs * ns + slots - 1) / slots;
-    const float cost = (float)rounds * ((float)(c / tile_rows) + 0.75f);
+    const float cost = (float)rounds * ((float)(c / tile_rows) + 0.75f) + (ns > 1 ? second_launch : 0.0f);
     if (cost < best) {
       best = cost;
       nsplit = ns;

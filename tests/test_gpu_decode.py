@@ -74,8 +74,10 @@ def test_decode_matrix(hq, hkv, d, L, kv):
     r64, p64 = T.decode_attention(q, k, v, hkv, L)
     check_attention_out(got, r64, "out vs f64")
     # no-scores launch (single-split direct path for short L) gives the same output
+    # (another cut of the row: the probabilities are rounded to f16 against another running maximum)
     got2 = run_decode(q, k, v, hkv, L, cap)
-    assert np.abs(got2 - got).max() < 1e-5
+    assert np.abs(got2 - got).max() < 1e-4
+    check_attention_out(got2, r64, "no-scores out vs f64")
 
 
 def test_seq_major_layout():
