@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void pfa_logits_mfma_kernel(const PfaParams p)
     if (key0 + ln < p.prefix_len) {
 #pragma unroll
       for (int i = 0; i < 16; ++i)
-        if (row_off[i] >= 0) p.logits[(int64_t)row_off[i] + key0 + ln] = __fmul_rn(acc[i], p.scale);
+        if (row_off[i] >= 0) __builtin_nontemporal_store(__fmul_rn(acc[i], p.scale), p.logits + (int64_t)row_off[i] + key0 + ln);
     }
   }
 }
