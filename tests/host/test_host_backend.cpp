@@ -6,6 +6,7 @@
 //   * KIVI residual-only pattern  engine/src/bin/test_cuda_quant_attn_device.rs:108-178 (Test A)
 //   * degraded capability handle  engine/tests/gate_c_kivi_backend_cap.rs:90-146
 // The CPU oracle (test infrastructure) supplies the expected values.
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -570,6 +571,37 @@ static void test_compaction_and_memory(HipBackend &be) {
   printf("[kv] compaction through buffer_shift (layer and per head), write_buffer_range ok\n");
 }
 
+// What one attention_gen call costs a compiled caller (no interpreter in the loop): calls issued back to
+// back on the default stream, wall time per call with one synchronisation at the end.  Printed, not
+// asserted: the figure depends on the host.
+static void report_call_cost(HipBackend &be) {
+  const size_t hq = 32, hkv = 8, d = 128, cap = 4096;
+  if (be.gpu_score_acc()) be.gpu_score_acc()->set_active(false);  // no score slice: the plain decode call
+  std::vector<uint16_t> kv(hkv * cap * d, 0x3c00);  // 1.0
+  std::vector<float> q(hq * d, 0.01f);
+  DevBuf dk(&be, kv.size() * 2, kv.data()), dv(&be, kv.size() * 2, kv.data()), dq(&be, q.size() * 4, q.data()), dout(&be, q.size() * 4);
+  Tensor tq{dq.p, DType::F32, {hq, d}, true}, tout{dout.p, DType::F32, {hq, d}, true};
+  Tensor tk{dk.p, DType::F16, {1, hkv, cap, d}, true}, tv = tk;
+  tv.ptr = dv.p;
+  for (size_t len : {(size_t)512, (size_t)4096}) {
+    auto first = be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, nullptr, 0);
+    CHECK(first.ok(), "attention_gen: %s", first.error().c_str());
+    for (int i = 0; i < 50; ++i) be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, nullptr, 0);
+    be.synchronize();
+    const int n = 2000;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < n; ++i) be.attention_gen(tq, tk, tv, tout, hq, hkv, d, len, nullptr, 0);
+    const auto t1 = std::chrono::steady_clock::now();
+    be.synchronize();
+    const auto t2 = std::chrono::steady_clock::now();
+    argus_hip_decode_plan plan{};
+    argus_hip_last_decode_plan(be.ctx(), &plan);
+    printf("[cost] attention_gen Hq32 Hkv8 d128 L%zu, one sequence, %d launch(es) per call: %.2f us per call to issue, %.2f us per call end to end\n",
+           len, plan.launches, std::chrono::duration<double, std::micro>(t1 - t0).count() / n,
+           std::chrono::duration<double, std::micro>(t2 - t0).count() / n);
+  }
+}
+
 int main() {
   auto r = HipBackend::create(0, 16, 32, 128, 32768);
   if (!r.ok()) {
@@ -586,6 +618,7 @@ int main() {
   test_quant_attn(be);
   test_quant_window_cache(be);
   test_compaction_and_memory(be);
+  report_call_cost(be);
   if (g_fail) {
     printf("%d check(s) FAILED\n", g_fail);
     return 1;
