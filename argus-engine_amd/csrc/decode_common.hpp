@@ -418,10 +418,11 @@ inline dim3 combine_grid(const DecodeParams &p, int batch) {
 // partial write-out).  Sets p.nsplit and p.chunk (a multiple of tile_rows).
 // `max_chunk` > 0: no chunk longer than that many tokens, when the split limit allows it.
 // `second_launch`: what the combine pass costs a plan with more than one split, in the same unit,
-// for launchers whose single-split plan needs no combine (it writes the output itself).  Measured
-// on rows of up to 1024 tokens, one to four sequences: a tile step of a lone workgroup takes about
-// 1 us and the second launch 3.2 us, so rows of up to four tile steps are better served by one
-// workgroup per KV head and a single launch (512 tokens x 4 sequences: 9.4 against 11.8 us per call).
+// for launchers whose single-split plan needs no combine (it writes the output itself).  A lone
+// workgroup walks its tile steps one memory round trip after the other, so the single launch only
+// pays for rows of up to two tile steps: a 32-layer decode loop replayed as a HIP graph, every layer
+// with a cache of its own, takes 250 against 271 us per token at 256 tokens of context with one
+// launch per layer, but 373 against 285 us at 512 tokens (four steps).
 inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slots, int max_chunk = 0, float second_launch = 0.0f) {
   const int max_splits = std::min((p.len + tile_rows - 1) / tile_rows, kMaxSplits);
   int nsplit = 1, chunk = (p.len + tile_rows - 1) / tile_rows * tile_rows;

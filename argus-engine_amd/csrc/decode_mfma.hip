@@ -360,7 +360,7 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
   const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_mfma_kernel<D, TW, false, false>, 64 * kWaves,
                                           max_chunk > 0 ? (size_t)kStageBytes : merge_bytes);
-  choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk, p.scores ? 0.0f : 3.0f);
+  choose_splits(p, pairs, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk, p.scores ? 0.0f : 1.5f);
   p.direct = (p.nsplit == 1 && !p.scores) ? 1 : 0;  // the split pass writes `out` itself: one launch
   p.stage_scores = p.scores && p.chunk <= max_chunk;
   const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);

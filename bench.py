@@ -531,9 +531,9 @@ def main():
         add("cfg3_L4096_b1", bench_decode(ctx, 32, 8, 128, 4096, 1, es, ew, rotate=16), "16 sets rotated")
         add("cfg3_L32768_b16_scores", bench_decode(ctx, 32, 8, 128, 32768, 16, es, ew, scores=True),
             "scores emitted (67 MB of logits per call); combine_us is the pass that rewrites them as probabilities")
-        add("cfg3_L512_b1", bench_decode(ctx, 32, 8, 128, 512, 1, es, ew, rotate=16),
+        add("cfg3_L256_b1", bench_decode(ctx, 32, 8, 128, 256, 1, es, ew, rotate=16),
             "short context: one workgroup per KV head, one launch (no combine pass)")
-        add("cfg3_L512_b16", bench_decode(ctx, 32, 8, 128, 512, 16, es, ew, rotate=4), "short context, 16 sequences: one launch")
+        add("cfg3_L256_b16", bench_decode(ctx, 32, 8, 128, 256, 16, es, ew, rotate=8), "short context, 16 sequences: one launch")
         add("cfg1_qwen_L1024_b1", bench_decode(ctx, 14, 2, 64, 1024, 1, es, ew), "latency-bound (0.5 MiB)")
         add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
             bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=8),
