@@ -426,7 +426,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
                     choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1",
-                             "q8_0", "copy_calib", "aux", "layers", "primary_scores", "cfg5_b64"],
+                             "q8_0", "copy_calib", "aux", "layers", "primary_scores", "cfg5_b64", "prefill_d64_16k"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -466,6 +466,8 @@ def main():
             res = bench_prefill(ctx, args.steps, args.warmup)
         elif w == "prefill_d128":
             res = bench_prefill(ctx, args.steps, args.warmup, hq=32, hkv=8, d=128, s=8192)
+        elif w == "prefill_d64_16k":
+            res = bench_prefill(ctx, args.steps, args.warmup, hq=32, hkv=8, d=64, s=16384)
         elif w in ("q4_0", "q8_0"):
             res = bench_decode_blocks(ctx, w, 32, 8, 128, 32768, 16, args.steps, args.warmup)
         elif w == "q4_0_b1":
