@@ -419,6 +419,18 @@ static int attention_gen_impl(argus_hip_ctx *ctx, const argus_hip_attention_gen_
   const bool want_scores = a->scores_out != nullptr;
   // ARGUS_HIP_DECODE=valu (read when the context is created) keeps the vector-ALU kernel for A/B measurements.
   const bool force_valu = ctx->env.decode_valu;
+  if (blocks && p.len < 64 && (p.row_stride % 32) == 0 && (p.head_stride % 32) == 0) {
+    // A handful of tokens gives the f16 roundings of the matrix-core kernel's weights nothing to
+    // average out against (q2_0 rows of 3 tokens with values near 8: 2.1-2.2e-3 in a seeded sweep,
+    // bar 2e-3); such rows cost nothing either way and take the vector-ALU kernel, which decodes the
+    // same blocks through their descriptor and works in f32, as F16 rows of this length do.
+    p.desc_block_elems = 32;
+    p.desc_bits = kv_dtype == ARGUS_HIP_Q8_0 ? 8 : kv_dtype == ARGUS_HIP_Q2_0 ? 2 : 4;
+    p.desc_scale_layout = (kv_dtype == ARGUS_HIP_Q4_1 || kv_dtype == ARGUS_HIP_Q2_0) ? 2 : 1;  // PerBlockF16WithMin : PerBlockF16
+    p.desc_packing = kv_dtype == ARGUS_HIP_Q8_0 ? 2 : kv_dtype == ARGUS_HIP_Q2_0 ? 3 : 1;     // Byte : Quad : Nibble
+    p.desc_block_bytes = kv_dtype == ARGUS_HIP_Q8_0 ? 34 : kv_dtype == ARGUS_HIP_Q2_0 ? 12 : kv_dtype == ARGUS_HIP_Q4_1 ? 20 : 18;
+    return dispatch_dim<DescRow>(ctx, p, D, a->batch, want_scores, stream);
+  }
   if (blocks) return launch_decode_blocks(ctx, p, D, kv_dtype, a->batch, stream);
   if (!force_valu && decode_mfma_supported(p, D, kv_dtype)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
   switch (kv_dtype) {

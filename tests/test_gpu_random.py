@@ -16,7 +16,8 @@ pytestmark = pytest.mark.gpu
 BLOCK_FORMATS = {"q4_0": O.DESC_Q4_0, "q4_1": O.DESC_Q4_1, "q8_0": O.DESC_Q8_0, "q2_0": O.DESC_Q2_0}
 
 
-@pytest.mark.parametrize("case", range(60))
+# 11332, 11471, 11475: q2_0 rows of three tokens that the matrix-core block kernel put at 2.1-2.2e-3
+@pytest.mark.parametrize("case", list(range(60)) + [11332, 11471, 11475])
 def test_attention_gen_random(case):
     import argus_hip as A
     rng = np.random.default_rng(7_000_000 + case)
