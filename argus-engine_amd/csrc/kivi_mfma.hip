@@ -40,6 +40,7 @@ using namespace argus_decode;
 namespace {
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -215,8 +216,9 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   const uint8_t *qv_b = kp.qv + (int64_t)b * kp.qv_bs;
   const float qscale = p.scale * 1.4426950408889634f * kOpScale;  // log2 domain
 
-  // q of head rh for the slices this lane prepares: slice s -> channels 32*(ra + s*NREP) + 8j + e
-  float qf[NS][8];
+  // q of head rh for the slices this lane prepares: slice s -> channels 32*(ra + s*NREP) + 8j + e,
+  // scaled and split into f16 hi + lo once, as packed pairs (channels e, e + 1)
+  half2_t qh2[NS][4], ql2[NS][4];
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
     const int kk = ra + s * NREP;
@@ -227,7 +229,12 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     for (int e = 0; e < 8; ++e) qv[e] = qp[e];  // the address is clamped
     loaded8(qv);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qf[s][e] = ok ? qv[e] * qscale : 0.0f;
+    for (int e = 0; e < 8; ++e) {
+      _Float16 hi, lo;
+      split_f16(ok ? qv[e] * qscale : 0.0f, hi, lo);
+      qh2[s][e / 2][e % 2] = hi;
+      ql2[s][e / 2][e % 2] = lo;
+    }
   }
 
   const int foff = field_offset<BITS>(r);
@@ -346,16 +353,26 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       const int kk = min(ra + s * NREP, KK - 1);  // qf is zero where the slice does not exist
+      // Two blocks' headers (d | m << 16) at a time, as packed pairs.  With q = qh + ql and d all
+      // f16, hi = rn(qh * d) leaves a remainder qh * d - hi that is itself an f16 number (one fma),
+      // so hi + lo = q * d to the rounding of lo: the ~2^-22 the f32 product split gave, from three
+      // packed instructions per pair instead of two conversions, a product and a split per value.
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t hd = *(const uint32_t *)(sK + (32 * kk + 8 * j + e) * BB);
-        const float dd = (float)__builtin_bit_cast(_Float16, (uint16_t)(hd & 0xffffu));
-        const float mm = (float)__builtin_bit_cast(_Float16, (uint16_t)(hd >> 16));
-        _Float16 hi, lo;
-        split_f16(qf[s][e] * dd, hi, lo);
-        own_h[s][e] = hi;
-        own_l[s][e] = lo;
-        c0 = fmaf(qf[s][e], mm, c0);
+      for (int pr = 0; pr < 4; ++pr) {
+        const uint32_t h0 = *(const uint32_t *)(sK + (32 * kk + 8 * j + 2 * pr) * BB);
+        const uint32_t h1 = *(const uint32_t *)(sK + (32 * kk + 8 * j + 2 * pr + 1) * BB);
+        const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(h1, h0, 0x05040100u));  // [d0, d1]
+        const half2_t mm = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(h1, h0, 0x07060302u));  // [m0, m1]
+        half2_t hi = dd * qh2[s][pr];
+        asm("" : "+v"(hi));  // one rounded value for both uses
+        const half2_t rem = __builtin_elementwise_fma(dd, qh2[s][pr], -hi);
+        const half2_t lo = __builtin_elementwise_fma(dd, ql2[s][pr], rem);
+        own_h[s][2 * pr] = hi[0];
+        own_h[s][2 * pr + 1] = hi[1];
+        own_l[s][2 * pr] = lo[0];
+        own_l[s][2 * pr + 1] = lo[1];
+        c0 = __builtin_amdgcn_fdot2(mm, qh2[s][pr], c0, false);
+        c0 = __builtin_amdgcn_fdot2(mm, ql2[s][pr], c0, false);
       }
     }
     c0 += __shfl_xor(c0, 16, 64);
