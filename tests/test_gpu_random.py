@@ -93,6 +93,10 @@ def test_kivi_attention_random(case):
     out, sc = run_kivi(q, c, scale, scores="dev", res_f16=res_f16)
     check_attention_out(out, ref, what)
     check_scores(sc, p, what)
+    # the same call without scores (what a decode step without an eviction policy issues)
+    plain = run_kivi(q, c, scale, res_f16=res_f16)
+    plain = plain[0] if isinstance(plain, tuple) else plain
+    check_attention_out(plain, ref, what + " (no scores)")
 
 
 # the cases past 40 are F32-cache draws in which one key dominates a row with |v| near 4: they fail
