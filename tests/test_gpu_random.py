@@ -167,3 +167,60 @@ def test_prefill_attention_scores_random(case):
                            per_head, k_f16=k_f16, sum_init=init)
     close(got_s, ref_s)
     close(got_p, ref_p)
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_kv_scatter_random(case):
+    # Backend::kv_scatter_f32_to_f16[_batch] / kv_scatter_f32_batch (engine/src/backend.rs:425-593):
+    # rows [seq, kv_heads, head_dim] F32 into a HeadMajor cache at write_pos, bit for bit (the F16
+    # conversion is round-to-nearest-even), everything else untouched.
+    from gpu_util import ctx
+    rng = np.random.default_rng(12_000_000 + case)
+    hkv = int(rng.choice([1, 2, 3, 4, 8, 16]))
+    d = int(rng.choice([4, 32, 64, 80, 128, 256]))
+    cap = int(rng.choice([1, 7, 64, 129, 1000]))
+    seq = int(rng.integers(0, cap + 1))
+    pos = int(rng.integers(0, cap - seq + 1))
+    to_f16 = bool(rng.integers(0, 2))
+    ks = (rng.standard_normal((seq, hkv, d)) * float(rng.choice([1e-6, 1.0, 300.0, 1e5]))).astype(np.float32)
+    vs = (rng.standard_normal((seq, hkv, d)) * 3).astype(np.float32)
+    dt = np.float16 if to_f16 else np.float32
+    kd = rng.standard_normal((hkv, cap, d)).astype(dt)
+    vd = rng.standard_normal((hkv, cap, d)).astype(dt)
+    dk, dv = dev(kd), dev(vd)
+    what = "Hkv%d d%d cap%d seq%d pos%d f16 %d" % (hkv, d, cap, seq, pos, to_f16)
+    ctx().kv_scatter(dev(ks) if seq else dk, dev(vs) if seq else dv, dk, dv, hkv, d, cap, pos, seq_len=seq)
+    O.kv_scatter(ks, vs, kd, vd, pos)
+    view = np.uint16 if to_f16 else np.uint32
+    assert np.array_equal(host(dk).view(view), kd.view(view)), what
+    assert np.array_equal(host(dv).view(view), vd.view(view)), what
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_score_reduce_random(case):
+    # GpuScoreAccumulator's reduce kernels (engine/src/backend/cuda_pc/kernels.cu:305-360 and the
+    # per-layer form) against the restated CPU loops: decay, head mean, per-KV-head maximum over the
+    # group, maximum over layers; positions past cache_seq_len untouched.
+    from gpu_util import ctx
+    rng = np.random.default_rng(13_000_000 + case)
+    nl = int(rng.choice([1, 2, 5, 28, 33]))
+    hkv = int(rng.choice([1, 2, 4, 8, 16]))
+    hq = hkv * int(rng.choice([1, 2, 4, 7]))
+    L = int(rng.choice([1, 63, 64, 65, 300, 1025, 4000]))
+    stride = L + int(rng.integers(0, 70))
+    decay = float(rng.choice([0.0, 0.5, 0.9, 1.0]))
+    sc = rng.random((nl, hq, stride), dtype=np.float32)
+    imp0 = rng.random(stride, dtype=np.float32)
+    himp0 = rng.random(hkv * stride, dtype=np.float32)
+    lf0 = rng.random(nl * stride, dtype=np.float32)
+    imp, himp, lf = imp0.copy(), himp0.copy(), lf0.copy()
+    O.score_fused_reduce(sc, imp, himp, decay, nl, hq, hkv, L, stride, stride)
+    O.score_reduce_per_layer(sc, lf, decay, nl, hq, L, stride, stride)
+    s, di, dh, dl = dev(sc), dev(imp0), dev(himp0), dev(lf0)
+    ctx().score_reduce(s, di, dh, decay, nl, hq, hkv, L, stride, stride)
+    ctx().score_reduce_per_layer(s, dl, decay, nl, hq, hkv, L, stride, stride)
+    what = "layers%d Hq%d Hkv%d L%d stride%d decay%g" % (nl, hq, hkv, L, stride, decay)
+    assert np.allclose(host(di), imp, rtol=1e-5, atol=1e-7), what
+    assert np.allclose(host(dh), himp, rtol=1e-5, atol=1e-7), what
+    assert np.allclose(host(dl), lf, rtol=1e-5, atol=1e-7), what
+    assert np.array_equal(host(di)[L:], imp0[L:]), what
