@@ -69,6 +69,16 @@ __device__ __forceinline__ half8_t row_shr_into(half8_t v) {
   for (int i = 0; i < 4; ++i) w[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)w[i], (int)w[i], 0x110 + SHIFT, 0xf, BANKS, false);
   return __builtin_bit_cast(half8_t, w);
 }
+// Lanes of the banks (groups of 4 lanes) in BANKS take `src` from the lane the DPP control CTRL
+// names (0x100 + n: lane i + n, 0x110 + n: lane i - n, 0xe4: the lane itself); the rest keep `old`.
+template <int CTRL, int BANKS>
+__device__ __forceinline__ half8_t dpp_merge(half8_t old, half8_t src) {
+  u32x4_t o = __builtin_bit_cast(u32x4_t, old);
+  const u32x4_t w = __builtin_bit_cast(u32x4_t, src);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)o[i], (int)w[i], CTRL, 0xf, BANKS, false);
+  return __builtin_bit_cast(half8_t, o);
+}
 template <int SHIFT>
 __device__ __forceinline__ float row_shl_add(float x) {
   if constexpr (SHIFT > 0 && SHIFT < 16) x += __builtin_bit_cast(float, row_shl<SHIFT>(__builtin_bit_cast(uint32_t, x)));
@@ -240,7 +250,10 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   const int foff = field_offset<BITS>(r);
   const int presh = 6 - 4 * (r & 1);  // Q2 only: the lane's field is the low or the high nibble of its byte
 
-  // o_acc[2cb + sub]: lane (j, n = r) reg i -> head 4j + i, channel 32cb + 2r + sub
+  // o_acc[2cb + sub]: lane (j, n = r) reg i -> accumulator row 4j + i, channel 32cb + 2r + sub.  The
+  // rows GT*a .. GT*a + GT-1 belong to the heads 0 .. GT-1 as seen by the lanes that prepare for slot
+  // a = row / GT: block cb's sums are the ones in the rows of slot cb % NREP (its p*d operand is used
+  // where it was prepared; the other rows of that product are nobody's).
   float4_t o_acc[2 * KK];
   float4_t m_acc = {0.0f, 0.0f, 0.0f, 0.0f};  // zero-point term: lane (j, n = cb) reg i -> head 4j + i
 #pragma unroll
@@ -290,15 +303,19 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         pa[2 * i + w] = (_Float16)pw;
       }
     l_run = l_run * alpha + lsum;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-      float al[4];
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f && r < G) != 0) {  // (lanes past the group hold nobody's maximum)
+      // accumulator row 4j + i: head (4j + i) % GT in the output sums, head 4j + i in the zero-point sums
+      float al_o[4], al_m[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 4 * j + i, 64);
+      for (int i = 0; i < 4; ++i) {
+        al_o[i] = __shfl(alpha, (4 * j + i) % GT, 64);
+        al_m[i] = __shfl(alpha, 4 * j + i, 64);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int a = 0; a < 2 * KK; ++a) o_acc[a][i] *= al[i];
-        m_acc[i] *= al[i];
+        for (int a = 0; a < 2 * KK; ++a) o_acc[a][i] *= al_o[i];
+        m_acc[i] *= al_m[i];
       }
     }
     return pa;
@@ -396,14 +413,25 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
       }
       const half8_t a0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
       const half8_t a1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
-      const half8_t bh = row_shl<(kk % NREP) * GT>(own_h[kk / NREP]);
-      const half8_t bl = row_shl<(kk % NREP) * GT>(own_l[kk / NREP]);
-      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bh, s[0], 0, 0, 0);
-      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bh, s[1], 0, 0, 0);
-      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bl, s[0], 0, 0, 0);
-      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bl, s[1], 0, 0, 0);
+      // Operand columns 0 .. GT-1 take the high halves of the heads' q*d, columns GT .. 2GT-1 the low
+      // halves (the rest of the 16 columns are nobody's), so one MFMA per token set forms both
+      // partial sums; they are added once the slices are through.  The slice was prepared by the
+      // lanes ra*GT .. ra*GT+GT-1 of each row.
+      constexpr int ra_k = kk % NREP;
+      constexpr int kLoBanks = (GT == 4) ? 0x2 : 0xc;
+      constexpr int kLoCtrl = (ra_k == 0) ? 0x110 + GT : (ra_k == 1) ? 0xe4 : 0x100 + (ra_k - 1) * GT;
+      constexpr int kHiBanks = (GT == 4) ? 0x1 : 0x3;
+      half8_t bq;
+      if constexpr (ra_k == 1) bq = dpp_merge<0x100 + GT, kHiBanks>(own_l[kk / NREP], own_h[kk / NREP]);  // the low halves are in place
+      else bq = dpp_merge<kLoCtrl, kLoBanks>(row_shl<ra_k * GT>(own_h[kk / NREP]), own_l[kk / NREP]);
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bq, s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bq, s[1], 0, 0, 0);
     };
     static_for<KK>(qk_slice);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) s[w][i] = row_shl_add<GT>(s[w][i]);  // columns h: high + low
     // undo the field position and the operand units
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -434,7 +462,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     }
     auto pv_block = [&](auto cb_c) {
       constexpr int cb = decltype(cb_c)::value;
-      const half8_t pd = row_shl<(cb % NREP) * GT>(pd_own[cb / NREP]);
+      const half8_t pd = pd_own[cb / NREP];  // real in the rows of slot cb % NREP, where it was prepared
       uint32_t w0[4], w1[4];
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
@@ -513,13 +541,18 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     s[0] *= 1.0f / kOpScale;
     s[1] *= 1.0f / kOpScale;
     const half8_t pa = softmax_step(s, kp.q_tokens + ru * kUnit, n_valid);
+    // every slot's rows take their head's probabilities: whichever rows a block's sums are read from
+    // (see o_acc), the residual tokens are in them
+    half8_t pa_all = pa;
+    if constexpr (GT <= 4) pa_all = row_shr_into<4, 0x2>(pa_all);
+    if constexpr (GT <= 8) pa_all = row_shr_into<8, 0xc>(pa_all);
 #pragma unroll
     for (int cs = 0; cs < 2 * KK; ++cs) {
       half8_t bv;
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         bv[e] = (_Float16)(float)rv[(int64_t)min(8 * j + e, n_valid - 1) * D + 32 * (cs / 2) + 2 * r + (cs & 1)];
-      o_acc[cs] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, bv, o_acc[cs], 0, 0, 0);
+      o_acc[cs] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_all, bv, o_acc[cs], 0, 0, 0);
     }
   };
   for (; u < u_end; u += 4) {
@@ -539,16 +572,17 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     lds_m[wave][r] = m_run;
     lds_l[wave][r] = l_run;
   }
-  if (4 * j < kMaxGroup) {  // accumulator rows 4j + i are heads; only the first kMaxGroup can be real
 #pragma unroll
-    for (int cb = 0; cb < KK; ++cb)
+  for (int cb = 0; cb < KK; ++cb) {
+    if ((4 * j) / GT == cb % NREP) {  // this lane group's accumulator rows are block cb's (see o_acc)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        *(float2 *)&lds_acc[wave][4 * j + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
-    if (r < KK) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
+        *(float2 *)&lds_acc[wave][(4 * j) % GT + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
     }
+  }
+  if (4 * j < kMaxGroup && r < KK) {  // zero-point sums: row 4j + i is head 4j + i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
   }
   __syncthreads();
 
