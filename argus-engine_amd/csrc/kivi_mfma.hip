@@ -17,11 +17,14 @@
 //    field's bit position and the 2^-24 come back as one power-of-two factor on the result.
 //  * One byte (two for Q8) holds the codes of two neighbouring tokens (K) or channels (V).  A lane
 //    owns both: rows 2r and 2r+1 of the logits go to two accumulators fed from the same read.
-//  * The block scales ride on the other operand: q*d in f32, split into f16 hi + lo (the logits
-//    keep ~2^-22 relative accuracy, the 1e-4 bound on emitted scores needs it), and p*d in f16.
-//    Only `group` of the 16 operand columns are real heads, so the q*d work of a unit is spread
-//    over all 16 lanes of a row (each prepares one 32-channel slice for its head) and moved to the
-//    head's lane with a DPP row shift when the slice's MFMA is issued.
+//  * The block scales ride on the other operand: q*d as f16 hi + lo (the logits keep ~2^-22
+//    relative accuracy, the 1e-4 bound on emitted scores needs it), and p*d in f16.  Only `group`
+//    of the 16 operand columns are real heads, so the q*d work of a unit is spread over all 16
+//    lanes of a row (each prepares one 32-channel slice for its head).  When the slice's MFMA is
+//    issued the slice moves to the head's lanes with DPP row shifts, high halves into columns
+//    0 .. GT-1 and low halves into columns GT .. 2GT-1 of one operand, so a single MFMA forms both
+//    partial sums.  The p*d operands of the output sums do not move at all: each block's sums are
+//    read from the accumulator rows of the lanes that prepared its operand.
 //  * The zero-point terms: sum m*q on the vector ALU while the scales are read, sum p*m as one
 //    more MFMA whose operand is the f16 `m` header itself.
 //
