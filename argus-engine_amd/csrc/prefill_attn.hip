@@ -123,7 +123,7 @@ struct PrefillTile {
 // and of the probabilities each move an output by up to ~1e-3 on rows that see a handful of keys
 // (a seeded draw at d 256, 31 keys: 0.9e-3 + 1.1e-3 + 0.6e-3 = 2.06e-3, over the 2e-3 bar).  Those
 // instantiations therefore carry the query as f16 hi + lo and issue the logits MFMAs for both; F16
-// caches (the reference's GPU shape and every BASELINE configuration) are not touched.
+// caches (the reference's GPU shape and every benchmark configuration) are not touched.
 template <typename KV_T>
 constexpr bool kQueryLo = std::is_same<KV_T, float>::value;
 
@@ -542,8 +542,8 @@ int launch(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
   // Two waves per SIMD are needed to overlap anything.  When the grid alone provides them -- two
   // 4-wave workgroups per compute unit -- the workgroups run independently and measure 4-8 % faster
   // (S >= 4096 at Hq32/Hkv8).  Smaller grids get them from two KV groups inside an 8-wave workgroup:
-  // the groups take alternate key tiles of the same query block and merge at the end (BASELINE
-  // config 2: 32.3 us against 33.9 us).  Four groups would need a 128-VGPR cap that spills.
+  // the groups take alternate key tiles of the same query block and merge at the end (the 2K-token, head_dim 64
+  // prefill shape: 32.3 us against 33.9 us).  Four groups would need a 128-VGPR cap that spills.
   const size_t tile_bytes = (size_t)PrefillTile<D>::HALFS * sizeof(_Float16);
   const size_t lds_limit = ctx->props.sharedMemPerBlock;
   if constexpr (D <= 128) {

@@ -11,7 +11,7 @@ resident in HBM.  `value` is algorithmic bytes / wall time of the timed region.
 library on the launch stream around the split-KV kernel of every timed step).
 `cpu_baseline` times the restated reference CPU backend (AVX2+FMA+F16C, one task per Q head) on
 a bounded sample (one of the 16 sequences) on the host cores of the same box.
-`extras` reports the other BASELINE configurations with the same accounting.
+`extras` reports the other benchmark configurations with the same accounting.
 """
 import argparse
 import json
@@ -164,7 +164,7 @@ def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1,
 
 def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res_cap=128, res_f16=False,
                rotate=8, batch=1):
-    """BASELINE config 4: q_tokens = 8064 quantised + 128 residual tokens.  Blocks are synthetic
+    """Benchmark configuration 4: q_tokens = 8064 quantised + 128 residual tokens.  Blocks are synthetic
     (random codes, f16 scale/min headers); `rotate` block sets are cycled.  batch > 1 runs that many
     caches (e.g. the layers of a model) in one launch so the rate is not launch-latency bound."""
     import torch
@@ -204,7 +204,7 @@ def bench_kivi(ctx, bits, steps, warmup, hq=32, hkv=8, d=128, n_tokens=8192, res
 
 
 def bench_prefill(ctx, steps, warmup, hq=32, hkv=8, d=64, s=2048, batch=1, f16_io=True):
-    """BASELINE config 2: causal GQA prefill; FLOPs use the causal count 4*Hq*d*S(S+1)/2."""
+    """Benchmark configuration 2: causal GQA prefill; FLOPs use the causal count 4*Hq*d*S(S+1)/2."""
     import torch
     g = torch.Generator(device="cuda").manual_seed(42)
     io = torch.float16 if f16_io else torch.float32
@@ -226,7 +226,7 @@ def bench_prefill(ctx, steps, warmup, hq=32, hkv=8, d=64, s=2048, batch=1, f16_i
 
 
 def bench_aux(ctx, steps, warmup):
-    """The data-movement kernels either side of the attention calls, each at a size of the BASELINE
+    """The data-movement kernels either side of the attention calls, each at a size of the benchmark
     configurations: microseconds per call (torch events on the current stream, `steps` calls back to
     back) and the rate on the bytes the call has to move."""
     import torch

@@ -73,7 +73,7 @@ def normal(shape, seed, dtype=np.float32):
 
 
 def check_attention_out(got, ref, what=""):
-    """BASELINE tolerance for attention outputs: <= 2e-3 max-abs and <= 1e-3 mean-abs."""
+    """Required tolerance for attention outputs: <= 2e-3 max-abs and <= 1e-3 mean-abs."""
     diff = np.abs(np.asarray(got, np.float64) - np.asarray(ref, np.float64))
     assert np.all(np.isfinite(got)), what
     assert diff.max() <= 2e-3, "%s max-abs %g" % (what, diff.max())
@@ -82,7 +82,7 @@ def check_attention_out(got, ref, what=""):
 
 
 def check_scores(got, ref, what=""):
-    """BASELINE tolerance for H2O score vectors: <= 1e-4 relative (element-wise, with an
+    """Required tolerance for H2O score vectors: <= 1e-4 relative (element-wise, with an
     absolute floor at the f32 underflow scale of a softmax over <= 64K tokens)."""
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)

@@ -269,7 +269,7 @@ def test_index_list_per_sequence_in_a_batch():
 
 
 def test_config1_qwen_shape():
-    # BASELINE config 1: Hq14 Hkv2 d64 L1024, f32 N(0,1) -> F16 KV, scale 1/8.
+    # benchmark configuration 1: Hq14 Hkv2 d64 L1024, f32 N(0,1) -> F16 KV, scale 1/8.
     hq, hkv, d, L = 14, 2, 64, 1024
     q = normal((hq, d), 42)
     k = f16(normal((hkv, L, d), 137))
@@ -324,7 +324,7 @@ def test_config3_batch16_at_32k_properties_and_sampled_parity():
 
 
 def test_config3_batch16_at_4k():
-    # BASELINE config 3 at its shorter length: 16 independent sequences of 4096 tokens in one launch,
+    # benchmark configuration 3 at its shorter length: 16 independent sequences of 4096 tokens in one launch,
     # every one checked against the oracle, with and without scores.
     b, hq, hkv, d, L = 16, 32, 8, 128, 4096
     q = normal((b, hq, d), 42)

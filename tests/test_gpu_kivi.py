@@ -135,8 +135,8 @@ def test_kivi_soft_cap(bits, hq, hkv, d, R, n):
 
 @pytest.mark.parametrize("bits", [4, 8])
 def test_config4_llama8b_kivi(bits):
-    # BASELINE config 4: Hq32 Hkv8 d128, 8192 appended tokens, res_cap 128 -> q_tokens 8064 +
-    # residual 128; N(0,1) with 1% outlier channels x10; residual F32 (ABI) and F16 (BASELINE).
+    # benchmark configuration 4: Hq32 Hkv8 d128, 8192 appended tokens, res_cap 128 -> q_tokens 8064 +
+    # residual 128; N(0,1) with 1% outlier channels x10; residual F32 (ABI) and F16 (the benchmark's).
     hq, hkv, d, n, R = 32, 8, 128, 8192, 128
     rng = np.random.default_rng(4)
     k = rng.standard_normal((n, hkv, d), dtype=np.float32)

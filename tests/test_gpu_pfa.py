@@ -21,7 +21,7 @@ def run_dev(q, k, nq, nkv, d, seq_len, prefix, kps, khs, q_start, q_window, wind
 
 
 def close(got, ref):
-    # BASELINE tolerance for score vectors: 1e-4 relative (the reference's own PFA tests use 1e-4 absolute)
+    # required tolerance for score vectors: 1e-4 relative (the reference's own PFA tests use 1e-4 absolute)
     err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
     assert (err <= 1e-4 * np.abs(ref) + 1e-9).all(), err.max()
 

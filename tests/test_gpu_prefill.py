@@ -83,7 +83,7 @@ def test_prefill_closed_forms():
 
 
 def test_config2_llama1b_shape_all_f16():
-    # BASELINE config 2: Hq32 Hkv8 d64 S2048 batch 1, f16 Q/K/V N(0,1) seeded, f32 accumulate, f16 out.
+    # benchmark configuration 2: Hq32 Hkv8 d64 S2048 batch 1, f16 Q/K/V N(0,1) seeded, f32 accumulate, f16 out.
     s, hq, hkv, d = 2048, 32, 8, 64
     q = f16(normal((1, s, hq, d), 42))
     k = f16(normal((1, hkv, s, d), 137))

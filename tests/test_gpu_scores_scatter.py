@@ -1,4 +1,4 @@
-"""GPU parity: score reduce, KV scatter and the post-eviction + H2O flow (BASELINE config 5)."""
+"""GPU parity: score reduce, KV scatter and the post-eviction + H2O flow (benchmark configuration 5)."""
 import numpy as np
 import pytest
 
@@ -87,7 +87,7 @@ def test_kv_scatter(seq_len, write_pos, to_f16):
 @pytest.mark.parametrize("batch", [1, 8])
 @pytest.mark.parametrize("softcap", [50.0, 0.0])
 def test_config5_post_eviction_h2o_flow(batch, softcap):
-    # BASELINE config 5 (Gemma-2-2B shape): 8192-token history compacted StreamingLLM-style
+    # benchmark configuration 5 (Gemma-2-2B shape): 8192-token history compacted StreamingLLM-style
     # (sink 4 + recent 2044 -> kept positions {0..3} U {6148..8191}, 2048 valid slots) into a
     # capacity-4096 HeadMajor cache; decode with soft-cap 50; per-position probabilities are
     # emitted and reduced to H2O importance.  soft-cap 0 is the reference-CPU-semantics variant.
@@ -128,7 +128,7 @@ def test_config5_post_eviction_h2o_flow(batch, softcap):
 
 @pytest.mark.parametrize("hq,hkv,d,L,cap,softcap", [(8, 4, 256, 3000, 4096, 50.0), (32, 8, 128, 2500, 4096, 0.0)])
 def test_h2o_loop_scores_to_keep_list_to_post_eviction_attention(hq, hkv, d, L, cap, softcap):
-    # The loop BASELINE config 5 feeds, closed on the device: three decode steps emit scores, the fused
+    # The loop benchmark configuration 5 feeds, closed on the device: three decode steps emit scores, the fused
     # reduce accumulates importance (decay 0) and per-KV-head importance, H2O's keep-spec
     # (crates/techniques/h2o/src/lib.rs:138-160: flat, then per head) turns them into keep-lists on
     # the host, and the next decode attends the survivors (a) through kv_index over the untouched

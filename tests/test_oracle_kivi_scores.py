@@ -282,7 +282,7 @@ def test_keep_list_known_answers():
     assert O.streaming_keep(4, 6, 11, 0).tolist() == [0, 1, 2, 3, 5, 6, 7, 8, 9, 10]
     assert O.streaming_keep(4, 6, 20, 7).tolist() == [0, 1, 2, 3, 17, 18, 19]
     assert O.streaming_keep(4, 6, 20, 2).tolist() == [0, 1, 2, 3, 19]
-    # BASELINE config 5: history 8192, sink 4 + recent 2044 -> {0..3} U {6148..8191}
+    # benchmark configuration 5: history 8192, sink 4 + recent 2044 -> {0..3} U {6148..8191}
     k = O.streaming_keep(4, 2044, 8192, 0)
     assert len(k) == 2048 and k[:4].tolist() == [0, 1, 2, 3] and k[4] == 6148 and k[-1] == 8191
 
