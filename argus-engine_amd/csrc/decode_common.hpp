@@ -175,10 +175,29 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   const int slice = ((p.len + (int)gridDim.z - 1) / (int)gridDim.z + 255) / 256 * 256;
   const int t_end = min(p.len, ((int)blockIdx.z + 1) * slice);
   const int t0 = (int)blockIdx.z * slice + (int)threadIdx.x;
+  // Rows that start on a 16-byte boundary are read and written as float4: thread x then owns the
+  // tokens 4 (x + 256 k) .. + 3 of the slice's first 4096 instead of x + 256 k (k < kAhead).
+  const bool vec = p.scores && (((uintptr_t)srow) & 15) == 0;
+  const int s0 = (int)blockIdx.z * slice;
   float logit[kAhead];
   if (p.scores) {
+    if (vec) {
 #pragma unroll
-    for (int k = 0; k < kAhead; ++k) logit[k] = __builtin_nontemporal_load(srow + min(t0 + 256 * k, p.len - 1));
+      for (int k = 0; k < kAhead / 4; ++k) {
+        const int tv = s0 + 4 * ((int)threadIdx.x + 256 * k);
+        if (tv + 3 < p.len) {
+          const float4_t v = __builtin_nontemporal_load((const float4_t *)(srow + tv));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) logit[4 * k + e] = v[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) logit[4 * k + e] = __builtin_nontemporal_load(srow + min(tv + e, p.len - 1));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kAhead; ++k) logit[k] = __builtin_nontemporal_load(srow + min(t0 + 256 * k, p.len - 1));
+    }
   }
   float4_t part[PER];
   if (first) {
@@ -239,10 +258,27 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     }
   }
   if (p.scores) {
+    if (vec) {
 #pragma unroll
-    for (int k = 0; k < kAhead; ++k) {
-      const int t = t0 + 256 * k;
-      if (t < t_end) __builtin_nontemporal_store(__expf(logit[k] - mm) * inv, srow + t);
+      for (int k = 0; k < kAhead / 4; ++k) {
+        const int tv = s0 + 4 * ((int)threadIdx.x + 256 * k);
+        float4_t v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = __expf(logit[4 * k + e] - mm) * inv;
+        if (tv + 3 < t_end) {
+          __builtin_nontemporal_store(v, (float4_t *)(srow + tv));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (tv + e < t_end) __builtin_nontemporal_store(v[e], srow + tv + e);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kAhead; ++k) {
+        const int t = t0 + 256 * k;
+        if (t < t_end) __builtin_nontemporal_store(__expf(logit[k] - mm) * inv, srow + t);
+      }
     }
     for (int t = t0 + 256 * kAhead; t < t_end; t += 256)
       __builtin_nontemporal_store(__expf(__builtin_nontemporal_load(srow + t) - mm) * inv, srow + t);
