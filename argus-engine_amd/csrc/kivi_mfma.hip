@@ -130,8 +130,11 @@ __device__ __forceinline__ void field_pair(uint32_t v, int presh, uint32_t &w0, 
     w0 = v & 0x00ff00ffu;
     w1 = __builtin_amdgcn_perm(v, v, 0x0c030c01u);  // [v.b1, 0, v.b3, 0]
   } else if constexpr (BITS == 4) {
+    // Without PRECISE the second operand is the whole byte, 16 * high nibble + low nibble, still an
+    // exact small integer: its sums minus the low nibbles' sums are 16 times the high nibbles' sums,
+    // taken once at the end (byte_sums_to_high) instead of one more mask per pair here.
     w0 = PRECISE ? ((v << 4) & 0x00f000f0u) : (v & 0x000f000fu);
-    w1 = v & 0x00f000f0u;
+    w1 = PRECISE ? (v & 0x00f000f0u) : v;
   } else if constexpr (PRECISE) {
     v <<= presh;
     w0 = v & 0x00c000c0u;
@@ -189,7 +192,11 @@ constexpr float kCodeUnit = 16777216.0f;  // a raw code field n is the half n * 
 // Query heads per KV head the kernel takes (bounds the merge area).
 constexpr int kMaxGroup = 8;
 
-template <int BITS, int D, int GT, bool SOFTCAP>
+// FASTK (Q4 without scores): the logits take the whole code byte as the operand of the even tokens
+// and subtract the odd tokens' sums afterwards, like the output sums do.  The difference of two f32
+// sums, one of them 17 times the size of the result, keeps ~2^-20 of it: plenty for the outputs (2e-3)
+// and not enough for emitted scores (1e-4 on probabilities), which keep the shifted nibbles.
+template <int BITS, int D, int GT, bool SOFTCAP, bool FASTK>
 __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(const KiviParams kp) {
   constexpr int BB = 4 + 32 * BITS / 8;  // block bytes
   constexpr int KK = D / 32;             // 32-channel slices == V blocks per token
@@ -412,7 +419,14 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
         const uint8_t *cp = sK + (32 * kk + 8 * j + 2 * pr) * BB + foff;
-        field_pair<BITS, true>(field_read2<BITS>(cp, cp + BB), presh, w0[pr], w1[pr]);
+        // (FASTK: w0 = low nibbles in place ... unused; the byte and the high nibbles are the operands)
+        if constexpr (FASTK) {
+          const uint32_t v = field_read2<BITS>(cp, cp + BB);
+          w0[pr] = v;                // 16 * code(2r + 1) + code(2r)
+          w1[pr] = v & 0x00f000f0u;  // 16 * code(2r + 1)
+        } else {
+          field_pair<BITS, true>(field_read2<BITS>(cp, cp + BB), presh, w0[pr], w1[pr]);
+        }
       }
       const half8_t a0 = __builtin_bit_cast(half8_t, u32x4_t{w0[0], w0[1], w0[2], w0[3]});
       const half8_t a1 = __builtin_bit_cast(half8_t, u32x4_t{w1[0], w1[1], w1[2], w1[3]});
@@ -435,12 +449,13 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int w = 0; w < 2; ++w) s[w][i] = row_shl_add<GT>(s[w][i]);  // columns h: high + low
+    if constexpr (FASTK) s[0] -= s[1];  // byte sums -> the even tokens' sums, in units of 2^-24
     // undo the field position and the operand units
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int w = 0; w < 2; ++w)
-        s[w][i] = fmaf(s[w][i], kCodeUnit / (kOpScale * (float)(1 << field_shift<BITS>(w))), c0);
+        s[w][i] = fmaf(s[w][i], kCodeUnit / (kOpScale * (float)(1 << ((FASTK && w == 0) ? 0 : field_shift<BITS>(w)))), c0);
 
     const half8_t pa = softmax_step(s, u * kUnit, kUnit);
 
@@ -490,6 +505,11 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(half8_t, mw), m_acc, 0, 0, 0);
   }
 
+  // Q4: the second accumulator of a block holds the byte sums (see field_pair)
+  if constexpr (BITS == 4) {
+#pragma unroll
+    for (int cb = 0; cb < KK; ++cb) o_acc[2 * cb + 1] -= o_acc[2 * cb];
+  }
   // The code sums carry the field position and the operand units.
   const float v_unit = (BITS == 2) ? (float)(1 << presh) : 1.0f;  // Q2 fields sit 2^-presh below bit 6
 #pragma unroll
@@ -618,8 +638,8 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   const int pairs = p.n_heads_kv * p.head_chunks * batch;
   // One round of co-resident workgroups: a second, partly filled round would run at a fraction of
   // the occupancy the unit loop needs to hide its LDS and HBM latency.
-  const int wgs_per_cu = std::min(argus_wgs_per_cu(ctx, kivi_mfma_kernel<BITS, D, 4, false>, 256, 0),
-                                  argus_wgs_per_cu(ctx, kivi_mfma_kernel<BITS, D, 8, false>, 256, 0));
+  const int wgs_per_cu = std::min(argus_wgs_per_cu(ctx, kivi_mfma_kernel<BITS, D, 4, false, false>, 256, 0),
+                                  argus_wgs_per_cu(ctx, kivi_mfma_kernel<BITS, D, 8, false, false>, 256, 0));
   const int slots = ctx->compute_units * wgs_per_cu;
   const int max_splits = (kp.units_total + 3) / 4;  // at least one unit per wave
   int nsplit = std::max(1, std::min({slots / pairs, max_splits, kMaxSplits}));
@@ -633,10 +653,14 @@ int launch(argus_hip_ctx *ctx, KiviParams &kp, int batch, hipStream_t stream) {
   const dim3 grid(nsplit, p.n_heads_kv * p.head_chunks, batch);
   KernelTimer timer(ctx, stream);
   const bool cap = p.softcap > 0.0f;
-  if (p.group <= 4 && cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, true>), grid, dim3(256), 0, stream, kp);
-  else if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, false>), grid, dim3(256), 0, stream, kp);
-  else if (cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, true>), grid, dim3(256), 0, stream, kp);
-  else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false>), grid, dim3(256), 0, stream, kp);
+  constexpr bool kFast = BITS == 4;
+  const bool fast = kFast && !p.scores;  // (soft-capped calls take the exact form as well)
+  if (p.group <= 4 && cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, true, false>), grid, dim3(256), 0, stream, kp);
+  else if (p.group <= 4 && fast) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, false, kFast>), grid, dim3(256), 0, stream, kp);
+  else if (p.group <= 4) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 4, false, false>), grid, dim3(256), 0, stream, kp);
+  else if (cap) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, true, false>), grid, dim3(256), 0, stream, kp);
+  else if (fast) hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false, kFast>), grid, dim3(256), 0, stream, kp);
+  else hipLaunchKernelGGL((kivi_mfma_kernel<BITS, D, 8, false, false>), grid, dim3(256), 0, stream, kp);
   timer.mark();
   ARGUS_HIP_CHECK(ctx, hipGetLastError());
   hipLaunchKernelGGL((decode_combine_kernel<NoFallback, D>), combine_grid(p, batch), dim3(256), 0, stream, p);
