@@ -64,14 +64,6 @@ __device__ __forceinline__ half8_t row_shl(half8_t v) {
   for (int i = 0; i < 4; ++i) w[i] = row_shl<SHIFT>(w[i]);
   return __builtin_bit_cast(half8_t, w);
 }
-// Lanes of the banks (groups of 4 lanes) in BANKS take the value of lane i - SHIFT; the rest keep theirs.
-template <int SHIFT, int BANKS>
-__device__ __forceinline__ half8_t row_shr_into(half8_t v) {
-  u32x4_t w = __builtin_bit_cast(u32x4_t, v);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)w[i], (int)w[i], 0x110 + SHIFT, 0xf, BANKS, false);
-  return __builtin_bit_cast(half8_t, w);
-}
 // Lanes of the banks (groups of 4 lanes) in BANKS take `src` from the lane the DPP control CTRL
 // names (0x100 + n: lane i + n, 0x110 + n: lane i - n, 0xe4: the lane itself); the rest keep `old`.
 template <int CTRL, int BANKS>
@@ -81,6 +73,26 @@ __device__ __forceinline__ half8_t dpp_merge(half8_t old, half8_t src) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) o[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)o[i], (int)w[i], CTRL, 0xf, BANKS, false);
   return __builtin_bit_cast(half8_t, o);
+}
+// Lanes of the banks in BANKS take `src` as it is; the rest keep `old`.
+template <int BANKS>
+__device__ __forceinline__ float bank_select(float old, float src) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src), 0xe4, 0xf, BANKS, false));
+}
+// Lanes of the banks in BANKS take `src` from the lane the DPP control names; the rest keep `old`.
+template <int CTRL, int BANKS>
+__device__ __forceinline__ uint32_t dpp_merge(uint32_t old, uint32_t src) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, 0xf, BANKS, false);
+}
+// The 16-lane row rotated by SHIFT lanes (used with SHIFT = 8 and with 4 then 8, where the sense
+// of the rotation does not matter).
+template <int SHIFT>
+__device__ __forceinline__ float row_rot(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + SHIFT, 0xf, 0xf, true));
+}
+template <int SHIFT>
+__device__ __forceinline__ float row_shr_add(float x) {
+  return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + SHIFT, 0xf, 0xf, true));
 }
 template <int SHIFT>
 __device__ __forceinline__ float row_shl_add(float x) {
@@ -213,6 +225,8 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   constexpr int SMEM = (4 * WAVE_BYTES > MERGE_BYTES) ? 4 * WAVE_BYTES : MERGE_BYTES;
   constexpr int NREP = 16 / GT;               // lanes of a row that share one head
   constexpr int NS = (KK + NREP - 1) / NREP;  // slices each lane prepares
+  constexpr int CI = 4 / NREP;                // token pairs of a unit whose softmax a lane computes
+  static_assert(GT == 4 || GT == 8, "the lane roles below are written for 4 or 8 heads per row");
   __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM];
 
   const DecodeParams &p = kp.d;
@@ -265,70 +279,91 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   // a = row / GT: block cb's sums are the ones in the rows of slot cb % NREP (its p*d operand is used
   // where it was prepared; the other rows of that product are nobody's).
   float4_t o_acc[2 * KK];
-  float4_t m_acc = {0.0f, 0.0f, 0.0f, 0.0f};  // zero-point term: lane (j, n = cb) reg i -> head 4j + i
+  float4_t m_acc = {0.0f, 0.0f, 0.0f, 0.0f};  // zero-point term: lane (j, n = cb) reg i -> head (4j + i) % GT
 #pragma unroll
   for (int a = 0; a < 2 * KK; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;
 
-  // Online-softmax step for one unit.  In: s[w][i] = logit (log2 units) of token 8j + 2i + w for
-  // head r.  Out: pa[e] = probability of token 8j + e relative to the running maximum.
+  // Online-softmax step for one unit.  The 32 x GT logits of a unit are spread over all 64 lanes: lane
+  // (j, ra, rh) holds, for head rh, the CI token pairs 8j + 2(ra*CI + ii) + w.  In: t[w][ii] = logit
+  // (log2 units).  Out: the probabilities of tokens 8j .. 8j+7 for head rh, relative to the running
+  // maximum, in every lane of the head (row 16j + r of a p operand is head r % GT).
   const float inv_cap = SOFTCAP ? 1.0f / p.softcap : 0.0f;
-  auto softmax_step = [&](float4_t(&s)[2], int tok0, int n_valid) -> half8_t {
+  auto softmax_step = [&](float(&t)[2][CI], int tok0, int n_valid) -> half8_t {
     float mt = kNegInf;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int ii = 0; ii < CI; ++ii)
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
         if constexpr (SOFTCAP) {
           // cap * tanh(logit / cap) on the natural-unit logit, back to log2 units; NaN stays NaN
-          const float sv = s[w][i];
+          const float sv = t[w][ii];
           const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * 1.4426950408889634f;
-          s[w][i] = (sv != sv) ? sv : capped;
+          t[w][ii] = (sv != sv) ? sv : capped;
         }
-        if (8 * j + 2 * i + w >= n_valid) s[w][i] = kNegInf;
-        mt = fmaxf(mt, s[w][i]);  // a NaN logit propagates (the reference kernels have no guard)
+        if (8 * j + 2 * (ra * CI + ii) + w >= n_valid) t[w][ii] = kNegInf;
+        mt = fmaxf(mt, t[w][ii]);  // a NaN logit propagates (the reference kernels have no guard)
       }
-    if (p.scores && r < G) {
-      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(hbase + r) * p.score_stride + tok0 + 8 * j;
+    if (p.scores && rh < G) {
+      float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)(hbase + rh) * p.score_stride + tok0 + 8 * j + 2 * ra * CI;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int ii = 0; ii < CI; ++ii)
 #pragma unroll
         for (int w = 0; w < 2; ++w)
-          if (8 * j + 2 * i + w < n_valid) srow[2 * i + w] = s[w][i] * kLn2;
+          if (8 * j + 2 * (ra * CI + ii) + w < n_valid) srow[2 * ii + w] = t[w][ii] * kLn2;
     }
+    // the head's maximum over its lanes: the other banks of the row, then the other rows
+    if constexpr (NREP >= 4) mt = fmaxf(mt, row_rot<GT>(mt));
+    mt = fmaxf(mt, row_rot<8>(mt));
     mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = fmaxf(m_run, mt);
     const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
     m_run = m_new;
-    half8_t pa;
-    float lsum = 0.0f;  // f32 sum: the emitted probabilities are normalised by it
+    uint32_t own[CI];
+    float lsum = 0.0f;  // f32 sum of this lane's tokens: the emitted probabilities are normalised by it
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int ii = 0; ii < CI; ++ii) {
+      half2_t pw;
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
-        const float pw = __builtin_amdgcn_exp2f(s[w][i] - m_ref);  // NaN stays NaN
-        lsum += pw;
-        pa[2 * i + w] = (_Float16)pw;
+        const float e = __builtin_amdgcn_exp2f(t[w][ii] - m_ref);  // NaN stays NaN
+        lsum += e;
+        pw[w] = (_Float16)e;
       }
+      own[ii] = __builtin_bit_cast(uint32_t, pw);  // token pair ra*CI + ii
+    }
     l_run = l_run * alpha + lsum;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f && r < G) != 0) {  // (lanes past the group hold nobody's maximum)
-      // accumulator row 4j + i: head (4j + i) % GT in the output sums, head 4j + i in the zero-point sums
-      float al_o[4], al_m[4];
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f && rh < G) != 0) {  // (lanes past the group hold nobody's maximum)
+      // accumulator row 4j + i belongs to head (4j + i) % GT
+      float al[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        al_o[i] = __shfl(alpha, (4 * j + i) % GT, 64);
-        al_m[i] = __shfl(alpha, 4 * j + i, 64);
-      }
+      for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, (4 * j + i) % GT, 64);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int a = 0; a < 2 * KK; ++a) o_acc[a][i] *= al_o[i];
-        m_acc[i] *= al_m[i];
+        for (int a = 0; a < 2 * KK; ++a) o_acc[a][i] *= al[i];
+        m_acc[i] *= al[i];
       }
     }
-    return pa;
+    // every lane of the head collects the four token pairs
+    u32x4_t pa;
+    if constexpr (GT == 8) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        pa[ii] = dpp_merge<0x110 + 8, 0xc>(own[ii], own[ii]);      // lanes 8..15 take pair ii from lanes 0..7
+        pa[2 + ii] = dpp_merge<0x100 + 8, 0x3>(own[ii], own[ii]);  // lanes 0..7 take pair 2 + ii from lanes 8..15
+      }
+    } else {
+      const uint32_t ev = dpp_merge<0x110 + 4, 0xa>(own[0], own[0]);  // pair 0 in banks 0, 1; pair 2 in banks 2, 3
+      const uint32_t od = dpp_merge<0x100 + 4, 0x5>(own[0], own[0]);  // pair 1 in banks 0, 1; pair 3 in banks 2, 3
+      pa[0] = dpp_merge<0x110 + 8, 0xc>(ev, ev);
+      pa[2] = dpp_merge<0x100 + 8, 0x3>(ev, ev);
+      pa[1] = dpp_merge<0x110 + 8, 0xc>(od, od);
+      pa[3] = dpp_merge<0x100 + 8, 0x3>(od, od);
+    }
+    return __builtin_bit_cast(half8_t, pa);
   };
 
   const int u_begin = split * kp.units_per_split;
@@ -404,11 +439,9 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     }
     c0 += __shfl_xor(c0, 16, 64);
     c0 += __shfl_xor(c0, 32, 64);
-    if constexpr (NREP >= 16) c0 = row_shl_add<8 * GT>(c0);
-    if constexpr (NREP >= 8) c0 = row_shl_add<4 * GT>(c0);
-    if constexpr (NREP >= 4) c0 = row_shl_add<2 * GT>(c0);
-    if constexpr (NREP >= 2) c0 = row_shl_add<GT>(c0);
-    c0 *= 1.0f / kOpScale;  // lanes r < GT now hold sum_ch m[ch] q[r][ch]
+    if constexpr (NREP >= 4) c0 += row_rot<GT>(c0);
+    c0 += row_rot<8>(c0);
+    c0 *= 1.0f / kOpScale;  // every lane now holds sum_ch m[ch] q[rh][ch]
 
     // ---- logits: rows m = r -> tokens 2r (s[0]) and 2r + 1 (s[1]) ----------------------------------
     float4_t s[2];
@@ -445,26 +478,40 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
       s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bq, s[1], 0, 0, 0);
     };
     static_for<KK>(qk_slice);
+    // Column h plus column GT + h is head h's sum; token pair i of it goes to the lanes (ra, rh) =
+    // (i / CI, h), so that the softmax below is computed once per logit instead of once per column.
+    float t[2][CI];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int w = 0; w < 2; ++w) {
+      if constexpr (GT == 8) {
 #pragma unroll
-      for (int w = 0; w < 2; ++w) s[w][i] = row_shl_add<GT>(s[w][i]);  // columns h: high + low
-    if constexpr (FASTK) s[0] -= s[1];  // byte sums -> the even tokens' sums, in units of 2^-24
-    // undo the field position and the operand units
+        for (int ii = 0; ii < 2; ++ii)
+          t[w][ii] = bank_select<0xc>(row_shl_add<8>(s[w][ii]), row_shr_add<8>(s[w][2 + ii]));
+      } else {
+        float y[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) y[i] = row_shl_add<4>(s[w][i]);  // lanes 0..3: the heads' sums
+        uint32_t x = __builtin_bit_cast(uint32_t, y[0]);
+        x = dpp_merge<0x110 + 4, 0x2>(x, __builtin_bit_cast(uint32_t, y[1]));
+        x = dpp_merge<0x110 + 8, 0x4>(x, __builtin_bit_cast(uint32_t, y[2]));
+        x = dpp_merge<0x110 + 12, 0x8>(x, __builtin_bit_cast(uint32_t, y[3]));
+        t[w][0] = __builtin_bit_cast(float, x);
+      }
+    }
+#pragma unroll
+    for (int ii = 0; ii < CI; ++ii) {
+      if constexpr (FASTK) t[0][ii] -= t[1][ii];  // byte sums -> the even tokens' sums, in units of 2^-24
+      // undo the field position and the operand units
 #pragma unroll
       for (int w = 0; w < 2; ++w)
-        s[w][i] = fmaf(s[w][i], kCodeUnit / (kOpScale * (float)(1 << ((FASTK && w == 0) ? 0 : field_shift<BITS>(w)))), c0);
+        t[w][ii] = fmaf(t[w][ii], kCodeUnit / (kOpScale * (float)(1 << ((FASTK && w == 0) ? 0 : field_shift<BITS>(w)))), c0);
+    }
 
-    const half8_t pa = softmax_step(s, u * kUnit, kUnit);
+    const half8_t pa_all = softmax_step(t, u * kUnit, kUnit);
 
     // ---- output: contraction slot e -> token 8j + e -------------------------------------------------
-    // Like q*d, the p*d operand only has `group` real rows: every lane of the row gets its head's
-    // probabilities, scales them for the V blocks it owns, and hands the result to the head's lane.
-    half8_t pa_all = pa;
-    if constexpr (GT <= 4) pa_all = row_shr_into<4, 0x2>(pa_all);
-    if constexpr (GT <= 8) pa_all = row_shr_into<8, 0xc>(pa_all);
+    // Like q*d, the p*d operand only has `group` real rows: every lane of the row has its head's
+    // probabilities and scales them for the V blocks it owns.
     const half8_t pa_s = pa_all * (_Float16)kOpScale;
     half8_t pd_own[NS];
 #pragma unroll
@@ -502,7 +549,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         mw[pr] = half_read2(mp, mp + KK * BB);
       }
     }
-    m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(half8_t, mw), m_acc, 0, 0, 0);
+    m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_all, __builtin_bit_cast(half8_t, mw), m_acc, 0, 0, 0);
   }
 
   // Q4: the second accumulator of a block holds the byte sums (see field_pair)
@@ -526,7 +573,8 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     const int64_t rbase = (int64_t)b * kp.res_bs + (int64_t)kvh * kp.res_cap * D + (int64_t)ru * kUnit * D;
     const RES_T *rk = (const RES_T *)kp.res_k + rbase;
     const RES_T *rv = (const RES_T *)kp.res_v + rbase;
-    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(hbase + min(r, G - 1)) * D + 8 * j;
+    // operand column r carries head r % GT: every bank of the row gets the head's logits
+    const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)(hbase + min(rh, G - 1)) * D + 8 * j;
     float4_t s[2];
     s[0] = s[1] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -539,7 +587,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         _Float16 hi, lo;
-        split_f16((r < G) ? qv[e] * qscale : 0.0f, hi, lo);
+        split_f16((rh < G) ? qv[e] * qscale : 0.0f, hi, lo);
         qh[e] = hi;
         ql[e] = lo;
       }
@@ -561,14 +609,20 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         s[w] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, qh, s[w], 0, 0, 0);
       }
     }
-    s[0] *= 1.0f / kOpScale;
-    s[1] *= 1.0f / kOpScale;
-    const half8_t pa = softmax_step(s, kp.q_tokens + ru * kUnit, n_valid);
-    // every slot's rows take their head's probabilities: whichever rows a block's sums are read from
+    // bank ra keeps its token pairs
+    float t[2][CI];
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      if constexpr (GT == 8) {
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) t[w][ii] = bank_select<0xc>(s[w][ii], s[w][2 + ii]) * (1.0f / kOpScale);
+      } else {
+        t[w][0] = bank_select<0x8>(bank_select<0x4>(bank_select<0x2>(s[w][0], s[w][1]), s[w][2]), s[w][3]) * (1.0f / kOpScale);
+      }
+    }
+    // every slot's rows hold their head's probabilities: whichever rows a block's sums are read from
     // (see o_acc), the residual tokens are in them
-    half8_t pa_all = pa;
-    if constexpr (GT <= 4) pa_all = row_shr_into<4, 0x2>(pa_all);
-    if constexpr (GT <= 8) pa_all = row_shr_into<8, 0xc>(pa_all);
+    const half8_t pa_all = softmax_step(t, kp.q_tokens + ru * kUnit, n_valid);
 #pragma unroll
     for (int cs = 0; cs < 2 * KK; ++cs) {
       half8_t bv;
@@ -586,6 +640,8 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   // ---- merge: lane groups (row sum), then the 4 waves through LDS --------------------------------
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
+  if constexpr (NREP >= 4) l_run = row_shl_add<2 * GT>(l_run);
+  l_run = row_shl_add<GT>(l_run);  // lanes r < GT: the head's sum over the banks
   __syncthreads();  // every wave is done with its tile region
   float(*lds_acc)[kMaxGroup][D + 4] = (float(*)[kMaxGroup][D + 4]) smem;
   float(*lds_mt)[kMaxGroup][KK] = (float(*)[kMaxGroup][KK])(smem + 4 * kMaxGroup * (D + 4) * 4);
@@ -603,7 +659,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         *(float2 *)&lds_acc[wave][(4 * j) % GT + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
     }
   }
-  if (4 * j < kMaxGroup && r < KK) {  // zero-point sums: row 4j + i is head 4j + i
+  if (4 * j < GT && r < KK) {  // zero-point sums: row 4j + i < GT is head 4j + i
 #pragma unroll
     for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
   }
