@@ -226,6 +226,10 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   constexpr int NREP = 16 / GT;               // lanes of a row that share one head
   constexpr int NS = (KK + NREP - 1) / NREP;  // slices each lane prepares
   constexpr int CI = 4 / NREP;                // token pairs of a unit whose softmax a lane computes
+  // Where a lane prepares a single V block, its headers are read whole (scale and zero point in one
+  // word) and the lane's column collects that block's zero-point sum; with more blocks per lane,
+  // picking the zero points for the column costs more than reading them again.
+  constexpr bool kHeaderWords = NS == 1;
   static_assert(GT == 4 || GT == 8, "the lane roles below are written for 4 or 8 heads per row");
   __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM];
 
@@ -514,6 +518,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     // probabilities and scales them for the V blocks it owns.
     const half8_t pa_s = pa_all * (_Float16)kOpScale;
     half8_t pd_own[NS];
+    u32x4_t mw = {0u, 0u, 0u, 0u};  // zero points of the block whose sum this lane's column collects
 #pragma unroll
     for (int s2 = 0; s2 < NS; ++s2) {
       const int cb = min(ra + s2 * NREP, KK - 1);
@@ -521,7 +526,14 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
         const uint8_t *dp = sVj + (2 * pr * KK + cb) * BB;
-        dw[pr] = half_read2(dp, dp + KK * BB);
+        if constexpr (kHeaderWords) {
+          // whole headers (d | m << 16) of two tokens, like the K blocks' above
+          const uint32_t h0 = *(const uint32_t *)dp, h1 = *(const uint32_t *)(dp + KK * BB);
+          dw[pr] = __builtin_amdgcn_perm(h1, h0, 0x05040100u);
+          mw[pr] = __builtin_amdgcn_perm(h1, h0, 0x07060302u);
+        } else {
+          dw[pr] = half_read2(dp, dp + KK * BB);
+        }
       }
       pd_own[s2] = pa_s * __builtin_bit_cast(half8_t, dw);  // p * d[token][cb]
     }
@@ -540,13 +552,15 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
       o_acc[2 * cb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pd, b1, o_acc[2 * cb + 1], 0, 0, 0);
     };
     static_for<KK>(pv_block);
-    // zero-point term: column n = cb holds sum_t p[h][t] m[t][cb]
-    u32x4_t mw = {0u, 0u, 0u, 0u};
-    if (r < KK) {
+    // zero-point term: sum_t p[h][t] m[t][cb], in column n = cb, or with whole-header reads in the
+    // columns of the lanes ra = cb, which had block cb's headers anyway
+    if constexpr (!kHeaderWords) {
+      if (r < KK) {
 #pragma unroll
-      for (int pr = 0; pr < 4; ++pr) {
-        const uint8_t *mp = sVj + (2 * pr * KK + r) * BB + 2;
-        mw[pr] = half_read2(mp, mp + KK * BB);
+        for (int pr = 0; pr < 4; ++pr) {
+          const uint8_t *mp = sVj + (2 * pr * KK + r) * BB + 2;
+          mw[pr] = half_read2(mp, mp + KK * BB);
+        }
       }
     }
     m_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_all, __builtin_bit_cast(half8_t, mw), m_acc, 0, 0, 0);
@@ -659,9 +673,11 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         *(float2 *)&lds_acc[wave][(4 * j) % GT + i][32 * cb + 2 * r] = make_float2(o_acc[2 * cb][i], o_acc[2 * cb + 1][i]);
     }
   }
-  if (4 * j < GT && r < KK) {  // zero-point sums: row 4j + i < GT is head 4j + i
+  // zero-point sums: row 4j + i < GT is head 4j + i, the column depends on how the headers were read
+  const int m_cb = kHeaderWords ? ra : r;
+  if (4 * j < GT && m_cb < KK && (!kHeaderWords || rh == 0)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][r] = m_acc[i];
+    for (int i = 0; i < 4; ++i) lds_mt[wave][4 * j + i][m_cb] = m_acc[i];
   }
   __syncthreads();
 
