@@ -90,6 +90,23 @@ template <int SHIFT>
 __device__ __forceinline__ float row_rot(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + SHIFT, 0xf, 0xf, true));
 }
+// op over the four 16-lane rows of the wave, result in every row: the row swaps of this target
+// exchange odd and even rows (then the wave's halves) of two registers without going through LDS.
+// (SWAP false: through LDS permutes, which measured 3-4 % faster for the 2-bit kernels at head_dim
+// 64 and 128 and 1-4 % slower everywhere else.)
+template <bool SWAP, typename OP>
+__device__ __forceinline__ float reduce_rows(float x, OP op) {
+  if constexpr (!SWAP) {
+    x = op(x, __shfl_xor(x, 16, 64));
+    return op(x, __shfl_xor(x, 32, 64));
+  }
+  const uint32_t b0 = __builtin_bit_cast(uint32_t, x);
+  const auto s16 = __builtin_amdgcn_permlane16_swap(b0, b0, false, false);
+  x = op(__builtin_bit_cast(float, (uint32_t)s16[0]), __builtin_bit_cast(float, (uint32_t)s16[1]));
+  const uint32_t b1 = __builtin_bit_cast(uint32_t, x);
+  const auto s32 = __builtin_amdgcn_permlane32_swap(b1, b1, false, false);
+  return op(__builtin_bit_cast(float, (uint32_t)s32[0]), __builtin_bit_cast(float, (uint32_t)s32[1]));
+}
 template <int SHIFT>
 __device__ __forceinline__ float row_shr_add(float x) {
   return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + SHIFT, 0xf, 0xf, true));
@@ -230,6 +247,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   // word) and the lane's column collects that block's zero-point sum; with more blocks per lane,
   // picking the zero points for the column costs more than reading them again.
   constexpr bool kHeaderWords = NS == 1;
+  constexpr bool kRowSwap = BITS != 2;
   static_assert(GT == 4 || GT == 8, "the lane roles below are written for 4 or 8 heads per row");
   __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM];
 
@@ -319,8 +337,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     // the head's maximum over its lanes: the other banks of the row, then the other rows
     if constexpr (NREP >= 4) mt = fmaxf(mt, row_rot<GT>(mt));
     mt = fmaxf(mt, row_rot<8>(mt));
-    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    mt = reduce_rows<kRowSwap>(mt, [](float a, float b) { return fmaxf(a, b); });
     const float m_new = fmaxf(m_run, mt);
     const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
@@ -441,8 +458,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
         c0 = __builtin_amdgcn_fdot2(mm, ql2[s][pr], c0, false);
       }
     }
-    c0 += __shfl_xor(c0, 16, 64);
-    c0 += __shfl_xor(c0, 32, 64);
+    c0 = reduce_rows<kRowSwap>(c0, [](float a, float b) { return a + b; });
     if constexpr (NREP >= 4) c0 += row_rot<GT>(c0);
     c0 += row_rot<8>(c0);
     c0 *= 1.0f / kOpScale;  // every lane now holds sum_ch m[ch] q[rh][ch]
