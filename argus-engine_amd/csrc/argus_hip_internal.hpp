@@ -143,6 +143,27 @@ __device__ __forceinline__ float dpp_mov(float x) {
       float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
 }
 
+// Lane i's value paired with that of lane i ^ 16 / i ^ 32 without an LDS round trip: the row swaps
+// of this target exchange the odd 16-lane rows of one register with the even rows of another
+// (v_permlane16_swap), or the wave's halves (v_permlane32_swap); started from two copies of x, the
+// two results hold x of the lower and of the upper partner in every lane.
+template <typename OP>
+__device__ __forceinline__ float xor16_combine(float x, OP op) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, x);
+  const auto sw = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  return op(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
+}
+template <typename OP>
+__device__ __forceinline__ float xor32_combine(float x, OP op) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, x);
+  const auto sw = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return op(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
+}
+__device__ __forceinline__ float rows_allreduce_max(float x) {  // over lanes i, i^16, i^32, i^48
+  const auto mx = [](float a, float b) { return fmaxf(a, b); };
+  return xor32_combine(xor16_combine(x, mx), mx);
+}
+
 // All-reduce (sum) over aligned groups of LANES consecutive lanes; every lane gets the total.
 template <int LANES>
 __device__ __forceinline__ float group_allreduce_sum(float x) {

@@ -669,8 +669,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     base_last = base;
 
     // ---- online softmax: the running max of a head is shared by the four lane groups -----------
-    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    mt = rows_allreduce_max(mt);
     const float m_new = fmaxf(m_run, mt);
     const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);

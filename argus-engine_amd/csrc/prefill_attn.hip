@@ -339,7 +339,7 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64)) * p.scale_log2e;
+    mt = xor32_combine(mt, [](float a, float b) { return fmaxf(a, b); }) * p.scale_log2e;
     const float m_new = (mt > m_run + kLazy) ? mt : m_run;  // also takes the first finite maximum
     TileMax t;
     t.m_ref = (m_new == kNegInf) ? 0.0f : m_new;
