@@ -550,6 +550,8 @@ def main():
             "32 caches (sequences) per launch, 365 MB: amortised rate")
         add("cfg4_kivi_q8_x32_caches", bench_kivi(ctx, 8, es, ew, batch=32, rotate=2),
             "32 caches (sequences) per launch, 629 MB: amortised rate")
+        add("kivi_q4_d64_Hq32_Hkv8_x32_caches", bench_kivi(ctx, 4, es, ew, hq=32, hkv=8, d=64, batch=32, rotate=2),
+            "head_dim 64 (Llama-3.2-1B head shape), 32 caches per launch, 183 MB")
         add("cfg3_q4_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q4_0 rows attended in-kernel, 604 MB of blocks")
         add("cfg3_q4_0_blocks_L32768_b16_scores", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew, scores=True),
