@@ -368,7 +368,26 @@ struct BlockShape {
 // q8_0 would spill there and stays at 2), 2 at 256.  Without the bound most instantiations came out a
 // few registers on one or the other side of a step depending on unrelated edits (q4_0 at 128: 165 or
 // 170 registers; q8_0 at 256: 256 or 257).
-template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED>
+// Row (16 lanes) i of the wave takes v[i].
+__device__ __forceinline__ float row_pick(const float4_t &v) {
+  // The elements are copied out as floats first: __builtin_bit_cast applied to a vector element
+  // directly read element 0 whatever the index.
+  const float f0 = v[0], f1 = v[1], f2 = v[2], f3 = v[3];
+  int x = __builtin_bit_cast(int, f0);
+  x = __builtin_amdgcn_update_dpp(x, __builtin_bit_cast(int, f1), 0xe4, 0x2, 0xf, false);
+  x = __builtin_amdgcn_update_dpp(x, __builtin_bit_cast(int, f2), 0xe4, 0x4, 0xf, false);
+  x = __builtin_amdgcn_update_dpp(x, __builtin_bit_cast(int, f3), 0xe4, 0x8, 0xf, false);
+  return __builtin_bit_cast(float, x);
+}
+
+// TOKCOL (calls without scores, at most four query heads per KV head): the logits MFMA takes the
+// query as its row operand, head r % 4 in row r, and the codes as its column operand, so result lane
+// (j, n) holds token n of the tile for the heads 0..3 in its four registers, the same in every lane
+// group.  Lane group j keeps head j: the token's block scales are the lane's own (no exchange), the
+// softmax runs once per logit instead of once per operand column, a head's maximum is a reduction
+// inside one 16-lane row, and the probabilities reach the P operand's layout (lane (j, r): tokens
+// 4j..4j+3 of head r % 4) through 256 bytes of LDS per wave.
+template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, bool TOKCOL>
 __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
@@ -382,6 +401,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane >> 4, r = lane & 15;
   const int G = p.group;
+  const int rh = TOKCOL ? (r & 3) : r;  // head whose query this lane's operand row (or column) carries
 
   const int t_begin = split * p.chunk;
   const int t_end = min(p.len, t_begin + p.chunk);
@@ -510,7 +530,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   float qinit[KK];  // what a block's MFMA accumulator starts from: -sum over the block of (slot bias + zero point) * q
   {
     const float c = p.scale * 1.4426950408889634f;
-    const int h = kvh * G + min(r, G - 1);
+    const int h = kvh * G + min(rh, G - 1);
     const float *qp = p.q + (int64_t)b * p.q_bs + (int64_t)h * D;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
@@ -521,7 +541,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       float part = 0.0f, biased = 0.0f;
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
-        const float x = (r < G) ? qv[s] * c : 0.0f;
+        const float x = (rh < G) ? qv[s] * c : 0.0f;
         part += x;
         if constexpr (FMT == kFmtQ2_0) biased = fmaf(CD::slot_bias(s), x, biased);
         _Float16 hi, lo;
@@ -532,10 +552,12 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       // the four lane groups hold the four quarters of the block
       part += __shfl_xor(part, 16, 64);
       part += __shfl_xor(part, 32, 64);
+      if constexpr (TOKCOL) part = __shfl(part, j, 64);  // the sums of head j, whose logits this lane keeps
       qsum[kk] = part;
       if constexpr (FMT == kFmtQ2_0) {
         biased += __shfl_xor(biased, 16, 64);
         biased += __shfl_xor(biased, 32, 64);
+        if constexpr (TOKCOL) biased = __shfl(biased, j, 64);
         qinit[kk] = -biased;
       } else {
         qinit[kk] = -(CD::kBias + CD::kZero) * part;
@@ -576,6 +598,101 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   int base_last = -(1 << 30);
 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
+    half4_t pa[TW];
+    if constexpr (TOKCOL) {
+      // ---- logits: token base + 16 tw + r, head j ------------------------------------------------
+      float sc[TW];
+      RawPiece<FMT> both[4];  // head_dim 64: lane group g held block g % 2 of tile g / 2
+      if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        sc[tw] = 0.0f;
+        RawPiece<FMT> kpc[KK];
+        if constexpr (D == 64) {
+          kpc[0] = both[2 * tw];
+          kpc[1] = both[2 * tw + 1];
+        } else {
+#pragma unroll
+          for (int u = 0; u < KQ; ++u) {
+            RawPiece<FMT> four[4];
+            block_to_pieces<FMT>(kblk[tw * KQ + u], four);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) kpc[4 * u + x] = four[x];
+          }
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const half8_t kb_op = code_operand<FMT>(kpc[kk], k_sel);
+          float4_t dot = {0.0f, 0.0f, 0.0f, 0.0f};
+          dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[kk], kb_op, dot, 0, 0, 0);
+          dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql[kk], kb_op, dot, 0, 0, 0);
+          // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q, times the
+          // token's scale for this block, which the lane holds itself
+          const half2_t dm = __builtin_bit_cast(half2_t, kpc[kk].hdr);
+          const float mine = row_pick(dot) + qinit[kk];
+          if constexpr (F::kHasMin) sc[tw] = fmaf((float)dm[0], mine, fmaf((float)dm[1], qsum[kk], sc[tw]));
+          else sc[tw] = fmaf((float)dm[0], mine, sc[tw]);
+        }
+      }
+      if constexpr (D != 64) __builtin_amdgcn_sched_barrier(0);  // (see the other arm)
+      load_k(base + kWaves * TILE);
+      load_idx_k(base + 2 * kWaves * TILE);
+      float mt = kNegInf;
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        if constexpr (SOFTCAP) {
+          const float sv = sc[tw];
+          const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * kLog2e;
+          sc[tw] = (sv != sv) ? kNegInf : capped;
+        }
+        if (base + 16 * tw + r >= t_end) sc[tw] = kNegInf;
+        sc[tw] = fmaxf(sc[tw], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
+        mt = fmaxf(mt, sc[tw]);
+      }
+      // ---- online softmax: a head's tokens are the 16 lanes of one row ---------------------------
+      mt = group_allreduce_max<16>(mt);
+      const float m_new = fmaxf(m_run, mt);
+      const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+      m_run = m_new;
+      half2_t pk = {(_Float16)0.0f, (_Float16)0.0f};
+      float lsum = 0.0f;
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const float e = __builtin_amdgcn_exp2f(sc[tw] - m_ref);  // the row sum takes the unrounded weight
+        lsum += e;
+        pk[tw] = (_Float16)e;
+      }
+      l_run = l_run * alpha + lsum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        // O accumulator register i belongs to head i, whose factor every lane of row i holds
+        float al[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 16 * i, 64);
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o_acc[a][i] *= al[i];
+        if constexpr (kHdrTerm) {
+#pragma unroll
+          for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h_acc[sg][i] *= al[i];
+        }
+      }
+      // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of head r % 4
+      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][4][20];
+      wave_lds_fence();  // the previous iteration's reads are done
+      p_strip[wave][j][r] = __builtin_bit_cast(uint32_t, pk);
+      wave_lds_fence();
+      const u32x4_t w = *(const u32x4_t *)&p_strip[wave][rh][4 * j];
+      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const uint32_t sel = tw ? 0x07060302u : 0x05040100u;
+        pa[tw] = __builtin_bit_cast(half4_t, u32x2_t{__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel)});
+      }
+    } else {
     // ---- logits ---------------------------------------------------------------------------------
     float4_t s[TW];
     RawPiece<FMT> both[4];  // head_dim 64: lane group g held block g % 2 of tile g / 2
@@ -674,7 +791,6 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
     m_run = m_new;
-    half4_t pa[TW];
     float lsum = 0.0f;
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
@@ -703,6 +819,8 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
           for (int i = 0; i < 4; ++i) h_acc[sg][i] *= al[i];
       }
+    }
+
     }
 
     // ---- O += P . V -----------------------------------------------------------------------------
@@ -771,10 +889,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
-  if (p.stage_scores) {
+  if (!TOKCOL && p.stage_scores) {
     flush_staged_logits(p, dyn_lds, stage_row, b, kvh * G, G, t_begin, t_end);
   } else {
-    sink.store_tail(base_last);
+    if constexpr (!TOKCOL) sink.store_tail(base_last);
     __syncthreads();  // the other waves' spare slots lie in the merge area
   }
 
@@ -789,14 +907,18 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   }
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
+  if constexpr (TOKCOL) {
+    l_run = group_allreduce_sum<16>(l_run);  // lane group j holds head j
+  } else {
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+  }
   float (*lds_m)[16] = (float (*)[16])dyn_lds;
   float (*lds_l)[16] = lds_m + kWaves;
   float (*lds_acc)[SH::MAXH][D + 4] = (float (*)[SH::MAXH][D + 4])(dyn_lds + 2 * kWaves * 16);
-  if (j == 0) {
-    lds_m[wave][r] = m_run;
-    lds_l[wave][r] = l_run;
+  if (TOKCOL ? r == 0 : j == 0) {
+    lds_m[wave][TOKCOL ? j : r] = m_run;
+    lds_l[wave][TOKCOL ? j : r] = l_run;
   }
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg)
@@ -805,7 +927,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       const int ch = 32 * vblk[sg] + ((D == 64) ? half_slot_elem<FMT>(r & 3, r >> 3, c) : slot_elem<FMT>(r & 3, c));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][ch] = o_acc[sg * VCH + c][i];
+        if (TOKCOL ? j == 0 : 4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][ch] = o_acc[sg * VCH + c][i];  // (TOKCOL: rows 4j + i repeat head i)
     }
   __syncthreads();
 
@@ -842,15 +964,17 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   constexpr int kStageBytes = 48 * 1024;
   constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * BlockShape<D>::MAXH * (D + 4)) * sizeof(float);
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
-  const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_blocks_kernel<FMT, D, TW, false, false>, 64 * kWaves,
+  const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_blocks_kernel<FMT, D, TW, false, false, false>, 64 * kWaves,
                                           max_chunk > 0 ? (size_t)kStageBytes : merge_bytes);
   choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   p.direct = 0;
   p.stage_scores = p.scores && p.chunk <= max_chunk;
   const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-  auto kern = cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true> : decode_blocks_kernel<FMT, D, TW, true, false>)
-                  : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true> : decode_blocks_kernel<FMT, D, TW, false, false>);
+  const bool tokcol = !p.scores && !cap && p.group <= 4;
+  auto kern = cap      ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, false> : decode_blocks_kernel<FMT, D, TW, true, false, false>)
+              : tokcol ? (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, true> : decode_blocks_kernel<FMT, D, TW, false, false, true>)
+                       : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, false> : decode_blocks_kernel<FMT, D, TW, false, false, false>);
   ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + 1024));
   const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
