@@ -380,7 +380,7 @@ __device__ __forceinline__ float row_pick(const float4_t &v) {
   return __builtin_bit_cast(float, x);
 }
 
-// TOKCOL (calls without scores, at most four query heads per KV head): the logits MFMA takes the
+// TOKCOL (at most four query heads per KV head): the logits MFMA takes the
 // query as its row operand, head r % 4 in row r, and the codes as its column operand, so result lane
 // (j, n) holds token n of the tile for the heads 0..3 in its four registers, the same in every lane
 // group.  Lane group j keeps head j: the token's block scales are the lane's own (no exchange), the
@@ -649,6 +649,23 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         sc[tw] = fmaxf(sc[tw], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
         mt = fmaxf(mt, sc[tw]);
       }
+      // Emitted logits: parked in the chunk's LDS rows (lanes with nothing to park write to a spare
+      // slot of their own), or stored through the sink's bounds-checked descriptor with an offset
+      // that drops the store.  Under a uniform branch: calls without scores run 2 % faster that way
+      // than with the stores always issued and dropped.
+      if (p.scores) {  // uniform
+        const bool parks = j < staged_heads;
+        float *dst = parks ? dyn_lds + j * stage_row + (base - t_begin) + r : spare + 4 * TW * (int)threadIdx.x;
+        const uint32_t row_off = (uint32_t)(((int64_t)j * p.score_stride + r) * 4);
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          const float logit = sc[tw] * kLn2;
+          dst[parks ? 16 * tw : tw] = logit;
+          const bool writes = sink.on && j < G && base + 16 * tw + r < t_end;
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, logit), sink.rsrc,
+                                                writes ? row_off + 4u * (uint32_t)(base + 16 * tw) : LogitSink<TW>::kDropped, 0u, 2);
+        }
+      }
       // ---- online softmax: a head's tokens are the 16 lanes of one row ---------------------------
       mt = group_allreduce_max<16>(mt);
       const float m_new = fmaxf(m_run, mt);
@@ -889,10 +906,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
-  if (!TOKCOL && p.stage_scores) {
+  if (p.stage_scores) {
     flush_staged_logits(p, dyn_lds, stage_row, b, kvh * G, G, t_begin, t_end);
   } else {
-    if constexpr (!TOKCOL) sink.store_tail(base_last);
+    if constexpr (!TOKCOL) sink.store_tail(base_last);  // (TOKCOL stores single logits: no group is cut)
     __syncthreads();  // the other waves' spare slots lie in the merge area
   }
 
@@ -971,10 +988,13 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   p.stage_scores = p.scores && p.chunk <= max_chunk;
   const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-  const bool tokcol = !p.scores && !cap && p.group <= 4;
-  auto kern = cap      ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, false> : decode_blocks_kernel<FMT, D, TW, true, false, false>)
-              : tokcol ? (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, true> : decode_blocks_kernel<FMT, D, TW, false, false, true>)
-                       : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, false> : decode_blocks_kernel<FMT, D, TW, false, false, false>);
+  const bool tokcol = p.group <= 4;
+  auto pick = [&](auto tc) {
+    constexpr bool TC = decltype(tc)::value;
+    return cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, TC> : decode_blocks_kernel<FMT, D, TW, true, false, TC>)
+               : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, TC> : decode_blocks_kernel<FMT, D, TW, false, false, TC>);
+  };
+  auto kern = tokcol ? pick(std::true_type{}) : pick(std::false_type{});
   ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + 1024));
   const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
