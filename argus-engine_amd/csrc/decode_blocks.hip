@@ -698,7 +698,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         }
       }
       // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of head r % 4
-      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][4][20];
+      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][4][16];  // 64 words: writes and reads each touch every bank once
       wave_lds_fence();  // the previous iteration's reads are done
       p_strip[wave][j][r] = __builtin_bit_cast(uint32_t, pk);
       wave_lds_fence();
