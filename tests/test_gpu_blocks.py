@@ -137,6 +137,18 @@ def test_ragged_lengths_at_every_head_dim(fmt, d):
         run_case(fmt, 8, 2, d, L, cap=400, seed=L + d)
 
 
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_every_group_width_with_and_without_scores(fmt, d):
+    # Up to four query heads per KV head the kernel keeps one head per lane group (the logits MFMA
+    # has the tokens in its columns); wider groups keep the heads in the columns.  Every head must
+    # get its own logits in both, with the scores emitted or not, over ragged and multi-tile rows.
+    for g in (1, 2, 3, 4, 5, 8):
+        for L in (97, 1300):
+            run_case(fmt, 2 * g, 2, d, L, cap=L + 5, seed=g + L + d, scores=bool((g + L) & 1))
+            run_case(fmt, 2 * g, 2, d, L, cap=L + 5, seed=g + L + d + 1, scores=not ((g + L) & 1))
+
+
 @pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_0", 16, 8, 256, 2048), ("q8_0", 8, 4, 256, 1000), ("q4_1", 32, 8, 128, 1500), ("q4_0", 14, 2, 64, 777),
                                             ("q2_0", 32, 8, 128, 900)])
 def test_soft_cap_on_block_caches(fmt, hq, hkv, d, L):
