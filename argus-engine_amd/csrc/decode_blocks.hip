@@ -23,6 +23,9 @@
 //       result: the result lane (j, h) holds tokens 4j..4j+3, whose scales sit in lanes 20j + i of
 //       the wave and are fetched with ds_bpermute (q4_1 adds m_kk(token) * sum of Q_kk).  Logits
 //       therefore carry no f16 rounding of d * (n - 8), and the emitted scores keep the 1e-4 bar.
+//       With at most four query heads per KV head the two operands change places (TOKCOL, see the
+//       kernel): S[head][token], the result lane (j, n) holds token n for the heads 0..3, lane
+//       group j keeps head j and applies the scales of its own token.
 //   O[head][channel] = P . V     v_mfma_f32_16x16x16_f16
 //       B: lane (j, r) loads, for tokens 4j..4j+3, code bytes 4(r%4).. of block r/4, dequantises
 //       them to f16 (one rounding, 2^-12 relative: far below the 2e-3 output bar) and gets
