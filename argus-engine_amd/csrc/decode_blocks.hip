@@ -277,6 +277,33 @@ __device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p, uint32_t
   return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
 }
 
+// The values d * code of the pieces of two tokens (4-bit formats), slot by slot: out[s] = {token a's
+// value of slot s, token b's}.  The code words are interleaved first -- bytes 0, 1 of both tokens in
+// one word, bytes 2, 3 in another -- and the four shifts of piece_codes then bring out one nibble
+// position of both tokens at a time: byte 0 low, byte 1 low, byte 0 high, byte 1 high from the first
+// word are slots 0, 2, 4, 6, the same from the second word slots 1, 3, 5, 7.
+template <int FMT, int N>
+__device__ __forceinline__ void scaled_pair(const RawPiece<FMT> &a, const RawPiece<FMT> &b, uint32_t upper, half2_t (&out)[N]) {
+  static_assert((FMT == kFmtQ4_0 || FMT == kFmtQ4_1) && (N == 8 || N == 4), "nibble formats; whole or half pieces");
+  const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b.hdr, a.hdr, 0x05040100u));  // {d_a, d_b}
+  const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};                               // exact
+  uint32_t mask = 0x00f000f0u, exponent = 0x54005400u;
+  asm("" : "+v"(mask), "+v"(exponent));  // keep both in vector registers
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    uint32_t w = __builtin_amdgcn_perm(b.code[0], a.code[0], h ? 0x07060302u : 0x05040100u);
+    // Half pieces (head_dim 64, N = 4): the lane's half is the low or the high nibbles (`upper`),
+    // brought down by a per-lane shift; slots 0..3 are bytes 0, 2, 1, 3 of that half.
+    if constexpr (N == 4) w >>= 4u * upper;
+    out[0 + h] = __builtin_elementwise_fma(nibbles(w << 4, mask, exponent), dd, nb);
+    out[2 + h] = __builtin_elementwise_fma(nibbles(w >> 4, mask, exponent), dd, nb);
+    if constexpr (N == 8) {
+      out[4 + h] = __builtin_elementwise_fma(nibbles(w, mask, exponent), dd, nb);
+      out[6 + h] = __builtin_elementwise_fma(nibbles(w >> 8, mask, exponent), dd, nb);
+    }
+  }
+}
+
 // Half a piece (head_dim 64): the element held by slot s of the half `upper` of code index x, and
 // its 4 values d * code.  q4: `upper` selects the high nibbles, brought down by a per-lane shift so
 // that both halves run the same instructions; q8: the piece's one code dword is already the half;
@@ -884,12 +911,23 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
           for (int e = 0; e < 4; ++e) vpc[e] = vraw[tw][sg][e];
         }
+        // The V operand of channel c wants the four tokens' values side by side.  The 4-bit formats
+        // interleave the code words of two tokens before the nibbles come out (scaled_pair), so a
+        // register holds one channel of two tokens and no value is moved afterwards; the others
+        // dequantise token by token and transpose.
+        constexpr bool kPairV = FMT == kFmtQ4_0 || FMT == kFmtQ4_1;
         typedef _Float16 vrow_t __attribute__((ext_vector_type(VCH)));
         vrow_t vrow[4];
+        half2_t vpair[2][VCH];
+        if constexpr (kPairV) {
+          scaled_pair<FMT, VCH>(vpc[0], vpc[1], (uint32_t)(r >> 3), vpair[0]);
+          scaled_pair<FMT, VCH>(vpc[2], vpc[3], (uint32_t)(r >> 3), vpair[1]);
+        } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (D == 64) vrow[e] = scaled_half<FMT>(vpc[e], (uint32_t)(r >> 3), v_half_sel);
-          else vrow[e] = scaled_codes<FMT>(vpc[e], v_sel);
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (D == 64) vrow[e] = scaled_half<FMT>(vpc[e], (uint32_t)(r >> 3), v_half_sel);
+            else vrow[e] = scaled_codes<FMT>(vpc[e], v_sel);
+          }
         }
         if constexpr (kHdrTerm) {
           // d (q4_0: low halves of the headers) or m (q4_1, q2_0: high halves) of the lane's four tokens
@@ -902,7 +940,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         }
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {
-          const half4_t bv = {vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
+          half4_t bv;
+          if constexpr (kPairV) bv = half4_t{vpair[0][c][0], vpair[0][c][1], vpair[1][c][0], vpair[1][c][1]};
+          else bv = half4_t{vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
           o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * VCH + c], 0, 0, 0);
         }
       }
