@@ -237,7 +237,12 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   // would put groups j and j+2 on the same banks.
   constexpr int VPAD = 16;
   constexpr int V8_VEC = 8 * KK * BB / 16;  // 16-byte vectors per 8 tokens
-  constexpr int WAVE_BYTES = 2 * TILE_BYTES + 4 * VPAD;
+  // ... and the K tile 16 bytes after every two slices: slices lie 32 blocks = 32 (mod 64) dwords
+  // apart, so the lanes that read the headers of slices kk and kk + 2 in one instruction would
+  // otherwise hit the same banks with different addresses.
+  constexpr int K2_VEC = 2 * 32 * BB / 16;  // 16-byte vectors per two slices
+  constexpr int KPADS = 16 * ((KK + 1) / 2);
+  constexpr int WAVE_BYTES = 2 * TILE_BYTES + KPADS + 4 * VPAD;
   constexpr int MERGE_BYTES = 4 * kMaxGroup * (D + 4) * 4 + 4 * kMaxGroup * KK * 4 + 2 * 4 * 16 * 4;
   constexpr int SMEM = (4 * WAVE_BYTES > MERGE_BYTES) ? 4 * WAVE_BYTES : MERGE_BYTES;
   constexpr int NREP = 16 / GT;               // lanes of a row that share one head
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
   const int q_units = kp.q_tokens / kUnit;
 
   uint8_t *sK = smem + wave * WAVE_BYTES;
-  uint8_t *sV = sK + TILE_BYTES;
+  uint8_t *sV = sK + TILE_BYTES + KPADS;
   const uint8_t *sVj = sV + j * (8 * KK * BB + VPAD);  // this lane group's 8 tokens
   const uint8_t *qk_b = kp.qk + (int64_t)b * kp.qk_bs;
   const uint8_t *qv_b = kp.qv + (int64_t)b * kp.qv_bs;
@@ -423,7 +428,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
     for (int c = 0; c < NCH; ++c) {
       const int i = lane + 64 * c;
       if (i < TILE_VEC) {
-        ((u32x4_t *)sK)[i] = pk[c];
+        ((u32x4_t *)sK)[i + i / K2_VEC] = pk[c];
         ((u32x4_t *)sV)[i + i / V8_VEC] = pv[c];
       }
     }
@@ -442,8 +447,8 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
       // packed instructions per pair instead of two conversions, a product and a split per value.
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint32_t h0 = *(const uint32_t *)(sK + (32 * kk + 8 * j + 2 * pr) * BB);
-        const uint32_t h1 = *(const uint32_t *)(sK + (32 * kk + 8 * j + 2 * pr + 1) * BB);
+        const uint32_t h0 = *(const uint32_t *)(sK + (32 * kk + 8 * j + 2 * pr) * BB + 16 * (kk / 2));
+        const uint32_t h1 = *(const uint32_t *)(sK + (32 * kk + 8 * j + 2 * pr + 1) * BB + 16 * (kk / 2));
         const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(h1, h0, 0x05040100u));  // [d0, d1]
         const half2_t mm = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(h1, h0, 0x07060302u));  // [m0, m1]
         half2_t hi = dd * qh2[s][pr];
@@ -471,7 +476,7 @@ __global__ __launch_bounds__(256, (D == 256) ? 2 : 3) void kivi_mfma_kernel(cons
       uint32_t w0[4], w1[4];
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
-        const uint8_t *cp = sK + (32 * kk + 8 * j + 2 * pr) * BB + foff;
+        const uint8_t *cp = sK + (32 * kk + 8 * j + 2 * pr) * BB + 16 * (kk / 2) + foff;
         // (FASTK: w0 = low nibbles in place ... unused; the byte and the high nibbles are the operands)
         if constexpr (FASTK) {
           const uint32_t v = field_read2<BITS>(cp, cp + BB);
