@@ -27,6 +27,10 @@
 //    read from the accumulator rows of the lanes that prepared its operand.
 //  * The zero-point terms: sum m*q on the vector ALU while the scales are read, sum p*m as one
 //    more MFMA whose operand is the f16 `m` header itself.
+//  * The softmax is computed once per logit: the 32 x GT sums of a unit move from the operand
+//    columns to the lanes (bank, head) of their row first, a lane exponentiates 8 * GT / 16 values,
+//    and the packed probabilities return to every lane of the head with DPP moves.  The maximum and
+//    the zero-point dot product cross the wave's four rows with v_permlane16/32_swap.
 //
 // Waves are autonomous: a wave prefetches its next unit into registers while it works on the
 // current one, and there is no workgroup barrier inside the unit loop.  The residual window (F32
