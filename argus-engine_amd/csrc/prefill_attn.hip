@@ -82,24 +82,33 @@ __device__ __forceinline__ half8_t load_kv_chunk<float>(__amdgpu_buffer_rsrc_t r
   }
   return h;
 }
-// 8 consecutive f32 query elements rounded to f16
-__device__ __forceinline__ half8_t load_q_f32(const float *p) {
+// 8 consecutive f32 query elements times `c`, rounded to f16
+__device__ __forceinline__ half8_t load_q_f32(const float *p, float c) {
   const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
   half8_t h;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    h[e] = (_Float16)a[e];
-    h[4 + e] = (_Float16)b[e];
+    h[e] = (_Float16)(a[e] * c);
+    h[4 + e] = (_Float16)(b[e] * c);
   }
+  return h;
+}
+// 8 consecutive f16 query elements times `c`
+__device__ __forceinline__ half8_t load_q_f16(const _Float16 *p, float c) {
+  const half8_t r = *(const half8_t *)p;
+  half8_t h;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) h[e] = (_Float16)((float)r[e] * c);
   return h;
 }
 
 // The same as hi + lo (lo = the f16 nearest to what hi leaves; zero where that is not finite)
-__device__ __forceinline__ void load_q_f32_split(const float *p, half8_t &hi, half8_t &lo) {
+__device__ __forceinline__ void load_q_f32_split(const float *p, float c, half8_t &hi, half8_t &lo) {
   const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const float x = e < 4 ? a[e] : b[e - 4];
+    float x = (e < 4 ? a[e] : b[e - 4]) * c;
+    asm("" : "+v"(x));  // one f32 product for both halves (no fused re-rounding)
     const _Float16 h = (_Float16)x;
     const float rest = x - (float)h;
     hi[e] = h;
@@ -143,6 +152,13 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   constexpr int CH = NG * BN * D / 8 / NT;   // 16-byte chunks per thread per iteration
   constexpr int kLdsAhead = 4;               // MFMA operand reads kept in flight
   constexpr int kVAhead = (D <= 64) ? 4 : 3;
+#ifndef PF_VALU_MASK
+#define PF_VALU_MASK 0x402
+#endif
+#ifndef PF_PHASE_VALU
+#define PF_PHASE_VALU ((D <= 64) ? 4 : 0)
+#endif
+  constexpr int kPhaseValu = PF_PHASE_VALU;  // vector-ALU instructions placed behind each MFMA of a phase
 
   // [2 buffers][NG tiles][K tile | V^T tile]; reused at the end for the cross-group merge.
   extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
@@ -181,11 +197,11 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     const int64_t qoff = (((int64_t)b * p.seq_len + min(row, p.seq_len - 1)) * p.n_heads_q + h) * D + 8 * hl;
     if (p.q_f16) {
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) qreg[kk] = *(const half8_t *)((const _Float16 *)p.q + qoff + 16 * kk);
+      for (int kk = 0; kk < KK; ++kk) qreg[kk] = load_q_f16((const _Float16 *)p.q + qoff + 16 * kk, p.scale_log2e);
     } else {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
-        qreg[kk] = load_q_f32((const float *)p.q + qoff + 16 * kk);
+        qreg[kk] = load_q_f32((const float *)p.q + qoff + 16 * kk, p.scale_log2e);
       }
     }
   };
@@ -195,7 +211,18 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   for (int r = 0; r < RB; ++r)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o_acc[r][i] = 0.0f;
-  float m_run = kNegInf, l_run = 0.0f;
+  // The query is held times scale * log2(e), and the logit accumulators start from -m_ref (negm: sixteen
+  // copies of it, the shape of an accumulator block; m_ref = m_run, or 0 while the row has seen no key),
+  // so the matrix cores deliver exponents ready for v_exp_f32.
+  // (kFold; where registers allow.  Otherwise the accumulators start from zero and m_ref is
+  // subtracted in front of the exponential.)
+  constexpr bool kFold = D <= 64;
+  float m_run = kNegInf, l_run = 0.0f, m_ref = 0.0f;
+  float16_t negm;
+  if constexpr (kFold) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) negm[i] = 0.0f;
+  }
 
   // ---- key range of the workgroup -----------------------------------------------------------
   const int wg_row_last = min(p.seq_len, (qt + 1) * QPW * 32) - 1;
@@ -267,36 +294,56 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     const int key0 = kt * BN;
     return it < n_it && kt < kt_end && r0 < p.seq_len && key0 <= wave_hi && key0 + BN > wave_lo;
   };
+  // Instruction order of a phase, given once all of its code has been emitted (the groups only draw on
+  // instructions in front of them): operand reads kept a few MFMAs ahead (one LDS round trip is
+  // several times an MFMA's 32 cycles), and behind every MFMA NV of the phase's vector-ALU
+  // instructions -- the exponentials of another tile -- because a wave issues in order and MFMAs back
+  // to back would hold them up until the last has started.
+  auto sched_qk = [&](auto nv_c) {
+    constexpr int NV = decltype(nv_c)::value;
+    __builtin_amdgcn_sched_group_barrier(0x100, kLdsAhead, 0);
+#pragma unroll
+    for (int i = 0; i < KK * KB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (i < KK * KB - kLdsAhead) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if constexpr (NV > 0) __builtin_amdgcn_sched_group_barrier(PF_VALU_MASK, NV, 0);
+    }
+  };
+  auto sched_pv = [&](auto nv_c) {  // two transposing reads per MFMA
+    constexpr int NV = decltype(nv_c)::value;
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kVAhead, 0);
+#pragma unroll
+    for (int i = 0; i < (BN / 16) * RB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (i < (BN / 16) * RB - kVAhead) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      if constexpr (NV > 0) __builtin_amdgcn_sched_group_barrier(PF_VALU_MASK, NV, 0);
+    }
+  };
   // S^T = K . Q^T for this wave's tile of iteration `it`
-  auto qk_tile = [&](int it, float16_t(&s_acc)[KB]) {
+  auto qk_tile = [&](int it, float16_t(&s_acc)[KB], bool hints = true) {
     const _Float16 *sK = sKb + ((it & 1) * NG + kvg) * (BN * KP);
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s_acc[kb][i] = 0.0f;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
-        s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
+        if (kFold && kk == 0)
+          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], negm, 0, 0, 0);
+        else if (kk == 0)
+          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], float16_t{0.0f}, 0, 0, 0);
+        else
+          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], s_acc[kb], 0, 0, 0);
       }
     // Keep kLdsAhead operand reads in flight ahead of the MFMA that consumes them: one LDS round
     // trip per MFMA is several times the MFMA's own 32 cycles.
-    __builtin_amdgcn_sched_group_barrier(0x100, kLdsAhead, 0);
-#pragma unroll
-    for (int i = 0; i < KK * KB - kLdsAhead; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kLdsAhead, 0);
+    if (hints) sched_qk(std::integral_constant<int, 0>{});
     if constexpr (QLO) {
       if (few_keys) {  // uniform over the workgroup
         const int64_t qoff = (((int64_t)b * p.seq_len + min(row, p.seq_len - 1)) * p.n_heads_q + h) * D + 8 * hl;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
           half8_t hi, lo;
-          load_q_f32_split((const float *)p.q + qoff + 16 * kk, hi, lo);
+          load_q_f32_split((const float *)p.q + qoff + 16 * kk, p.scale_log2e, hi, lo);
 #pragma unroll
           for (int kb = 0; kb < KB; ++kb) {
             const half8_t a = *(const half8_t *)(sK + (32 * kb + ln) * KP + 16 * kk + 8 * hl);
@@ -307,22 +354,41 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
       }
     }
   };
-  // Per-tile softmax state handed from the phase that finds the maximum to the one that exponentiates.
-  struct TileMax {
-    float m_ref;  // reference the tile's probabilities are taken against (log2 units)
-    float alpha;  // factor the running sums take before this tile is added
-  };
-  // Mask (edge tiles only) and row maximum of the tile of iteration `it`.  The running maximum is
-  // only moved when a row's maximum exceeds it by more than kLazy (log2 units): probabilities then
-  // reach at most 2^kLazy, which f16 and the f32 sums hold easily, and almost every tile leaves the
-  // accumulators unscaled.
+  // Mask (edge tiles only) and row maximum of the tile of iteration `it`, whose accumulators hold
+  // logit - m_ref.  The reference only moves when a row's maximum exceeds it by more than kLazy (log2
+  // units), or when the row sees its first key: the tile's exponents, the accumulator start values
+  // and m_run move at once, and the factor the running sums must take before this tile is added is
+  // returned (1 for almost every tile).
   constexpr float kLazy = 8.0f;
-  auto mask_max = [&](int it, float16_t(&s_acc)[KB], auto interior_c) -> TileMax {
-    constexpr bool INTERIOR = decltype(interior_c)::value;
+  auto row_max = [&](float16_t(&s_acc)[KB]) {
+    float mt = kNegInf;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
+    return xor32_combine(mt, [](float a, float b) { return fmaxf(a, b); });
+  };
+  // exponents of a tile whose accumulators were formed against the old reference follow it
+  auto shift_tile = [&](float16_t(&s_acc)[KB], float delta) {
+    if constexpr (kFold) {
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_acc[kb][i] -= delta;
+    }
+  };
+  auto shift_ref = [&](float delta) {  // m_ref += delta (a no-op in lanes whose delta is zero)
+    if constexpr (kFold) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) negm[i] -= delta;
+    }
+    m_ref += delta;
+  };
+  auto mask_max = [&](int it, float16_t(&s_acc)[KB]) -> float {
     const int key0 = (kt_begin + it * NG + kvg) * BN;
     const int q_pos = row + p.q_start;
-    const bool need_mask = !INTERIOR && ((key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
-                                         (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1));
+    const bool need_mask = (key0 + BN - 1 > r0 + p.q_start) || (key0 + BN > p.cache_len) ||
+                           (p.window > 0 && key0 < r0 + 31 + p.q_start - p.window + 1);
     if (need_mask) {
       const int lo = p.window > 0 ? q_pos - p.window : -1;  // keys <= lo are outside the window
       const int hi = min(q_pos, p.cache_len - 1);
@@ -334,46 +400,68 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
           s_acc[kb][i] = (key <= hi && key > lo) ? s_acc[kb][i] : kNegInf;
         }
     }
-    float mt = kNegInf;
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mt = fmaxf(mt, s_acc[kb][i]);
-    mt = xor32_combine(mt, [](float a, float b) { return fmaxf(a, b); }) * p.scale_log2e;
-    const float m_new = (mt > m_run + kLazy) ? mt : m_run;  // also takes the first finite maximum
-    TileMax t;
-    t.m_ref = (m_new == kNegInf) ? 0.0f : m_new;
-    t.alpha = __builtin_amdgcn_exp2f(m_run - t.m_ref);
-    m_run = m_new;
-    return t;
+    const float mt = row_max(s_acc) - (kFold ? 0.0f : m_ref);
+    const bool first = m_run == kNegInf;
+    const float delta = first ? (mt == kNegInf ? 0.0f : mt) : (mt > kLazy ? mt : 0.0f);
+    const float alpha = first ? 0.0f : __builtin_amdgcn_exp2f(-delta);
+    if (__builtin_amdgcn_ballot_w64(delta != 0.0f) != 0) {
+      shift_tile(s_acc, delta);
+      shift_ref(delta);
+    }
+    if (!first || mt != kNegInf) m_run = m_ref;
+    return alpha;
   };
-  // Probabilities of the current tile (exp2 against t.m_ref), rounded to f16 in P^T operand order.
-  half8_t pb[BN / 16];
-  auto rescale = [&](const TileMax &t) {
-    if (__builtin_amdgcn_ballot_w64(t.alpha != 1.0f) != 0) {
+  auto rescale = [&](float alpha) {
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
       for (int r = 0; r < RB; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[r][i] *= t.alpha;
-      l_run *= t.alpha;
+        for (int i = 0; i < 16; ++i) o_acc[r][i] *= alpha;
+      l_run *= alpha;
     }
   };
-  auto exp_tile = [&](float16_t(&s_acc)[KB], const TileMax &t) {
+  typedef half8_t PTile[BN / 16];
+  // probabilities of P^T slices [J0, J1) of a tile (16 keys each) into pt; returns their row sum
+  auto exp_part = [&](float16_t(&s_acc)[KB], PTile &pt, auto j0_c, auto j1_c) -> float {
     // The row sum is taken over the f16-rounded probabilities the matrix cores consume, so the
     // rounding cancels in the final normalisation.
     float lsum = 0.0f;
 #pragma unroll
-    for (int jn = 0; jn < BN / 16; ++jn) {
+    for (int jn = decltype(j0_c)::value; jn < decltype(j1_c)::value; ++jn) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        pb[jn][e] = (_Float16)__builtin_amdgcn_exp2f(fmaf(s_acc[jn / 2][8 * (jn % 2) + e], p.scale_log2e, -t.m_ref));
+      for (int e = 0; e < 8; ++e) {
+        const float x = s_acc[jn / 2][8 * (jn % 2) + e];
+        pt[jn][e] = (_Float16)__builtin_amdgcn_exp2f(kFold ? x : x - m_ref);
+      }
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
-        const half2_t pr = {pb[jn][e], pb[jn][e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
+        const half2_t pr = {pt[jn][e], pt[jn][e + 1]}, one = {(_Float16)1.0f, (_Float16)1.0f};
         lsum = __builtin_amdgcn_fdot2(pr, one, lsum, false);
       }
     }
-    l_run += lsum;
+    return lsum;
+  };
+  typedef std::integral_constant<int, 0> J0;
+  typedef std::integral_constant<int, BN / 16> JN;
+  // Interior steps form the first kSplit slices of a tile's probabilities one phase early (beside
+  // the output MFMAs of the tile before), so both phases of a step carry vector-ALU work.
+  constexpr int kSplit = (D <= 64) ? BN / 32 : 0;
+  typedef std::integral_constant<int, kSplit> JS;
+  auto exp_tile = [&](float16_t(&s_acc)[KB], PTile &pt) -> float { return exp_part(s_acc, pt, J0{}, JN{}); };
+  // Interior tiles take no maximum: the exponents stand against a reference that some earlier tile
+  // of the row set, and a probability only leaves f16's range when a logit exceeds that reference
+  // by 16 -- which shows in the tile's row sum.  Then (rarely) the reference moves up to the tile's
+  // maximum: the sums so far, this tile's exponents and the next tile's (already formed against the
+  // old reference) are corrected and the probabilities taken again.
+  auto overflow_fix = [&](float16_t(&s_cur)[KB], float16_t(&s_next)[KB], PTile &pt) -> float {
+    const float mt = row_max(s_cur) - (kFold ? 0.0f : m_ref);
+    const float delta = mt > kLazy ? mt : 0.0f;
+    rescale(__builtin_amdgcn_exp2f(-delta));
+    shift_tile(s_cur, delta);
+    shift_tile(s_next, delta);
+    shift_ref(delta);
+    m_run = m_ref;
+    return exp_tile(s_cur, pt);
   };
   // O^T += V^T . P^T for the tile of iteration `it`.
   // V stays row major in LDS.  The A operand wants, per lane, 8 keys of one channel:
@@ -384,7 +472,7 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   // 4 hl + {0..3} and 8 + 4 hl + {0..3} of each 16 in the contraction slots of lane half hl.
   const int g16 = lane >> 4, s16 = lane & 15;
   const int vlane_off = (4 * (g16 >> 1) + (s16 >> 2)) * VP + 16 * (g16 & 1) + 4 * (s16 & 3);
-  auto pv_tile = [&](int it) {
+  auto pv_tile = [&](int it, PTile &pb, bool hints = true) {
     const _Float16 *vlane = sVb + ((it & 1) * NG + kvg) * (BN * VP) + vlane_off;
 #pragma unroll
     for (int jn = 0; jn < BN / 16; ++jn)
@@ -396,13 +484,7 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
         o_acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[jn], o_acc[r], 0, 0, 0);
       }
     // two transposing reads per MFMA, kept kVAhead MFMAs ahead
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kVAhead, 0);
-#pragma unroll
-    for (int i = 0; i < (BN / 16) * RB - kVAhead; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kVAhead, 0);
+    if (hints) sched_pv(std::integral_constant<int, 0>{});
   };
 
   // One pipeline step.  On entry s_cur holds the logits of iteration `it` and t_cur their maximum
@@ -411,7 +493,12 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   // of tile it+1.  Interior steps (every tile of the iteration lies below the diagonal of every
   // wave, inside the cache and the window, and there is a next iteration) have no per-wave
   // conditions, so each phase is one basic block the scheduler can interleave.
-  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], TileMax &t_cur, auto interior_c, auto parity_c) {
+  // Probabilities, rounded to f16 in P^T operand order: of the current tile, and (interior steps)
+  // the first slices of the next one.
+  PTile pb_a, pb_b;
+  float l_head = 0.0f;  // row sum of the slices formed early
+  auto step = [&](int it, float16_t(&s_cur)[KB], float16_t(&s_next)[KB], PTile &pb_cur, PTile &pb_next, float &a_cur,
+                  auto interior_c, auto parity_c) {
     constexpr bool INTERIOR = decltype(interior_c)::value;
     // register set fetched into during this step, and the one staged at its end
     typedef std::integral_constant<int, kDeep ? decltype(parity_c)::value : 0> FetchSet;
@@ -419,15 +506,28 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     constexpr int AHEAD = kDeep ? 1 : 0;
     const bool act = INTERIOR || tile_active(it);
     const bool has_next = INTERIOR || it + 1 < n_it;
-    if (act) rescale(t_cur);  // its branch stays out of the phases below
+    if (!INTERIOR && act) rescale(a_cur);  // its branch stays out of the phases below
     fetch_k(it + 2 + AHEAD, FetchSet{});  // past the last tile: all zeros, nothing is read
     fetch_v(it + 1 + AHEAD, FetchSet{});
     // ---- phase A
-    if (has_next) qk_tile(it + 1, s_next);  // harmless on a tile the wave cannot see
-    if (act) exp_tile(s_cur, t_cur);
+    if (has_next) qk_tile(it + 1, s_next, !INTERIOR);  // harmless on a tile the wave cannot see
+    if constexpr (INTERIOR) {
+      float lsum = l_head + exp_part(s_cur, pb_cur, JS{}, JN{});
+      sched_qk(std::integral_constant<int, kPhaseValu>{});
+      if (__builtin_amdgcn_ballot_w64(!(lsum < 1e30f)) != 0) lsum = overflow_fix(s_cur, s_next, pb_cur);
+      l_run += lsum;
+    } else {
+      if (act) l_run += exp_tile(s_cur, pb_cur);
+    }
     // ---- phase B
-    if (act) pv_tile(it);
-    if (INTERIOR || tile_active(it + 1)) t_cur = mask_max(it + 1, s_next, interior_c);
+    if (act) pv_tile(it, pb_cur, !INTERIOR);
+    if constexpr (INTERIOR) {
+      l_head = exp_part(s_next, pb_next, J0{}, JS{});
+      sched_pv(std::integral_constant<int, kPhaseValu>{});
+      a_cur = 1.0f;
+    } else {
+      if (tile_active(it + 1)) a_cur = mask_max(it + 1, s_next);
+    }
     if (INTERIOR || it + 2 < n_it) stage_k(it & 1, StageSet{});  // a fill nobody reads is harmless
     if (has_next) stage_v((it + 1) & 1, StageSet{});
     __syncthreads();  // fills are visible; every wave is done with the buffers the next step refills
@@ -454,9 +554,9 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
     }
   }
   __syncthreads();
-  TileMax t_cur = {0.0f, 1.0f};
+  float t_cur = 1.0f;
   if (n_it > 0) qk_tile(0, s_a);
-  if (tile_active(0)) t_cur = mask_max(0, s_a, std::false_type{});
+  if (tile_active(0)) t_cur = mask_max(0, s_a);
   __syncthreads();  // sKb[0] is refilled by the first step
   // leading interior iterations, rounded down to pairs so that s_a holds the current logits after them
   int n_int = 0;
@@ -468,13 +568,17 @@ __global__ __launch_bounds__(256 * NG, (NG == 1 && D <= 128) ? 2 : 1) void prefi
   // then only ever concern the loads of the loop itself and can leave the youngest in flight.
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   int it = 0;
+  if (n_int > 0) l_head = exp_part(s_a, pb_a, J0{}, JS{});
   for (; it < n_int; it += 2) {
-    step(it, s_a, s_b, t_cur, std::true_type{}, std::integral_constant<int, 0>{});
-    step(it + 1, s_b, s_a, t_cur, std::true_type{}, std::integral_constant<int, 1>{});
+    step(it, s_a, s_b, pb_a, pb_b, t_cur, std::true_type{}, std::integral_constant<int, 0>{});
+    step(it + 1, s_b, s_a, pb_b, pb_a, t_cur, std::true_type{}, std::integral_constant<int, 1>{});
   }
+  // the tile the interior steps leave behind has its exponents but no maximum yet (and the slices of
+  // its probabilities formed early are formed again with the others)
+  if (it > 0) t_cur = mask_max(it, s_a);
   for (; it < n_it; it += 2) {
-    step(it, s_a, s_b, t_cur, std::false_type{}, std::integral_constant<int, 0>{});
-    if (it + 1 < n_it) step(it + 1, s_b, s_a, t_cur, std::false_type{}, std::integral_constant<int, 1>{});
+    step(it, s_a, s_b, pb_a, pb_a, t_cur, std::false_type{}, std::integral_constant<int, 0>{});
+    if (it + 1 < n_it) step(it + 1, s_b, s_a, pb_a, pb_a, t_cur, std::false_type{}, std::integral_constant<int, 1>{});
   }
 
   // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
