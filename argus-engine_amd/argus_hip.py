@@ -36,6 +36,7 @@ EXPORTED_SYMBOLS = [
     "argus_hip_attention_gen_quant_ex", "argus_hip_gather_update_quant", "argus_hip_quant_flush",
     "argus_hip_quant_dequant_flush", "argus_hip_quant_scatter_residual",
     "argus_hip_score_reduce", "argus_hip_score_reduce_per_layer",
+    "argus_hip_score_reduce_ex", "argus_hip_score_reduce_per_layer_ex",
     "argus_hip_kv_scatter_f32_to_f16", "argus_hip_kv_scatter_f32_to_f16_batch",
     "argus_hip_kv_scatter_f32_batch", "argus_hip_kv_decode_descriptor", "argus_hip_kv_encode_descriptor",
     "argus_hip_attention_gen_desc", "argus_hip_quant_requant",
@@ -91,7 +92,8 @@ class AttentionGenArgs(C.Structure):
                 ("q_batch_stride", C.c_int64), ("out_batch_stride", C.c_int64),
                 ("kv_batch_stride", C.c_int64), ("score_batch_stride", C.c_int64),
                 ("index_batch_stride", C.c_int64),
-                ("softcap", C.c_float), ("scale", C.c_float)]
+                ("softcap", C.c_float), ("scale", C.c_float),
+                ("score_stats", C.c_void_p), ("stats_batch_stride", C.c_int64)]
 
 
 class PrefillArgs(C.Structure):
@@ -125,7 +127,11 @@ class QuantAttnExt(C.Structure):
     _fields_ = [("scores_dev", C.c_uint64), ("score_stride", C.c_size_t),
                 ("res_dtype", C.c_int32), ("softcap", C.c_float), ("batch", C.c_int32),
                 ("block_batch_stride_bytes", C.c_int64), ("res_batch_stride", C.c_int64),
-                ("score_batch_stride", C.c_int64)]
+                ("score_batch_stride", C.c_int64), ("score_stats_dev", C.c_uint64)]
+
+
+class ScoreReduceExt(C.Structure):
+    _fields_ = [("stats", C.c_uint64)]
 
 
 class QuantGatherArgs(C.Structure):
@@ -251,6 +257,8 @@ def _bind():
     lib.argus_hip_quant_scatter_residual.argtypes = [vp, C.POINTER(QuantScatterResidualArgs)]
     lib.argus_hip_score_reduce.argtypes = [vp, C.POINTER(ScoreReduceArgs)]
     lib.argus_hip_score_reduce_per_layer.argtypes = [vp, C.POINTER(ScoreReduceArgs)]
+    lib.argus_hip_score_reduce_ex.argtypes = [vp, C.POINTER(ScoreReduceArgs), C.POINTER(ScoreReduceExt)]
+    lib.argus_hip_score_reduce_per_layer_ex.argtypes = [vp, C.POINTER(ScoreReduceArgs), C.POINTER(ScoreReduceExt)]
     sc16 = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32]
     lib.argus_hip_kv_scatter_f32_to_f16.argtypes = sc16
     lib.argus_hip_kv_scatter_f32_to_f16_batch.argtypes = sc16 + [i32]
@@ -449,11 +457,12 @@ class Context:
     def attention_gen(self, q, k, v, out, num_heads_kv, cache_seq_len, capacity=0,
                       layout=HEAD_MAJOR, scores=None, score_stride=0, kv_index=None, kv_start=0,
                       batch=1, kv_batch_stride=0, index_batch_stride=0, softcap=0.0, scale=0.0,
-                      check=True, kv_dtype=None, noalloc=False, desc=None):
+                      check=True, kv_dtype=None, noalloc=False, desc=None, score_stats=None):
         """q/out [batch, Hq, d] (or [Hq, d]) f32; k/v device caches; scores [batch, Hq, stride].
         kv_dtype: Q4_0 / Q4_1 / Q8_0 / Q2_0 for uint8 tensors of blocks (default: from the tensor dtype).
         noalloc: go through argus_hip_attention_gen_noalloc (partials in the library's static array).
-        desc: KVLayoutDesc tuple of a uint8 cache of blocks: go through argus_hip_attention_gen_desc."""
+        desc: KVLayoutDesc tuple of a uint8 cache of blocks: go through argus_hip_attention_gen_desc.
+        score_stats [batch, Hq, 2] f32: `scores` keeps the logits, (max, sum) of every row go here."""
         hq, d = q.shape[-2], q.shape[-1]
         a = AttentionGenArgs(
             stream=_stream(), q=_ptr(q), k_cache=_ptr(k), v_cache=_ptr(v), out=_ptr(out),
@@ -463,7 +472,8 @@ class Context:
             kv_dtype=0 if desc is not None else _kv_dtype(k) if kv_dtype is None else kv_dtype,
             batch=batch, score_stride=score_stride, q_batch_stride=0, out_batch_stride=0,
             kv_batch_stride=kv_batch_stride, score_batch_stride=0,
-            index_batch_stride=index_batch_stride, softcap=softcap, scale=scale)
+            index_batch_stride=index_batch_stride, softcap=softcap, scale=scale,
+            score_stats=_ptr(score_stats), stats_batch_stride=0)
         if desc is not None:
             dd = KvLayoutDesc(*desc)
             return self._check(lib.argus_hip_attention_gen_desc(self.handle, C.byref(a), C.byref(dd)), check)
@@ -503,7 +513,7 @@ class Context:
     def attention_gen_quant(self, q, qk, qv, res_k, res_v, out, num_heads_kv, q_tokens, res_tokens,
                             res_cap, scale, bits, scores_host=None, scores_dev=None,
                             score_stride=0, softcap=0.0, batch=1, block_batch_stride_bytes=0,
-                            res_batch_stride=0, check=True):
+                            res_batch_stride=0, check=True, score_stats=None):
         """scores_host: numpy float32 array (host readback, reference contract);
         scores_dev: torch tensor (device)."""
         import torch
@@ -516,12 +526,13 @@ class Context:
             num_heads_kv=num_heads_kv, head_dim=d, q_tokens=q_tokens, res_tokens=res_tokens,
             res_cap=res_cap, scale=scale, bits=bits)
         res_dtype = F16 if res_k.dtype == torch.float16 else F32
-        if scores_dev is None and res_dtype == F32 and softcap == 0.0 and batch == 1:
+        if scores_dev is None and res_dtype == F32 and softcap == 0.0 and batch == 1 and score_stats is None:
             return self._check(lib.argus_hip_attention_gen_quant(self.handle, C.byref(a)), check)
         e = QuantAttnExt(scores_dev=_ptr(scores_dev), score_stride=score_stride,
                          res_dtype=res_dtype, softcap=softcap, batch=batch,
                          block_batch_stride_bytes=block_batch_stride_bytes,
-                         res_batch_stride=res_batch_stride, score_batch_stride=0)
+                         res_batch_stride=res_batch_stride, score_batch_stride=0,
+                         score_stats_dev=_ptr(score_stats) or 0)
         return self._check(lib.argus_hip_attention_gen_quant_ex(self.handle, C.byref(a), C.byref(e)), check)
 
     def gather_update_quant(self, inp, residual, kv_heads, res_cap, head_dim, seq_len, res_pos,
@@ -588,15 +599,22 @@ class Context:
             layer_flat_importance=_ptr(layer_flat))
 
     def score_reduce(self, scores, importance, head_importance, decay_factor, n_layers, n_heads_q,
-                     n_kv_heads, cache_seq_len, score_stride, max_seq_len, check=True):
+                     n_kv_heads, cache_seq_len, score_stride, max_seq_len, check=True, stats=None):
+        """stats [n_layers, n_heads_q, 2]: `scores` holds logits, normalised while they are read."""
         a = self._score_args(scores, importance, head_importance, decay_factor, n_layers, n_heads_q,
                              n_kv_heads, cache_seq_len, score_stride, max_seq_len, None)
+        if stats is not None:
+            e = ScoreReduceExt(stats=_ptr(stats))
+            return self._check(lib.argus_hip_score_reduce_ex(self.handle, C.byref(a), C.byref(e)), check)
         return self._check(lib.argus_hip_score_reduce(self.handle, C.byref(a)), check)
 
     def score_reduce_per_layer(self, scores, layer_flat, decay_factor, n_layers, n_heads_q,
-                               n_kv_heads, cache_seq_len, score_stride, max_seq_len, check=True):
+                               n_kv_heads, cache_seq_len, score_stride, max_seq_len, check=True, stats=None):
         a = self._score_args(scores, None, None, decay_factor, n_layers, n_heads_q, n_kv_heads,
                              cache_seq_len, score_stride, max_seq_len, layer_flat)
+        if stats is not None:
+            e = ScoreReduceExt(stats=_ptr(stats))
+            return self._check(lib.argus_hip_score_reduce_per_layer_ex(self.handle, C.byref(a), C.byref(e)), check)
         return self._check(lib.argus_hip_score_reduce_per_layer(self.handle, C.byref(a)), check)
 
     # -- (f-1) ---------------------------------------------------------------------------

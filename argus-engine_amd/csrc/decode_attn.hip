@@ -358,6 +358,8 @@ static int attention_gen_impl(argus_hip_ctx *ctx, const argus_hip_attention_gen_
   if (a->scores_out && a->score_stride < a->cache_seq_len)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: score_stride %d < cache_seq_len %d",
                       a->score_stride, a->cache_seq_len);
+  if (a->score_stats && !a->scores_out)
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: score_stats without scores_out");
   if (a->batch > 65535 || a->num_heads_kv > 65535)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: batch / kv heads beyond grid limits");
 
@@ -374,6 +376,8 @@ static int attention_gen_impl(argus_hip_ctx *ctx, const argus_hip_attention_gen_
   p.v = a->v_cache;
   p.out = a->out;
   p.scores = a->scores_out;
+  p.score_stats = a->score_stats;
+  p.stats_bs = a->stats_batch_stride ? a->stats_batch_stride : (int64_t)a->num_heads_q * 2;
   p.kv_index = a->kv_index;
   p.n_heads_q = a->num_heads_q;
   p.n_heads_kv = a->num_heads_kv;

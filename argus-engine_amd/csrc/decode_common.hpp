@@ -17,6 +17,9 @@ struct DecodeParams {
   const void *v;
   float *out;
   float *scores;
+  // When set, `scores` keeps the logits and the combine pass writes each row's (max, sum) here
+  // instead of rewriting the row as probabilities: [batch, Hq, 2], batch stride stats_bs.
+  float *score_stats;
   const int32_t *kv_index;
   float *ws_ml;  // [batch, Hq, nsplit, 2]
   float *ws_o;   // [batch, Hq, nsplit, D]
@@ -25,7 +28,7 @@ struct DecodeParams {
   int32_t score_stride;
   int64_t row_stride;   // elements between consecutive token rows of one KV head
   int64_t head_stride;  // elements between KV heads
-  int64_t q_bs, out_bs, kv_bs, score_bs, index_bs;
+  int64_t q_bs, out_bs, kv_bs, score_bs, index_bs, stats_bs;
   float scale, softcap;
   int32_t direct;  // nsplit == 1 and no scores: first pass writes `out` itself
   int32_t slot_bound;  // slots an index list may name (the cache capacity)
@@ -100,7 +103,13 @@ __device__ void uniform_fallback(const DecodeParams &p, int b, int h, int D) {
   }
   if (p.scores) {
     float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = u;
+    // (logits + statistics form: exp(0 - 0) / len is the same uniform weight)
+    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = p.score_stats ? 0.0f : u;
+    if (p.score_stats && threadIdx.x == 0) {
+      float *st = p.score_stats + (int64_t)b * p.stats_bs + (int64_t)h * 2;
+      st[0] = 0.0f;
+      st[1] = (float)p.len;
+    }
   }
 }
 
@@ -123,7 +132,13 @@ __device__ inline void uniform_fallback<DescRow>(const DecodeParams &p, int b, i
   }
   if (p.scores) {
     float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = u;
+    // (logits + statistics form: exp(0 - 0) / len is the same uniform weight)
+    for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = p.score_stats ? 0.0f : u;
+    if (p.score_stats && threadIdx.x == 0) {
+      float *st = p.score_stats + (int64_t)b * p.stats_bs + (int64_t)h * 2;
+      st[0] = 0.0f;
+      st[1] = (float)p.len;
+    }
   }
 }
 
@@ -171,16 +186,17 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
   // slice is 4096 tokens, kAhead per thread), so the rewrite does not start a second round trip
   // once the row's maximum and sum are known.
   constexpr int kAhead = 16;
+  const bool rewrite = p.scores && !p.score_stats;  // else the row keeps its logits and only (max, sum) are written
   float *srow = p.scores ? p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride : nullptr;
   const int slice = ((p.len + (int)gridDim.z - 1) / (int)gridDim.z + 255) / 256 * 256;
   const int t_end = min(p.len, ((int)blockIdx.z + 1) * slice);
   const int t0 = (int)blockIdx.z * slice + (int)threadIdx.x;
   // Rows that start on a 16-byte boundary are read and written as float4: thread x then owns the
   // tokens 4 (x + 256 k) .. + 3 of the slice's first 4096 instead of x + 256 k (k < kAhead).
-  const bool vec = p.scores && (((uintptr_t)srow) & 15) == 0;
+  const bool vec = rewrite && (((uintptr_t)srow) & 15) == 0;
   const int s0 = (int)blockIdx.z * slice;
   float logit[kAhead];
-  if (p.scores) {
+  if (rewrite) {
     if (vec) {
 #pragma unroll
       for (int k = 0; k < kAhead / 4; ++k) {
@@ -242,6 +258,11 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     if (first && FALLBACK::run(p, b, h, D)) return;
   }
   const float inv = 1.0f / ll;  // non-finite when the fallback declined: NaN propagates
+  if (first && p.score_stats && threadIdx.x == 0) {
+    float *st = p.score_stats + (int64_t)b * p.stats_bs + (int64_t)h * 2;
+    st[0] = mm;
+    st[1] = ll;
+  }
   if (first) {
     float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -257,7 +278,7 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
       *(float4_t *)(p.out + (int64_t)b * p.out_bs + (int64_t)h * D + 4 * cq) = o * inv;
     }
   }
-  if (p.scores) {
+  if (rewrite) {
     if (vec) {
 #pragma unroll
       for (int k = 0; k < kAhead / 4; ++k) {
@@ -441,7 +462,7 @@ inline bool score_rows_addressable(const DecodeParams &p) {
 
 // Grid of the combine pass: one workgroup per (head, sequence), more along z for long score rows.
 inline dim3 combine_grid(const DecodeParams &p, int batch) {
-  const int z = p.scores ? std::max(1, std::min(64, p.len / 4096)) : 1;
+  const int z = (p.scores && !p.score_stats) ? std::max(1, std::min(64, p.len / 4096)) : 1;
   return dim3((unsigned)p.n_heads_q, (unsigned)batch, (unsigned)z);
 }
 

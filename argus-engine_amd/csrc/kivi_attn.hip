@@ -433,6 +433,12 @@ ARGUS_API int argus_hip_attention_gen_quant_ex(argus_hip_ctx *ctx, const argus_h
   p.score_stride = (int32_t)stride;
   p.q_bs = p.out_bs = (int64_t)a->num_heads_q * D;
   p.score_bs = (int64_t)a->num_heads_q * stride;
+  if (ext && ext->score_stats_dev) {
+    if (!want_dev || want_host)
+      return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen_quant: score_stats_dev goes with scores_dev (and no host slice)");
+    p.score_stats = (float *)ext->score_stats_dev;
+    p.stats_bs = (int64_t)a->num_heads_q * 2;
+  }
   p.scale = a->scale;
   p.softcap = ext ? ext->softcap : 0.0f;
   kp.qk = (const uint8_t *)a->qk_mem;

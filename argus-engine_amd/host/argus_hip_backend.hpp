@@ -15,6 +15,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
+#include <limits>
 #include <memory>
 #include <string>
 #include <utility>
@@ -328,6 +329,9 @@ class HipScoreReduceBackend {
   const char *name() const { return "attn_score"; }
   int reduce(const argus_hip_score_reduce_args &a) const { return ctx_ ? argus_hip_score_reduce(ctx_, &a) : -1; }
   int reduce_per_layer(const argus_hip_score_reduce_args &a) const { return ctx_ ? argus_hip_score_reduce_per_layer(ctx_, &a) : -1; }
+  // score buffers in the logits + (max, sum) form
+  int reduce_ex(const argus_hip_score_reduce_args &a, const argus_hip_score_reduce_ext &e) const { return ctx_ ? argus_hip_score_reduce_ex(ctx_, &a, &e) : -1; }
+  int reduce_per_layer_ex(const argus_hip_score_reduce_args &a, const argus_hip_score_reduce_ext &e) const { return ctx_ ? argus_hip_score_reduce_per_layer_ex(ctx_, &a, &e) : -1; }
 
  private:
   argus_hip_ctx *ctx_;
@@ -462,6 +466,10 @@ class HipQuantWindowCache {
 // CudaGpuScoreAccumulator twin (engine/src/backend/cuda_pc/gpu_score.rs:72-403): persistent device
 // buffers [n_layers, n_heads_q, max_seq_len] scores + cumulative flat / per-head importance; the
 // attention kernel writes each layer's slice, end_step() folds them with the fused reducer.
+// The slices are kept in the library's logits + (max, sum) form (argus_hip_attention_gen_args::
+// score_stats, a [n_layers, n_heads_q, 2] buffer beside the scores): the reducer normalises while it
+// reads, with the arithmetic the attention call would have used to rewrite the rows, so the cumulative
+// buffers come out bit for bit as from probabilities, and no layer's row is read twice.
 class HipGpuScoreAccumulator {
  public:
   static Result<std::unique_ptr<HipGpuScoreAccumulator>> create(HipBackend *be, size_t n_layers, size_t n_heads_q,
@@ -483,14 +491,23 @@ class HipGpuScoreAccumulator {
     if (!alloc_zeroed(n_layers * n_heads_q * max_seq_len, &a->score_buf_) || !alloc_zeroed(max_seq_len, &a->importance_) ||
         !alloc_zeroed(n_kv_heads * max_seq_len, &a->head_importance_) || !alloc_zeroed(n_layers * max_seq_len, &a->layer_flat_))
       return R::Err("score buffer allocation failed: " + be->last_error());
+    // (max, sum) = (+inf, 1): a layer no call has written yet reads as all-zero probabilities
+    std::vector<float> st(n_layers * n_heads_q * 2);
+    for (size_t i = 0; i < st.size(); i += 2) { st[i] = std::numeric_limits<float>::infinity(); st[i + 1] = 1.0f; }
+    auto r = be->alloc(st.size() * sizeof(float));
+    if (!r.ok()) return R::Err("score statistics allocation failed: " + be->last_error());
+    a->stats_ = r.value();
+    if (!be->write_buffer(a->stats_, st.data(), st.size() * sizeof(float)).ok()) return R::Err(be->last_error());
     return R::Ok(std::move(a));
   }
   ~HipGpuScoreAccumulator() {
-    for (void *p : {score_buf_, importance_, head_importance_, layer_flat_})
+    for (void *p : {score_buf_, importance_, head_importance_, layer_flat_, stats_})
       if (p) be_->free(p);
   }
 
   uint64_t score_buf_device_ptr() const { return (uint64_t)score_buf_; }
+  // statistics rows of a layer's heads, or null while the buffer holds probabilities (debug fill)
+  float *layer_stats_ptr(size_t layer_idx) const { return logits_form_ ? (float *)stats_ + layer_idx * n_heads_q_ * 2 : nullptr; }
   size_t score_stride() const { return score_stride_; }
   size_t layer_offset_elems(size_t layer_idx) const { return layer_idx * n_heads_q_ * score_stride_; }
   size_t current_layer_idx() const { return current_layer_idx_; }
@@ -509,10 +526,12 @@ class HipGpuScoreAccumulator {
     a.cache_seq_len = cache_seq_len; a.score_stride = score_stride_; a.max_seq_len = max_seq_len_;
     a.layer_flat_importance = (uint64_t)layer_flat_;
     HipScoreReduceBackend reducer(be_->ctx());
-    int ret = reducer.reduce(a);
+    argus_hip_score_reduce_ext ext{};
+    ext.stats = logits_form_ ? (uint64_t)stats_ : 0;
+    int ret = reducer.reduce_ex(a, ext);
     if (ret != 0) return Status::Err("attn_score HIP reduce failed: code " + std::to_string(ret));
     if (per_layer_flat_) {
-      ret = reducer.reduce_per_layer(a);
+      ret = reducer.reduce_per_layer_ex(a, ext);
       if (ret != 0) return Status::Err("attn_score HIP per-layer reduce failed: code " + std::to_string(ret));
     }
     steps_ += 1;
@@ -590,13 +609,15 @@ class HipGpuScoreAccumulator {
   // Test-only, like the reference's debug_fill_score_buf.
   Status debug_fill_score_buf(const std::vector<float> &scores) {
     if (scores.size() != n_layers_ * n_heads_q_ * score_stride_) return Status::Err("debug_fill_score_buf: wrong length");
+    logits_form_ = false;  // the values given are probabilities
     return be_->write_buffer(score_buf_, scores.data(), scores.size() * 4);
   }
 
  private:
   explicit HipGpuScoreAccumulator(HipBackend *be) : be_(be) {}
   HipBackend *be_;
-  void *score_buf_ = nullptr, *importance_ = nullptr, *head_importance_ = nullptr, *layer_flat_ = nullptr;
+  void *score_buf_ = nullptr, *importance_ = nullptr, *head_importance_ = nullptr, *layer_flat_ = nullptr, *stats_ = nullptr;
+  bool logits_form_ = true;
   size_t n_layers_ = 0, n_heads_q_ = 0, n_kv_heads_ = 0, max_seq_len_ = 0, score_stride_ = 0;
   float decay_factor_ = 1.0f;
   bool active_ = false, per_layer_flat_ = false;
@@ -643,6 +664,7 @@ inline Status HipBackend::attention_gen_indexed(const Tensor &q, const Tensor &k
   if (acc_ && acc_->is_active()) {
     a.scores_out = (float *)acc_->score_buf_device_ptr() + acc_->layer_offset_elems(acc_->current_layer_idx());
     a.score_stride = (int32_t)acc_->score_stride();
+    a.score_stats = acc_->layer_stats_ptr(acc_->current_layer_idx());
   } else if (scores_out && num_heads_q > 0) {
     stride = scores_len / num_heads_q;
     if (stride != 0 && stride >= cache_seq_len) {

@@ -139,9 +139,10 @@ def result(wall, kernel_ms, tail_ms, nbytes, **more):
 
 
 def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores=False, softcap=0.0,
-                 rotate=1, seed=137):
+                 rotate=1, seed=137, stats=False):
     """Returns dict(ms_per_step, kernel_ms, bytes).  `rotate` distinct KV buffers are cycled so a
-    cache smaller than the rotation set cannot serve repeated reads."""
+    cache smaller than the rotation set cannot serve repeated reads.  stats: scores in the logits +
+    (max, sum) form that the device-side reduce consumes (no rewrite of the rows as probabilities)."""
     import torch
     cap = capacity or L
     g = torch.Generator(device="cuda").manual_seed(seed)
@@ -152,13 +153,15 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
     q = torch.randn((batch, hq, d), generator=g, device="cuda", dtype=torch.float32)
     out = torch.empty((batch, hq, d), device="cuda", dtype=torch.float32)
     scs = [torch.empty((batch, hq, cap), device="cuda", dtype=torch.float32) for _ in range(rotate)] if scores else None
+    st = torch.empty((batch, hq, 2), device="cuda", dtype=torch.float32) if (scores and stats) else None
     state = {"i": 0}
 
     def step():
         i = state["i"] % rotate
         state["i"] += 1
         ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, cap, scores=scs[i] if scores else None,
-                          score_stride=cap if scores else 0, batch=batch, kv_batch_stride=hkv * cap * d, softcap=softcap)
+                          score_stride=cap if scores else 0, batch=batch, kv_batch_stride=hkv * cap * d, softcap=softcap,
+                          score_stats=st)
 
     wall, kernel_ms, tail_ms = measure(ctx, step, steps, warmup)
     r = result(wall, kernel_ms, tail_ms, decode_bytes(hq, hkv, d, L, batch, 2, scores))
@@ -309,6 +312,10 @@ def bench_aux(ctx, steps, warmup):
           "fused importance + per-KV-head importance; 3 score buffers cycled (411 MB)")
     timed("score_reduce_per_layer_L32768_32x32", lambda: ctx.score_reduce_per_layer(next_scores(), lf, 0.9, nl, hq, hkv, L, L, L),
           bufs[0].numel() * 4 + 2 * lf.numel() * 4, "per-layer importance; 3 score buffers cycled (411 MB)")
+    stats = torch.rand((nl, hq, 2), generator=g, device="cuda") + 1.0
+    timed("score_reduce_L32768_32x32_from_logits", lambda: ctx.score_reduce(next_scores(), imp, himp, 0.9, nl, hq, hkv, L, L, L, stats=stats),
+          bufs[0].numel() * 4 + 2 * (imp.numel() + himp.numel()) * 4,
+          "the same reduce over logits + (max, sum): exp(s - max) / sum applied while reading")
     del bufs
 
     # (f-1) KV scatter of a 2048-token prefill chunk, F32 rows -> F16 HeadMajor cache
@@ -478,7 +485,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
-                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1",
+                    choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1", "primary_scores_stats",
                              "q8_0", "copy_calib", "aux", "layers", "primary_scores", "cfg5_b64", "prefill_d64_16k"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
@@ -511,6 +518,8 @@ def main():
             res = bench_layer_loop(ctx, args.steps, args.warmup)
         elif w == "primary_scores":
             res = bench_decode(ctx, 32, 8, 128, 32768, 16, args.steps, args.warmup, scores=True)
+        elif w == "primary_scores_stats":
+            res = bench_decode(ctx, 32, 8, 128, 32768, 16, args.steps, args.warmup, scores=True, stats=True)
         elif w == "cfg5_b64":
             res = bench_decode(ctx, 8, 4, 256, 2048, 64, args.steps, args.warmup, capacity=4096, scores=True, softcap=50.0)
         elif w == "decode_b1":
@@ -527,7 +536,7 @@ def main():
             res = bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=8)
         elif w == "cfg5":
             res = bench_decode(ctx, 8, 4, 256, 2048, 8, args.steps, args.warmup, capacity=4096, scores=True,
-                               softcap=50.0, rotate=8)
+                               softcap=50.0, rotate=8, stats=True)
         else:
             res = bench_kivi(ctx, 4 if w == "kivi_q4" else 8, args.steps, args.warmup, batch=32, rotate=2)
         print(json.dumps({"workload": w, "steps": args.steps, "warmup": args.warmup, "result": res}))
@@ -584,17 +593,22 @@ def main():
             "4 KV buffer sets rotated (512 MiB > Infinity Cache)")
         add("cfg3_L4096_b16", bench_decode(ctx, 32, 8, 128, 4096, 16, es, ew, rotate=2), "2 sets rotated")
         add("cfg3_L4096_b1", bench_decode(ctx, 32, 8, 128, 4096, 1, es, ew, rotate=16), "16 sets rotated")
-        add("cfg3_L32768_b16_scores", bench_decode(ctx, 32, 8, 128, 32768, 16, es, ew, scores=True),
-            "scores emitted (67 MB of logits per call); combine_us is the pass that rewrites them as probabilities")
+        add("cfg3_L32768_b16_scores", bench_decode(ctx, 32, 8, 128, 32768, 16, es, ew, scores=True, stats=True),
+            "scores emitted as logits + (max, sum) per row, the form the device-side H2O reduce reads (67 MB per call)")
+        add("cfg3_L32768_b16_scores_as_probabilities", bench_decode(ctx, 32, 8, 128, 32768, 16, es, ew, scores=True),
+            "the trait's form: combine_us is the pass that rewrites the 67 MB of logits as probabilities")
         add("cfg3_L256_b1", bench_decode(ctx, 32, 8, 128, 256, 1, es, ew, rotate=16),
             "short context: one workgroup per KV head, one launch (no combine pass)")
         add("cfg3_L256_b16", bench_decode(ctx, 32, 8, 128, 256, 16, es, ew, rotate=8), "short context, 16 sequences: one launch")
         add("cfg1_qwen_L1024_b1", bench_decode(ctx, 14, 2, 64, 1024, 1, es, ew), "latency-bound (0.5 MiB)")
         add("cfg5_gemma2_L2048_cap4096_b8_scores_softcap50",
+            bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=8, stats=True),
+            "scores emitted as logits + (max, sum); 8 KV and score buffer sets rotated (537 MB of attended rows)")
+        add("cfg5_gemma2_L2048_cap4096_b8_scores_as_probabilities",
             bench_decode(ctx, 8, 4, 256, 2048, 8, es, ew, capacity=4096, scores=True, softcap=50.0, rotate=8),
-            "scores emitted; 8 KV and score buffer sets rotated (537 MB of attended rows)")
+            "the trait's form (rows rewritten as probabilities by the combine pass)")
         add("cfg5_gemma2_L2048_cap4096_b64_scores_softcap50",
-            bench_decode(ctx, 8, 4, 256, 2048, 64, es, ew, capacity=4096, scores=True, softcap=50.0),
+            bench_decode(ctx, 8, 4, 256, 2048, 64, es, ew, capacity=4096, scores=True, softcap=50.0, stats=True),
             "the same shape with 64 sequences per call (542 MB): the kernel's rate once the call is not latency-bound")
         add("cfg4_kivi_q4_L8192_res128_f32", bench_kivi(ctx, 4, es, ew), "8 block sets rotated; single launch, 11.4 MB")
         add("cfg4_kivi_q8_L8192_res128_f32", bench_kivi(ctx, 8, es, ew), "8 block sets rotated; single launch, 19.7 MB")

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define ARGUS_HIP_ABI_VERSION 1
+#define ARGUS_HIP_ABI_VERSION 2
 
 /* Return codes. */
 #define ARGUS_HIP_OK 0
@@ -141,7 +141,12 @@ int argus_hip_synchronize(argus_hip_ctx *ctx, void *stream);
  *                            zeros or the last slot; the result for such a list is unspecified);
  *   softcap                : cap*tanh(s/cap) after scaling
  *                            (engine/kernels/flash_attn_f32_f16.cl:563-565; host passes 0);
- *   scale                  : 0 selects 1/sqrt(head_dim) (x86.rs:192).
+ *   scale                  : 0 selects 1/sqrt(head_dim) (x86.rs:192);
+ *   score_stats            : opt-in score form for consumers that reduce the scores on the device
+ *                            (argus_hip_score_reduce_ex): `scores_out` then keeps the LOGITS s_t (after
+ *                            scale and soft-cap, NaN as -inf) and score_stats[h*2 .. +1] = (max_t s_t,
+ *                            sum_t exp(s_t - max)), so that p_t = exp(s_t - max) / sum -- the call does
+ *                            not read the row again to rewrite it.  NULL: probabilities, as the trait says.
  * Block-quantised caches (kv_dtype ARGUS_HIP_Q4_0 / Q4_1 / Q8_0 / Q2_0): the Q4_0 arm of the reference
  * (common.rs:676-850, rows dequantised on the fly) and the in-kernel form of the `--kv-format`
  * attention whose reference floor decodes the whole cache to F32 first
@@ -174,6 +179,8 @@ typedef struct argus_hip_attention_gen_args {
   int64_t index_batch_stride; /* elements; 0 = one index list shared by the batch */
   float softcap;
   float scale;
+  float *score_stats;         /* device, [batch, num_heads_q, 2] F32 (max, sum), or NULL; needs scores_out */
+  int64_t stats_batch_stride; /* elements; 0 = num_heads_q*2 */
 } argus_hip_attention_gen_args;
 int argus_hip_attention_gen(argus_hip_ctx *ctx, const argus_hip_attention_gen_args *args);
 
@@ -273,6 +280,9 @@ typedef struct argus_hip_quant_attn_ext {
   int64_t block_batch_stride_bytes; /* between consecutive qk (and qv) block streams */
   int64_t res_batch_stride;         /* elements between consecutive residual windows */
   int64_t score_batch_stride;       /* elements; 0 = num_heads_q * score_stride */
+  /* Opt-in score form of argus_hip_attention_gen_args::score_stats: scores_dev keeps the logits and
+   * (max, sum) per head go here ([batch, num_heads_q, 2] F32, device); 0 = probabilities. */
+  uint64_t score_stats_dev;
 } argus_hip_quant_attn_ext;
 
 /* CudaQuantAttnBackend::{has_quant_attn_kernel, attention_gen_quant, gather_update_quant},
@@ -580,6 +590,20 @@ typedef struct argus_hip_score_reduce_args {
 } argus_hip_score_reduce_args;
 int argus_hip_score_reduce(argus_hip_ctx *ctx, const argus_hip_score_reduce_args *args);
 int argus_hip_score_reduce_per_layer(argus_hip_ctx *ctx, const argus_hip_score_reduce_args *args);
+/* The same reduces over a score buffer in the logits + (max, sum) form (argus_hip_attention_gen_args::
+ * score_stats): `stats` is [n_layers, n_heads_q, 2] F32 on the device and every score is taken as
+ * exp(s - max) / sum while it is read -- the arithmetic of the rewrite the attention call skipped, so the
+ * results equal those of the probability form bit for bit.  The reference reduce
+ * (crates/techniques/attn-score/src/score_reduce.cu:13-91) reads probabilities only; this form exists
+ * because the rewrite of a 32K-token score buffer costs as much as the reduce itself.  stats == 0:
+ * identical to the calls above. */
+typedef struct argus_hip_score_reduce_ext {
+  uint64_t stats;
+} argus_hip_score_reduce_ext;
+int argus_hip_score_reduce_ex(argus_hip_ctx *ctx, const argus_hip_score_reduce_args *args,
+                              const argus_hip_score_reduce_ext *ext);
+int argus_hip_score_reduce_per_layer_ex(argus_hip_ctx *ctx, const argus_hip_score_reduce_args *args,
+                                        const argus_hip_score_reduce_ext *ext);
 
 /* ---- (f-1) KV write path ---------------------------------------------------------------------- */
 /* Backend::kv_scatter_f32_to_f16 / _batch / _f32_batch, engine/src/backend.rs:425-545; device

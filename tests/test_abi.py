@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(A.lib, name), "missing export " + name
     assert sorted(A.EXPORTED_SYMBOLS) == declared
-    assert A.lib.argus_hip_abi_version() == 1
+    assert A.lib.argus_hip_abi_version() == 2
 
 
 def test_struct_layouts_match_header_field_order():

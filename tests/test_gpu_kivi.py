@@ -185,6 +185,38 @@ def test_batched_caches_match_single_calls():
         check_scores(host(sc)[i], p, "cache %d" % i)
 
 
+def test_scores_as_logits_and_statistics():
+    # the opt-in score form of the decode calls (rows keep their logits, (max, sum) beside them):
+    # probabilities rebuilt from it equal the default form's, outputs are identical
+    import torch
+    nb, hq, hkv, d, R, n, bits = 2, 8, 2, 128, 64, 64 * 5 + 17, 4
+    rng = np.random.default_rng(78)
+    caches = [O.kivi_build(rng.standard_normal((n, hkv, d)).astype(np.float32),
+                           rng.standard_normal((n, hkv, d)).astype(np.float32), R, bits) for _ in range(nb)]
+    q = dev(rng.standard_normal((nb, hq, d)).astype(np.float32))
+    nbytes = caches[0]["qk"].size
+    qk, qv = dev(np.stack([c["qk"] for c in caches])), dev(np.stack([c["qv"] for c in caches]))
+    rk, rv = dev(np.stack([c["res_k"] for c in caches])), dev(np.stack([c["res_v"] for c in caches]))
+    total = caches[0]["q_tokens"] + caches[0]["res_tokens"]
+    outs, scs = [], []
+    st = torch.zeros((nb, hq, 2), device="cuda")
+    for stats in (None, st):
+        out = torch.empty((nb, hq, d), device="cuda")
+        sc = torch.zeros((nb, hq, total), device="cuda")
+        ctx().attention_gen_quant(q, qk, qv, rk, rv, out, hkv, caches[0]["q_tokens"], caches[0]["res_tokens"], R,
+                                  1.0 / np.sqrt(d), bits, scores_dev=sc, score_stride=total, batch=nb,
+                                  block_batch_stride_bytes=nbytes, res_batch_stride=hkv * R * d, score_stats=stats)
+        outs.append(out)
+        scs.append(sc)
+    assert torch.equal(outs[0], outs[1])
+    assert torch.allclose(torch.exp(scs[1] - st[..., 0:1]) / st[..., 1:2], scs[0], rtol=1e-5, atol=0)
+    imp, himp = torch.zeros(total, device="cuda"), torch.zeros(hkv * total, device="cuda")
+    imp2, himp2 = torch.zeros(total, device="cuda"), torch.zeros(hkv * total, device="cuda")
+    ctx().score_reduce(scs[0], imp, himp, 1.0, nb, hq, hkv, total, total, total)
+    ctx().score_reduce(scs[1], imp2, himp2, 1.0, nb, hq, hkv, total, total, total, stats=st)
+    assert torch.equal(imp, imp2) and torch.equal(himp, himp2)
+
+
 def test_gather_update_and_flush_bit_exact():
     # Drive the container on the device: append tokens through gather_update_quant, quantise a
     # full residual with quant_flush, and compare blocks bit for bit with the CPU container

@@ -195,3 +195,120 @@ def test_h2o_loop_scores_to_keep_list_to_post_eviction_attention(hq, hkv, d, L, 
     ref, p = O.attention_gen(q, kg, vg, hkv, n, cap, scores=True, scores_stride=cap, softcap=softcap)
     check_attention_out(host(out), ref, "per-head compaction")
     check_scores(host(sc)[:, :n], p[:, :n], "scores after per-head compaction")
+
+
+def _decode_both_forms(q, kc, vc, hkv, L, cap, batch, softcap=0.0, context=None):
+    """One call with probabilities out, one with logits + (max, sum): (out, p, out2, logits, stats)."""
+    import torch
+    c = context or ctx()
+    hq, d = q.shape[-2], q.shape[-1]
+    qd, kd, vd = dev(q), dev(kc), dev(vc)
+    out = torch.empty((batch, hq, d), device="cuda")
+    sc = torch.zeros((batch, hq, cap), device="cuda")
+    c.attention_gen(qd, kd, vd, out, hkv, L, cap, scores=sc, score_stride=cap, batch=batch,
+                    kv_batch_stride=hkv * cap * d, softcap=softcap)
+    out2 = torch.empty_like(out)
+    lg = torch.zeros_like(sc)
+    st = torch.zeros((batch, hq, 2), device="cuda")
+    c.attention_gen(qd, kd, vd, out2, hkv, L, cap, scores=lg, score_stride=cap, batch=batch,
+                    kv_batch_stride=hkv * cap * d, softcap=softcap, score_stats=st)
+    return out, sc, out2, lg, st
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_config5_importance_through_the_logits_and_statistics_form(batch):
+    # The opt-in score form: the attention call leaves the logits and writes (max, sum) per row, the
+    # reduce normalises while it reads.  Same arithmetic as the rewrite it replaces, so the importance
+    # vectors must equal the probability form's bit for bit, and the oracle's to 1e-4 relative.
+    import torch
+    hq, hkv, d, hist, cap, softcap = 8, 4, 256, 8192, 4096, 50.0
+    keep = O.streaming_keep(4, 2044, hist, 0)
+    L = len(keep)
+    q = normal((batch, hq, d), 42)
+    kc = np.zeros((batch, hkv, cap, d), np.float16)
+    vc = np.zeros((batch, hkv, cap, d), np.float16)
+    for b in range(batch):
+        kc[b] = O.compact_keep(f16(normal((hkv, hist, d), 137 + b)), keep, cap)
+        vc[b] = O.compact_keep(f16(normal((hkv, hist, d), 53 + b)), keep, cap)
+    out, sc, out2, lg, st = _decode_both_forms(q, kc, vc, hkv, L, cap, batch, softcap)
+    assert torch.equal(out, out2)
+    m, l = st[..., 0:1], st[..., 1:2]
+    assert torch.allclose(torch.exp(lg[..., :L] - m) / l, sc[..., :L], rtol=1e-5, atol=0)
+    for b in range(batch):
+        imp, himp = torch.zeros(cap, device="cuda"), torch.zeros(hkv * cap, device="cuda")
+        ctx().score_reduce(sc[b], imp, himp, 1.0, 1, hq, hkv, L, cap, cap)
+        imp2, himp2 = torch.zeros(cap, device="cuda"), torch.zeros(hkv * cap, device="cuda")
+        ctx().score_reduce(lg[b], imp2, himp2, 1.0, 1, hq, hkv, L, cap, cap, stats=st[b])
+        assert torch.equal(imp, imp2) and torch.equal(himp, himp2)
+        lf, lf2 = torch.zeros(cap, device="cuda"), torch.zeros(cap, device="cuda")
+        ctx().score_reduce_per_layer(sc[b], lf, 0.5, 1, hq, hkv, L, cap, cap)
+        ctx().score_reduce_per_layer(lg[b], lf2, 0.5, 1, hq, hkv, L, cap, cap, stats=st[b])
+        assert torch.equal(lf, lf2)
+        _, p = O.attention_gen(q[b], kc[b], vc[b], hkv, L, cap, scores=True, scores_stride=cap, softcap=softcap)
+        oi, oh = np.zeros(cap, np.float32), np.zeros(hkv * cap, np.float32)
+        O.score_fused_reduce(p, oi, oh, 1.0, 1, hq, hkv, L, cap, cap)
+        check_scores(host(imp2), oi, "importance, seq %d" % b)
+        check_scores(host(himp2), oh, "head importance, seq %d" % b)
+
+
+def test_config3_batch16_importance_through_the_logits_and_statistics_form():
+    # 16 sequences of the Llama-3-8B head shape at 32K tokens; the 16 score buffers double as the
+    # "layers" of one reduce.  Bit equality with the probability form on everything, the oracle on a
+    # sampled sequence.
+    import torch
+    b, hq, hkv, d, L = 16, 32, 8, 128, 32768
+    g = torch.Generator(device="cuda").manual_seed(137)
+    k = torch.randn((b, hkv, L, d), generator=g, device="cuda", dtype=torch.float32).half()
+    v = torch.randn((b, hkv, L, d), generator=g, device="cuda", dtype=torch.float32).half()
+    q = dev(normal((b, hq, d), 42))
+    out, out2 = torch.empty((b, hq, d), device="cuda"), torch.empty((b, hq, d), device="cuda")
+    sc = torch.empty((b, hq, L), device="cuda")
+    lg = torch.empty((b, hq, L), device="cuda")
+    st = torch.zeros((b, hq, 2), device="cuda")
+    ctx().attention_gen(q, k, v, out, hkv, L, L, scores=sc, score_stride=L, batch=b, kv_batch_stride=hkv * L * d)
+    ctx().attention_gen(q, k, v, out2, hkv, L, L, scores=lg, score_stride=L, batch=b, kv_batch_stride=hkv * L * d,
+                        score_stats=st)
+    assert torch.equal(out, out2)
+    imp, himp = torch.zeros(L, device="cuda"), torch.zeros(hkv * L, device="cuda")
+    imp2, himp2 = torch.zeros(L, device="cuda"), torch.zeros(hkv * L, device="cuda")
+    ctx().score_reduce(sc, imp, himp, 0.9, b, hq, hkv, L, L, L)
+    ctx().score_reduce(lg, imp2, himp2, 0.9, b, hq, hkv, L, L, L, stats=st)
+    assert torch.equal(imp, imp2) and torch.equal(himp, himp2)
+    i = 5
+    _, p = O.attention_gen(host(q[i]), host(k[i]), host(v[i]), hkv, L, L, scores=True, impl="avx2")
+    imp1, himp1 = torch.zeros(L, device="cuda"), torch.zeros(hkv * L, device="cuda")
+    ctx().score_reduce(lg[i], imp1, himp1, 1.0, 1, hq, hkv, L, L, L, stats=st[i])
+    oi, oh = np.zeros(L, np.float32), np.zeros(hkv * L, np.float32)
+    O.score_fused_reduce(p, oi, oh, 1.0, 1, hq, hkv, L, L, L)
+    check_scores(host(imp1), oi, "importance")
+    check_scores(host(himp1), oh, "head importance")
+
+
+def test_statistics_form_on_the_other_decode_kernels_and_the_fallback_row():
+    # vector-ALU kernel (F32 cache), block cache (q4_0), KIVI; and a row without a finite logit,
+    # whose uniform weights come out of the statistics as exp(0 - 0) / len.
+    import torch
+    from blocks_util import random_blocks
+    hq, hkv, d, L, cap = 8, 2, 128, 700, 704
+    q = normal((1, hq, d), 1)
+    k32, v32 = normal((1, hkv, cap, d), 2), normal((1, hkv, cap, d), 3)
+    out, sc, out2, lg, st = _decode_both_forms(q, k32, v32, hkv, L, cap, 1)
+    assert torch.equal(out, out2)
+    assert torch.allclose(torch.exp(lg[..., :L] - st[..., 0:1]) / st[..., 1:2], sc[..., :L], rtol=1e-5, atol=0)
+    kq = random_blocks(O.DESC_Q4_0, hkv * cap * d // 32, 5)
+    vq = random_blocks(O.DESC_Q4_0, hkv * cap * d // 32, 6)
+    import argus_hip as A
+    qd, kd, vd = dev(q), dev(kq), dev(vq)
+    o1, o2 = torch.empty((1, hq, d), device="cuda"), torch.empty((1, hq, d), device="cuda")
+    s1, s2, t2 = torch.zeros((1, hq, cap), device="cuda"), torch.zeros((1, hq, cap), device="cuda"), torch.zeros((1, hq, 2), device="cuda")
+    ctx().attention_gen(qd, kd, vd, o1, hkv, L, cap, scores=s1, score_stride=cap, kv_dtype=A.Q4_0)
+    ctx().attention_gen(qd, kd, vd, o2, hkv, L, cap, scores=s2, score_stride=cap, kv_dtype=A.Q4_0, score_stats=t2)
+    assert torch.equal(o1, o2)
+    assert torch.allclose(torch.exp(s2[..., :L] - t2[..., 0:1]) / t2[..., 1:2], s1[..., :L], rtol=1e-5, atol=0)
+    # all-NaN query: no finite logit, uniform weights (common.rs:561-577)
+    qn = np.full((1, hq, d), np.nan, np.float32)
+    out, sc, out2, lg, st = _decode_both_forms(qn, f16(k32), f16(v32), hkv, L, cap, 1)
+    assert torch.equal(out, out2)
+    assert np.allclose(host(sc)[..., :L], 1.0 / L)
+    assert not host(lg)[..., :L].any() and np.array_equal(host(st).reshape(-1, 2), np.tile([0.0, float(L)], (hq, 1)))
+    assert ctx().attention_gen(dev(q), dev(f16(k32)), dev(f16(v32)), out, hkv, L, cap, score_stats=st, check=False) == A.ERR_INVALID
