@@ -144,7 +144,8 @@ class QuantFlushArgs(C.Structure):
     _fields_ = [("stream", C.c_void_p), ("res_k_mem", C.c_uint64), ("res_v_mem", C.c_uint64),
                 ("qk_mem", C.c_uint64), ("qv_mem", C.c_uint64), ("kv_heads", C.c_size_t),
                 ("res_cap", C.c_size_t), ("head_dim", C.c_size_t), ("flush_tokens", C.c_size_t),
-                ("k_block_start", C.c_size_t), ("v_block_start", C.c_size_t), ("bits", C.c_uint8)]
+                ("k_block_start", C.c_size_t), ("v_block_start", C.c_size_t), ("bits", C.c_uint8),
+                ("out_res_cap", C.c_size_t)]
 
 
 class QuantDequantFlushArgs(C.Structure):
@@ -543,11 +544,12 @@ class Context:
         return self._check(lib.argus_hip_gather_update_quant(self.handle, C.byref(a)), check)
 
     def quant_flush(self, res_k, res_v, qk, qv, kv_heads, res_cap, head_dim, flush_tokens,
-                    k_block_start, v_block_start, bits, check=True):
+                    k_block_start, v_block_start, bits, check=True, out_res_cap=0):
         a = QuantFlushArgs(stream=_stream(), res_k_mem=_ptr(res_k), res_v_mem=_ptr(res_v),
                            qk_mem=_ptr(qk), qv_mem=_ptr(qv), kv_heads=kv_heads, res_cap=res_cap,
                            head_dim=head_dim, flush_tokens=flush_tokens,
-                           k_block_start=k_block_start, v_block_start=v_block_start, bits=bits)
+                           k_block_start=k_block_start, v_block_start=v_block_start, bits=bits,
+                           out_res_cap=out_res_cap)
         return self._check(lib.argus_hip_quant_flush(self.handle, C.byref(a)), check)
 
     def quant_requant(self, src, dst, n_blocks, old_bits, new_bits, check=True):

@@ -28,7 +28,12 @@ struct KernelFacts {
   int wgs_per_cu;
 };
 
+// First word of every argus_hip_ctx: entry points that receive a context through an untyped slot of
+// the plugin interface check it before they touch anything else.
+constexpr uint64_t kArgusCtxTag = 0x4152475553484950ull;  // "ARGUSHIP"
+
 struct argus_hip_ctx {
+  uint64_t tag = kArgusCtxTag;
   int device = 0;
   int compute_units = 0;
   hipDeviceProp_t props;
@@ -58,6 +63,7 @@ struct argus_hip_ctx {
   std::vector<hipEvent_t> ev;
   size_t ev_used = 0;
   bool timing = false;
+  bool timer_held = false;  // an enclosing KernelTimer brackets the launches: inner ones stay off
   char err[512] = {0};
 };
 
@@ -68,7 +74,7 @@ struct KernelTimer {
   hipStream_t stream;
   bool on, marked;
   KernelTimer(argus_hip_ctx *c, hipStream_t s) : ctx(c), stream(s), on(false), marked(false) {
-    if (c->timing && c->ev_used + 3 <= c->ev.size()) {
+    if (c->timing && !c->timer_held && c->ev_used + 3 <= c->ev.size()) {
       on = true;
       (void)hipEventRecord(c->ev[c->ev_used], s);
     }

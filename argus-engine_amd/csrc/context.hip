@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 // Scratch of the entry point that allocates nothing (argus_hip_attention_gen_noalloc): the split-KV
@@ -14,10 +15,12 @@ constexpr size_t kScratchBytes = (size_t)16 << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kMaxDevices = 64;
 static void *g_scratch_addr[kMaxDevices] = {nullptr};
+static std::mutex g_scratch_lock;  // contexts may be created from several threads
 
 // With `device` current: the address of that device's copy of `scratch`, looked up once per device.
 static int scratch_lookup(argus_hip_ctx *ctx, int device) {
   if (device < 0 || device >= kMaxDevices) return ARGUS_HIP_OK;  // no scratch there: the entry point refuses
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
   if (!g_scratch_addr[device]) {
     void *ptr = nullptr;
     const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
@@ -115,6 +118,7 @@ ARGUS_API int argus_hip_destroy(argus_hip_ctx *ctx) {
   if (ctx->ws) (void)hipFree(ctx->ws);
   if (ctx->pfa_ws) (void)hipFree(ctx->pfa_ws);
   for (hipEvent_t e : ctx->ev) (void)hipEventDestroy(e);
+  ctx->tag = 0;  // a stale pointer no longer passes for a context
   delete ctx;
   return ARGUS_HIP_OK;
 }

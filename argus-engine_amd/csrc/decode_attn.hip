@@ -367,7 +367,9 @@ static int attention_gen_impl(argus_hip_ctx *ctx, const argus_hip_attention_gen_
   if (D != 64 && D != 128 && D != 256)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "attention_gen: head_dim %d not in {64,128,256}", D);
   // An index list names slots of a HeadMajor cache of `capacity` rows (of the `capacity` first
-  // positions of a SeqMajor one); the kernels treat a slot outside [0, capacity) as a masked token.
+  // positions of a SeqMajor one); a slot outside [0, capacity) never reaches memory outside the head's rows -- the vector-ALU kernel
+  // clamps it to the last slot, the matrix-core kernels read it as a row of zeros -- and the result
+  // for such a list is unspecified (the host mirror's attention_into_selected rejects it up front).
   if (a->kv_index && a->capacity <= 0)
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "attention_gen: kv_index needs capacity > 0 (got %d)", a->capacity);
   DecodeParams p{};

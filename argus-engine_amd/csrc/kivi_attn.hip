@@ -269,10 +269,11 @@ __device__ __forceinline__ void quantize_block(const float (&x)[32], uint8_t *ds
 template <int BITS>
 __global__ __launch_bounds__(128) void kivi_flush_k_kernel(const float *__restrict__ res_k, uint8_t *__restrict__ qk,
                                                            int kv_heads, int res_cap, int head_dim, int n_groups,
-                                                           int64_t block_start) {
+                                                           int64_t block_start, int out_gpf) {
   constexpr int BB = 4 + 32 * BITS / 8;
   // block order h -> group -> ch (quant_window_cache.rs:919-930); thread per block, ch fastest so
-  // the 32 strided row reads of a wave are coalesced across channels.
+  // the 32 strided row reads of a wave are coalesced across channels.  out_gpf: the groups are laid
+  // out as consecutive flushes of that many groups each (flush -> h -> group in flush -> ch).
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (int64_t)kv_heads * n_groups * head_dim) return;
   const int ch = (int)(i % head_dim);
@@ -281,15 +282,16 @@ __global__ __launch_bounds__(128) void kivi_flush_k_kernel(const float *__restri
   float x[32];
 #pragma unroll
   for (int t = 0; t < 32; ++t) x[t] = res_k[((int64_t)h * res_cap + g * 32 + t) * head_dim + ch];
-  quantize_block<BITS>(x, qk + (block_start + i) * BB);
+  const int64_t o = (((int64_t)(g / out_gpf) * kv_heads + h) * out_gpf + g % out_gpf) * head_dim + ch;
+  quantize_block<BITS>(x, qk + (block_start + o) * BB);
 }
 
 template <int BITS>
 __global__ __launch_bounds__(128) void kivi_flush_v_kernel(const float *__restrict__ res_v, uint8_t *__restrict__ qv,
                                                            int kv_heads, int res_cap, int head_dim, int flush_tokens,
-                                                           int64_t block_start) {
+                                                           int64_t block_start, int out_cap) {
   constexpr int BB = 4 + 32 * BITS / 8;
-  // block order h -> t -> b (quant_window_cache.rs:932-946)
+  // block order h -> t -> b (quant_window_cache.rs:932-946), in flushes of out_cap tokens
   const int bpt = head_dim / 32;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (int64_t)kv_heads * flush_tokens * bpt) return;
@@ -306,7 +308,8 @@ __global__ __launch_bounds__(128) void kivi_flush_v_kernel(const float *__restri
     x[4 * v + 2] = f[2];
     x[4 * v + 3] = f[3];
   }
-  quantize_block<BITS>(x, qv + (block_start + i) * BB);
+  const int64_t o = (((int64_t)(t / out_cap) * kv_heads + h) * out_cap + t % out_cap) * bpt + b;
+  quantize_block<BITS>(x, qv + (block_start + o) * BB);
 }
 
 // ---- bit-width transition ------------------------------------------------------------------------
@@ -516,19 +519,23 @@ ARGUS_API int argus_hip_quant_flush(argus_hip_ctx *ctx, const argus_hip_quant_fl
                       a->flush_tokens, a->res_cap);
   if ((a->qk_mem | a->qv_mem) & 3 || (a->res_v_mem & 15))
     return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "quant_flush: misaligned buffer");
+  if (a->out_res_cap && (a->out_res_cap % kUnit || a->flush_tokens % a->out_res_cap))
+    return argus_fail(ctx, ARGUS_HIP_ERR_INVALID, "quant_flush: out_res_cap %zu does not divide flush_tokens %zu into whole groups",
+                      a->out_res_cap, a->flush_tokens);
   if (a->flush_tokens == 0) return ARGUS_HIP_OK;
   hipStream_t stream = (hipStream_t)a->stream;
   const int n_groups = (int)(a->flush_tokens / kUnit);
+  const int out_cap = (int)(a->out_res_cap ? a->out_res_cap : a->flush_tokens);
   const int64_t nk = (int64_t)a->kv_heads * n_groups * a->head_dim;
   const int64_t nv = (int64_t)a->kv_heads * a->flush_tokens * (a->head_dim / kUnit);
   const dim3 gk((unsigned)((nk + 127) / 128)), gv((unsigned)((nv + 127) / 128));
 #define ARGUS_FLUSH(B)                                                                                              \
   hipLaunchKernelGGL((kivi_flush_k_kernel<B>), gk, dim3(128), 0, stream, (const float *)a->res_k_mem,               \
                      (uint8_t *)a->qk_mem, (int)a->kv_heads, (int)a->res_cap, (int)a->head_dim, n_groups,           \
-                     (int64_t)a->k_block_start);                                                                    \
+                     (int64_t)a->k_block_start, out_cap / kUnit);                                                   \
   hipLaunchKernelGGL((kivi_flush_v_kernel<B>), gv, dim3(128), 0, stream, (const float *)a->res_v_mem,               \
                      (uint8_t *)a->qv_mem, (int)a->kv_heads, (int)a->res_cap, (int)a->head_dim, (int)a->flush_tokens, \
-                     (int64_t)a->v_block_start)
+                     (int64_t)a->v_block_start, out_cap)
   switch (a->bits) {
     case 2: ARGUS_FLUSH(2); break;
     case 4: ARGUS_FLUSH(4); break;

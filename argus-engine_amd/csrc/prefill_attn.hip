@@ -887,6 +887,13 @@ ARGUS_API int argus_hip_flash_attention_prefill(argus_hip_ctx *ctx, const argus_
   // for |v| >= 4: over the bar in a few rows per thousand random cases.  A second pass over the same
   // logits with V's rounding remainder restores the f32 values (F32 outputs; an F16 output rounds by
   // more than that itself).
+  // (one timing bracket over both launches: an F32 cache with F32 output costs two passes)
+  KernelTimer both(ctx, stream);
+  struct Hold {
+    argus_hip_ctx *c;
+    ~Hold() { c->timer_held = false; }
+  } hold{ctx};
+  ctx->timer_held = true;
   const int rc = dispatch_dim<float>(ctx, p, a->head_dim, stream);
   if (rc != 1 || p.out_f16) return rc;
   p.v_residual = 1;

@@ -367,8 +367,9 @@ struct QuantWindowRawBuffers {
 // CACHE-category handle (argus_hip_quant_cache_*, the C form of QuantCacheBackend,
 // crates/argus-extension-api/src/lib.rs:2017-2035): an F32 residual ring that new tokens are
 // appended to and the two block streams it is quantised into when full, every step on the device.
-// Flush metrics (QCF / AWQE proxies) and the unquantised bits = 16 mode are host bookkeeping of
-// the reference with no device part and are not mirrored.
+// bits = 16 is the unquantised mode (residual of max_seq_len rows, which is also the view) with the
+// transitions to and from the quantised widths.  Flush metrics (QCF / AWQE proxies) are host
+// bookkeeping of the reference with no device part and are not mirrored.
 class HipQuantWindowCache {
  public:
   static Result<std::unique_ptr<HipQuantWindowCache>> new_gpu(HipBackend *be, size_t kv_heads, size_t head_dim, size_t max_seq_len,
@@ -432,13 +433,17 @@ class HipQuantWindowCache {
     return rc == 0 ? OkStatus() : Status::Err("attention_gen_quant failed (rc=" + std::to_string(rc) + "): " + be_->last_error());
   }
 
-  // get_view_gpu: F16 [max_seq_len, kv_heads, head_dim] views covering [0, current_pos).
+  // get_view_gpu: F16 [max_seq_len, kv_heads, head_dim] views covering [0, current_pos); while bits = 16
+  // the F32 residual itself, [1, kv_heads, max_seq_len, head_dim] (quant_window_cache.rs:2417-2429).
   Result<std::pair<Tensor, Tensor>> get_view_gpu() {
     using R = Result<std::pair<Tensor, Tensor>>;
     argus_hip_quant_cache_view_out o{};
     const int rc = argus_hip_quant_cache_assemble_view(h_, &o);
     if (rc != 0) return R::Err("assemble_view failed (rc=" + std::to_string(rc) + "): " + be_->last_error());
-    Tensor tk{o.k_mem, DType::F16, {1, max_seq_len_, kv_heads_, head_dim_}, true}, tv = tk;
+    const bool residual = o.layout == ARGUS_HIP_VIEW_HEADS_TOKENS_DIM;
+    Tensor tk{o.k_mem, residual ? DType::F32 : DType::F16,
+              residual ? std::vector<size_t>{1, kv_heads_, max_seq_len_, head_dim_} : std::vector<size_t>{1, max_seq_len_, kv_heads_, head_dim_}, true};
+    Tensor tv = tk;
     tv.ptr = o.v_mem;
     return R::Ok(std::make_pair(tk, tv));
   }

@@ -323,6 +323,13 @@ typedef struct argus_hip_quant_flush_args {
   size_t k_block_start;
   size_t v_block_start;
   uint8_t bits;
+  /* 0: the blocks of this call form one flush (order h -> group -> ch / h -> token -> block, as the
+   * CPU loop pushes them).  Otherwise a multiple of 32 that divides flush_tokens: the blocks are laid
+   * out as flush_tokens / out_res_cap consecutive flushes of a ring of that capacity, the order every
+   * reader assumes for a cache whose res_cap is out_res_cap (kivi_attn.cu:71-77, 173-177;
+   * quant_window_cache.rs:1463-1540).  Used by the 16 -> Q transition of the container, which
+   * quantises a residual of many groups in one go and continues with a ring of 32. */
+  size_t out_res_cap;
 } argus_hip_quant_flush_args;
 int argus_hip_quant_flush(argus_hip_ctx *ctx, const argus_hip_quant_flush_args *args);
 
@@ -391,8 +398,21 @@ int argus_hip_quant_scatter_residual(argus_hip_ctx *ctx, const argus_hip_quant_s
  * step on the device.  A handle allocates its ring and streams at `make` (sized for max_seq_len),
  * the F16 view at the first assemble_view, and new streams at a width transition; nothing else.
  * Work functions return 0 or a negative ARGUS_HIP_ERR_* (text in argus_hip_last_error of the context
- * given at make).  Widths 2, 4 and 8; bits = 16 (the unquantised fallback) is refused. */
+ * given at make).
+ * bits = 16 is the unquantised mode of the reference container (quant_window_cache.rs:292-300, 410-446,
+ * 2417-2429): the residual covers max_seq_len tokens, nothing is flushed, the view IS the residual
+ * (F32, [kv_heads, max_seq_len, head_dim], layout tag ARGUS_HIP_VIEW_HEADS_TOKENS_DIM) and there is no
+ * raw-buffer set.  transition_bits(16 -> b) quantises every full group of 32 on the device and
+ * continues with a ring of 32 tokens (quant_window_cache.rs:1140-1306; the block streams come out in
+ * the order a ring of 32 produces, which is what the readers assume -- the reference pushes h -> group
+ * -> ch over all groups at once, the same order only for one KV head); transition_bits(b -> 16)
+ * refills the residual from the F16 view, as the reference's GPU mode does (988-1034), and releases
+ * the view and the block streams.
+ * The context given at make must outlive the handle; `make` checks that the pointer is an
+ * argus_hip_ctx (a tag word at its head) and returns NULL for anything else -- a host that fills the
+ * slot with a context of its own kind passes NULL instead and the handle creates one. */
 #define ARGUS_HIP_VIEW_TOKENS_HEADS_DIM 0u /* ViewLayoutTag::HeadMajor of lib.rs:1917-1926: [tokens, kv_heads, head_dim] */
+#define ARGUS_HIP_VIEW_HEADS_TOKENS_DIM 1u /* ViewLayoutTag::SeqMajor: [kv_heads, tokens, head_dim]; bits = 16 only */
 typedef struct argus_hip_quant_cache_make_args {
   void *ctx;              /* cl_ctx slot: the argus_hip_ctx the cache allocates from and launches on; NULL: a
                              context of its own on the current device, destroyed with the handle */
@@ -402,20 +422,20 @@ typedef struct argus_hip_quant_cache_make_args {
   size_t kv_heads;
   size_t head_dim;      /* multiple of 32 */
   size_t max_seq_len;
-  size_t residual_size; /* positive multiple of 32 */
-  uint8_t bits;         /* 2, 4 or 8 */
+  size_t residual_size; /* positive multiple of 32 (not used while bits = 16) */
+  uint8_t bits;         /* 2, 4, 8 or 16 */
 } argus_hip_quant_cache_make_args;
 typedef struct argus_hip_quant_cache_update_args {
-  void *stream;   /* may be NULL: the handle's stream */
+  void *stream;   /* NULL or the stream given at make (the handle works on one stream) */
   void *k_in_mem; /* device F32 [seq_len, kv_heads, head_dim] */
   void *v_in_mem;
   size_t seq_len; /* 1 = decode, > 1 = prefill batch */
 } argus_hip_quant_cache_update_args;
 typedef struct argus_hip_quant_cache_view_out {
-  void *k_mem; /* F16 [max_seq_len, kv_heads, head_dim], rows [0, tokens) valid */
+  void *k_mem; /* F16 [max_seq_len, kv_heads, head_dim], rows [0, tokens) valid; bits = 16: the F32 residual */
   void *v_mem;
   size_t tokens;
-  uint32_t layout; /* ARGUS_HIP_VIEW_TOKENS_HEADS_DIM */
+  uint32_t layout; /* ARGUS_HIP_VIEW_TOKENS_HEADS_DIM, or ARGUS_HIP_VIEW_HEADS_TOKENS_DIM while bits = 16 */
 } argus_hip_quant_cache_view_out;
 typedef struct argus_hip_quant_cache_raw_buffers_out {
   void *qk_mem;
@@ -434,7 +454,7 @@ uint8_t argus_hip_quant_cache_current_bits(void *handle);
 int32_t argus_hip_quant_cache_update(void *handle, const argus_hip_quant_cache_update_args *args);
 int32_t argus_hip_quant_cache_flush_if_full(void *handle);
 int32_t argus_hip_quant_cache_assemble_view(void *handle, argus_hip_quant_cache_view_out *out);
-/* false (out untouched) when there is no native-consumable set: an empty cache. */
+/* false (out untouched) when there is no native-consumable set: an empty cache, or bits = 16. */
 bool argus_hip_quant_cache_get_raw_buffers(void *handle, argus_hip_quant_cache_raw_buffers_out *out);
 int32_t argus_hip_quant_cache_transition_bits(void *handle, uint8_t target_bits);
 void argus_hip_quant_cache_drop(void *handle);

@@ -513,7 +513,18 @@ static void test_quant_window_cache(HipBackend &be) {
       for (float x : got) finite = finite && std::isfinite(x);
       CHECK(finite, "attention after the transition is finite");
     }
-    CHECK(!c.transition_bits(16).ok(), "bits 16 refused");
+    // up to the unquantised mode and down again: positions kept, raw buffers only while quantised
+    CHECK(c.transition_bits(16).ok() && c.bits() == 16 && c.current_pos() == total && !c.get_raw_gpu_buffers().ok(), "transition to bits 16");
+    {
+      auto view = c.get_view_gpu();
+      CHECK(view.ok() && view.value().first.dtype == DType::F32 && view.value().first.dims[1] == hkv, "bits 16: the residual is the view");
+    }
+    CHECK(c.transition_bits(bits).ok() && c.bits() == bits && c.current_pos() == total, "transition back from bits 16");
+    {
+      auto raw = c.get_raw_gpu_buffers();
+      CHECK(raw.ok() && raw.value().res_cap == 32 && raw.value().q_tokens == total / 32 * 32, "ring of 32 after the transition");
+    }
+    CHECK(!c.transition_bits(5).ok(), "width 5 refused");
     CHECK(c.reset().ok() && c.current_pos() == 0 && !c.get_raw_gpu_buffers().ok(), "reset");
   }
   printf("[kivi] quant-window container on the device: update / flush / raw buffers / fused attention / F16 view ok (bits 2, 4, 8)\n");

@@ -404,7 +404,7 @@ def test_quant_cache_capability_through_the_c_abi(bits):
     k[:, 1, 9] *= 15.0
     q = rng.standard_normal((hq, d)).astype(np.float32)
     kd, vd, qd = dev(k), dev(v), dev(q)
-    assert ctx().quant_cache(hkv, d, max_seq, R, 16) is None           # the unquantised fallback is refused
+    assert ctx().quant_cache(hkv, d, max_seq, R, 3) is None            # widths 2, 4, 8 and 16 only
     assert ctx().quant_cache(hkv, d, max_seq, 48, bits) is None        # residual_size must be a multiple of 32
     c = ctx().quant_cache(hkv, d, max_seq, R, bits)
     assert c is not None and c.current_pos() == 0 and c.capacity() == max_seq and c.current_bits() == bits
@@ -454,12 +454,132 @@ def test_quant_cache_capability_through_the_c_abi(bits):
         ref = dict(ref, qk=O.kivi_requant(ref["qk"], old, nb), qv=O.kivi_requant(ref["qv"], old, nb), bits=nb)
         check_at(total, nb, ref)
     assert c.transition_bits(c.current_bits()) == 0                     # no-op
-    assert c.transition_bits(16, check=False) == A.ERR_UNSUPPORTED
+    assert c.transition_bits(5, check=False) == A.ERR_UNSUPPORTED
     assert c.update(dev(np.zeros((max_seq, hkv, d), np.float32)), dev(np.zeros((max_seq, hkv, d), np.float32)), check=False) == A.ERR_INVALID
     c.close()
     e = ctx().quant_cache(hkv, d, max_seq, R, 8)                        # test_kivi_transition_empty: no tokens, just the format
     assert e.transition_bits(2) == 0 and e.current_bits() == 2 and e.current_pos() == 0
     e.close()
+
+
+def _flushed_ring_of_32(k, v, bits):
+    """What a container with a ring of 32 tokens holds once every full group has been flushed: the
+    state after transition_bits(16 -> bits).  (A dummy token triggers the lazy flush of a full ring
+    and is dropped again.)"""
+    n, hkv, d = k.shape
+    if n % 32 == 0 and n > 0:
+        z = np.zeros((1, hkv, d), np.float32)
+        ref = O.kivi_build(np.concatenate([k, z]), np.concatenate([v, z]), 32, bits)
+        assert ref["q_tokens"] == n and ref["res_tokens"] == 1
+        ref["res_tokens"] = 0
+        return ref
+    return O.kivi_build(k, v, 32, bits)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("n", [32 * 5 + 9, 32 * 4, 7])
+def test_quant_cache_unquantised_mode_and_its_transitions(bits, n):
+    # bits = 16 (engine/src/kv/quant_window_cache.rs:292-300, 845-848, 2417-2429; tests 3695-3900):
+    # the residual spans max_seq_len and is the view, nothing is flushed, no raw-buffer set.
+    # 16 -> b quantises every full group and goes on with a ring of 32 (1137-1306); b -> 16 refills the
+    # residual from the F16 view (988-1034).  Blocks bit for bit against the CPU container with a ring
+    # of 32, views against the oracle's.
+    import torch
+    hq, hkv, d, max_seq = 8, 2, 128, 320
+    rng = np.random.default_rng(1600 + bits + n)
+    k = rng.standard_normal((n + 40, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((n + 40, hkv, d)).astype(np.float32)
+    k[:, 1, 9] *= 15.0
+    q = rng.standard_normal((hq, d)).astype(np.float32)
+    kd, vd, qd = dev(k), dev(v), dev(q)
+    c = ctx().quant_cache(hkv, d, max_seq, 64, 16)
+    assert c is not None and c.current_bits() == 16 and c.capacity() == max_seq
+    c.update(kd[:n], vd[:n])
+    assert c.current_pos() == n and c.flush_if_full() == 0 and c.current_pos() == n
+    assert c.get_raw_buffers() is None
+    view = c.assemble_view()
+    assert view.tokens == n and view.layout == 1
+    rk = _read_dev(view.k_mem, hkv * max_seq * d * 4).view(np.float32).reshape(hkv, max_seq, d)
+    rv = _read_dev(view.v_mem, hkv * max_seq * d * 4).view(np.float32).reshape(hkv, max_seq, d)
+    assert np.array_equal(rk[:, :n], k[:n].transpose(1, 0, 2)) and np.array_equal(rv[:, :n], v[:n].transpose(1, 0, 2))
+    assert c.transition_bits(16) == 0                                    # no-op
+
+    def check_quantised(ref, n_now, cur_bits):
+        raw = c.get_raw_buffers()
+        assert c.current_pos() == n_now and c.current_bits() == cur_bits
+        if n_now == 0:
+            assert raw is None
+            return
+        assert (raw.q_tokens, raw.res_tokens, raw.res_cap, raw.bits) == (ref["q_tokens"], ref["res_tokens"], 32, cur_bits)
+        used = ref["q_tokens"] * hkv * d // 32 * O.kivi_block_bytes(cur_bits)
+        if used:
+            assert np.array_equal(_read_dev(raw.qk_mem, used), ref["qk"][:used]), "key blocks"
+            assert np.array_equal(_read_dev(raw.qv_mem, used), ref["qv"][:used]), "value blocks"
+        ring = _read_dev(raw.res_k_mem, hkv * 32 * d * 4).view(np.float32).reshape(hkv, 32, d)
+        assert np.array_equal(ring[:, :ref["res_tokens"]], ref["res_k"][:, :ref["res_tokens"]])
+        out = torch.empty((hq, d), device="cuda")
+        ctx().attention_gen_quant(qd, _Raw(raw.qk_mem, torch.uint8), _Raw(raw.qv_mem, torch.uint8), _Raw(raw.res_k_mem, torch.float32),
+                                  _Raw(raw.res_v_mem, torch.float32), out, hkv, raw.q_tokens, raw.res_tokens, raw.res_cap,
+                                  1.0 / np.sqrt(d), cur_bits)
+        check_attention_out(host(out), O.kivi_attention(q, ref, 1.0 / np.sqrt(d)))
+        vw = c.assemble_view()
+        assert vw.tokens == n_now and vw.layout == 0
+        gk = _read_dev(vw.k_mem, n_now * hkv * d * 2).view(np.float16).reshape(n_now, hkv, d)
+        ak, av = O.kivi_assemble_view(ref)
+        assert np.array_equal(gk, ak.astype(np.float16))
+
+    # 16 -> b
+    assert c.transition_bits(bits) == 0
+    ref = _flushed_ring_of_32(k[:n], v[:n], bits)
+    check_quantised(ref, n, bits)
+    # the cache keeps working with its ring of 32: forty more tokens, one at a time
+    for t in range(n, n + 40):
+        c.update(kd[t:t + 1], vd[t:t + 1])
+    ref = O.kivi_build(k[:n + 40], v[:n + 40], 32, bits)
+    if n % 32 == 0:  # the transition flushed a ring the lazy rule would have kept full for one more token
+        assert ref["q_tokens"] == c.get_raw_buffers().q_tokens
+    check_quantised(ref, n + 40, bits)
+    # b -> 16: every token back in the residual, through the F16 view
+    ak, av = O.kivi_assemble_view(ref)
+    assert c.transition_bits(16) == 0 and c.current_bits() == 16 and c.current_pos() == n + 40
+    assert c.get_raw_buffers() is None
+    view = c.assemble_view()
+    assert view.tokens == n + 40 and view.layout == 1
+    rk = _read_dev(view.k_mem, hkv * max_seq * d * 4).view(np.float32).reshape(hkv, max_seq, d)[:, :n + 40]
+    rv = _read_dev(view.v_mem, hkv * max_seq * d * 4).view(np.float32).reshape(hkv, max_seq, d)[:, :n + 40]
+    k16 = ak.astype(np.float16).astype(np.float32).transpose(1, 0, 2)
+    v16 = av.astype(np.float16).astype(np.float32).transpose(1, 0, 2)
+    assert np.array_equal(rk, k16) and np.array_equal(rv, v16)
+    # and down again at another width, from the restored values
+    nb = 4 if bits != 4 else 8
+    assert c.transition_bits(nb) == 0
+    ref2 = _flushed_ring_of_32(np.ascontiguousarray(k16.transpose(1, 0, 2)), np.ascontiguousarray(v16.transpose(1, 0, 2)), nb)
+    check_quantised(ref2, n + 40, nb)
+    c.close()
+    e = ctx().quant_cache(hkv, d, max_seq, 64, 16)                       # empty cache: only the format changes
+    assert e.transition_bits(bits) == 0 and e.current_bits() == bits and e.current_pos() == 0 and e.get_raw_buffers() is None
+    e.update(kd[:3], vd[:3])
+    assert e.get_raw_buffers().res_cap == 32 and e.transition_bits(16) == 0 and e.assemble_view().tokens == 3
+    e.close()
+
+
+def test_quant_cache_make_refuses_a_foreign_context_and_another_stream():
+    # the ctx slot of the make arguments is untyped (the reference's cl_context): only this library's
+    # contexts are accepted; and a handle works on the stream it was made with
+    import argus_hip as A
+    import torch
+    junk = (C.c_uint64 * 64)(*([0x1234567890] * 64))
+    a = A.QuantCacheMakeArgs(ctx=C.addressof(junk), device=None, stream=None, build_opts=None, kv_heads=2, head_dim=64,
+                             max_seq_len=128, residual_size=32, bits=4)
+    assert not A.lib.argus_hip_quant_cache_make(C.byref(a))
+    c = ctx().quant_cache(2, 64, 128, 32, 4)
+    x = torch.zeros((1, 2, 64), device="cuda")
+    other = torch.cuda.Stream()
+    u = A.QuantCacheUpdateArgs(stream=other.cuda_stream, k_in_mem=x.data_ptr(), v_in_mem=x.data_ptr(), seq_len=1)
+    assert A.lib.argus_hip_quant_cache_update(c.handle, C.byref(u)) == A.ERR_INVALID
+    c.update(x, x)
+    assert c.current_pos() == 1
+    c.close()
 
 
 def test_plugin_protocol_end_to_end():
