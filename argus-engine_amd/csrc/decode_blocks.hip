@@ -43,6 +43,7 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32_a2 __attribute__((aligned(2)));  // code words sit at 2-byte boundaries (18- and 34-byte blocks)
 
 enum { kFmtQ4_0 = 0, kFmtQ4_1 = 1, kFmtQ8_0 = 2, kFmtQ2_0 = 3 };
+constexpr int kBufferFlags = 0x00020000;  // raw buffer, bounds-checked against num_records
 
 // Orders a wave's LDS accesses for the compiler when its lanes exchange data through LDS.
 __device__ __forceinline__ void wave_lds_fence() {
@@ -398,26 +399,22 @@ struct BlockShape {
 // q8_0 would spill there and stays at 2), 2 at 256.  Without the bound most instantiations came out a
 // few registers on one or the other side of a step depending on unrelated edits (q4_0 at 128: 165 or
 // 170 registers; q8_0 at 256: 256 or 257).
-// Row (16 lanes) i of the wave takes v[i].
-__device__ __forceinline__ float row_pick(const float4_t &v) {
-  // The elements are copied out as floats first: __builtin_bit_cast applied to a vector element
-  // directly read element 0 whatever the index.
-  const float f0 = v[0], f1 = v[1], f2 = v[2], f3 = v[3];
-  int x = __builtin_bit_cast(int, f0);
-  x = __builtin_amdgcn_update_dpp(x, __builtin_bit_cast(int, f1), 0xe4, 0x2, 0xf, false);
-  x = __builtin_amdgcn_update_dpp(x, __builtin_bit_cast(int, f2), 0xe4, 0x4, 0xf, false);
-  x = __builtin_amdgcn_update_dpp(x, __builtin_bit_cast(int, f3), 0xe4, 0x8, 0xf, false);
-  return __builtin_bit_cast(float, x);
-}
-
 // TOKCOL (at most four query heads per KV head): the logits MFMA takes the
-// query as its row operand, head r % 4 in row r, and the codes as its column operand, so result lane
-// (j, n) holds token n of the tile for the heads 0..3 in its four registers, the same in every lane
-// group.  Lane group j keeps head j: the token's block scales are the lane's own (no exchange), the
+// query as its row operand, head r / 4 in row r, and the codes as its column operand, so result lane
+// (g, n) holds token n of the tile for head g in each of its four registers (rows 4g..4g+3).  Lane
+// group g keeps head g: the token's block scales are the lane's own (no exchange), the
 // softmax runs once per logit instead of once per operand column, a head's maximum is a reduction
 // inside one 16-lane row, and the probabilities reach the P operand's layout (lane (j, r): tokens
 // 4j..4j+3 of head r % 4) through 256 bytes of LDS per wave.
-template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, bool TOKCOL>
+//
+// STREAM (rows packed back to back, no index list): a wave's tile is one contiguous run of bytes.
+// The per-lane block requests of the other path put a header and 16 or 32 code bytes at an 18- or
+// 34-byte stride under every lane, which the texture path serves lane by lane: the q4_0 kernel made
+// as many L1 accesses as the F16 kernel for 3.6 times fewer bytes (17 per 128-byte line, counter
+// TCP_TOTAL_CACHE_ACCESSES against TCP_TCC_READ_REQ).  Here the lanes fetch consecutive dwords of
+// the run (one access per 64 bytes), park them in a wave-private LDS copy of the tile, and every lane
+// then reads the pieces of its MFMA operands straight from there: no trades between lanes at all.
+template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, bool TOKCOL, bool STREAM>
 __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
@@ -431,7 +428,12 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane >> 4, r = lane & 15;
   const int G = p.group;
-  const int rh = TOKCOL ? (r & 3) : r;  // head whose query this lane's operand row (or column) carries
+  // Head whose query this lane's operand row (or column) carries.  TOKCOL: rows 4g..4g+3 all carry
+  // head g, so the four registers of a result lane in lane group g all hold head g's logit and no
+  // register has to be picked; the P operand of the output MFMAs has head r % 4 in row r.
+  const int rh = TOKCOL ? (r >> 2) : r;
+  const int ph = r & 3;
+  static_assert(!(STREAM && INDEXED), "an index list gathers rows: they are read block by block");
 
   const int t_begin = split * p.chunk;
   const int t_end = min(p.len, t_begin + p.chunk);
@@ -463,6 +465,104 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   constexpr int VL = (D == 64) ? 1 : TW * VSEG;
   RawPiece<FMT> vraw[TW][VSEG][kStageV ? 1 : 4];
   RawBlock<FMT> vblk_raw[kStageV ? VL : 1];
+  // STREAM: the tile as dwords in flight, and its LDS copy per wave (K and V apart, so the V copy
+  // can be made while the K pieces are still being read).  A request past the attended rows returns
+  // zeros (bounds-checked descriptor), so every request is unconditional here too.
+  constexpr int RBY = KK * F::BB;                  // bytes per packed row
+  static_assert(RBY % 4 == 0, "rows are whole dwords");
+  constexpr int RD = RBY / 4;                      // dwords per row
+  constexpr int NLD = (TILE * RD + 63) / 64;       // wave-wide dword requests per tile
+  uint32_t kst[STREAM ? NLD : 1], vst[STREAM ? NLD : 1];
+  // The copies live in the dynamic area behind whatever the token loop keeps there (the staged
+  // logits, or the spare slots of lanes that park nothing); the merge at the end reuses all of it.
+  constexpr int kTileDw = NLD * 64 + 4;  // the last request may run past the tile; a piece's second dword past a row
+  extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
+  const int stage_row = p.chunk + 4;
+  const int staged_heads = p.stage_scores ? p.group : 0;
+  constexpr int kSpareFloats = 64 * kWaves * TW * 4;  // 16 TW bytes per lane
+  uint32_t *const tiles = (uint32_t *)(dyn_lds + (p.stage_scores ? staged_heads * stage_row : kSpareFloats));
+  uint32_t *const k_tile = tiles + wave * kTileDw, *const v_tile = tiles + (kWaves + wave) * kTileDw;
+  const uint32_t run_bytes = (uint32_t)min((int64_t)p.len * RBY, (int64_t)0xffffffffll);
+  const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void *)kb, 0, STREAM ? run_bytes : 0u, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc((void *)vb, 0, STREAM ? run_bytes : 0u, kBufferFlags);
+  auto fetch_run = [&](__amdgpu_buffer_rsrc_t rs, int base, uint32_t (&st)[STREAM ? NLD : 1]) {
+    const uint32_t off = (uint32_t)min(base, p.len) * (uint32_t)RBY;  // scalar; past the end everything reads as zero
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) st[c] = __builtin_amdgcn_raw_buffer_load_b32(rs, 4u * (uint32_t)lane + 256u * (uint32_t)c, off, 0);
+  };
+  auto park_run = [&](uint32_t *tile, const uint32_t (&st)[STREAM ? NLD : 1]) {
+    wave_lds_fence();  // the reads of the tile before are done
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) tile[64 * c + lane] = st[c];
+    wave_lds_fence();
+  };
+  // Piece (code index x, CW dwords) of block blk of a parked row.  With a 2-byte header the code
+  // words of every other block straddle dwords: `sh` = 2 there, 0 where they are aligned.
+  auto parked_piece = [&](const uint32_t *row, uint32_t blk_byte, uint32_t code_dw, uint32_t sh) {
+    RawPiece<FMT> pc;
+    if constexpr (F::HDR == 4) {
+      pc.hdr = row[blk_byte / 4];
+#pragma unroll
+      for (int w = 0; w < F::CW; ++w) pc.code[w] = row[code_dw + w];
+    } else {
+      pc.hdr = *(const uint16_t *)((const uint8_t *)row + blk_byte);
+      uint32_t d[F::CW + 1];
+#pragma unroll
+      for (int w = 0; w <= F::CW; ++w) d[w] = row[code_dw + w];
+#pragma unroll
+      for (int w = 0; w < F::CW; ++w) pc.code[w] = __builtin_amdgcn_alignbyte(d[w + 1], d[w], sh);
+    }
+    return pc;
+  };
+  // K operand piece of token r of tile tw: code index j of block kk (q2_0: the dword that holds half j)
+  auto k_piece = [&](int tw, int kk) {
+    const uint32_t *row = k_tile + (16 * tw + r) * RD;
+    const uint32_t blk = (uint32_t)(kk * F::BB);
+    if constexpr (F::HDR == 4) {
+      return parked_piece(row, blk, blk / 4 + 1 + ((FMT == kFmtQ2_0) ? (uint32_t)(j >> 1) : (uint32_t)(F::CW * j)), 0u);
+    } else {
+      const uint32_t a = blk + 2u + 4u * (uint32_t)(F::CW * j);  // first code byte; a % 4 is the block's, known at compile time
+      RawPiece<FMT> pc;
+      pc.hdr = *(const uint16_t *)((const uint8_t *)row + blk);
+      if ((kk * F::BB) % 4 == 0) {
+        uint32_t d[F::CW + 1];
+#pragma unroll
+        for (int w = 0; w <= F::CW; ++w) d[w] = row[a / 4 + w];
+#pragma unroll
+        for (int w = 0; w < F::CW; ++w) pc.code[w] = __builtin_amdgcn_alignbyte(d[w + 1], d[w], 2u);
+      } else {
+#pragma unroll
+        for (int w = 0; w < F::CW; ++w) pc.code[w] = row[a / 4 + w];
+      }
+      return pc;
+    }
+  };
+  // V piece of token 4j + e of tile tw: block vblk[sg], code index r % 4 (head_dim 64, q8_0: the
+  // lane's half of the piece, one dword); the lane's offsets into a row are fixed
+  uint32_t v_blk_byte[VSEG], v_code_dw[VSEG], v_sh[VSEG];
+#pragma unroll
+  for (int sg = 0; sg < VSEG; ++sg) {
+    const uint32_t blk = (uint32_t)(vblk[sg] * F::BB);
+    uint32_t a;  // first code byte of the piece
+    if constexpr (FMT == kFmtQ2_0) a = blk + 4u + 4u * (uint32_t)((r & 3) >> 1);
+    else if constexpr (FMT == kFmtQ8_0 && D == 64) a = blk + (uint32_t)F::HDR + 4u * (uint32_t)(2 * (r & 3) + (r >> 3));
+    else a = blk + (uint32_t)F::HDR + 4u * (uint32_t)(F::CW * (r & 3));
+    v_blk_byte[sg] = blk;
+    v_code_dw[sg] = a / 4;
+    v_sh[sg] = a & 3u;
+  }
+  auto v_piece = [&](int tw, int sg, int e) {
+    const uint32_t *row = v_tile + (16 * tw + 4 * j + e) * RD;
+    if constexpr (FMT == kFmtQ8_0 && D == 64) {  // half a piece: one code dword
+      RawPiece<FMT> pc;
+      pc.hdr = *(const uint16_t *)((const uint8_t *)row + v_blk_byte[sg]);
+      pc.code[0] = __builtin_amdgcn_alignbyte(row[v_code_dw[sg] + 1], row[v_code_dw[sg]], v_sh[sg]);
+      pc.code[1] = 0u;
+      return pc;
+    } else {
+      return parked_piece(row, v_blk_byte[sg], v_code_dw[sg], v_sh[sg]);
+    }
+  };
   // Rows past the chunk re-read its last row (they are masked below), so every request is
   // unconditional and a tile may be asked for before it is known to exist.
   const int last = t_end - 1;
@@ -503,7 +603,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     else return (uint32_t)v_tok(base, i);
   };
   auto load_k = [&](int base) {
-    if constexpr (D == 64) {
+    if constexpr (STREAM) {
+      fetch_run(k_rs, base, kst);
+    } else if constexpr (D == 64) {
       const uint32_t off = __umul24(k_rowof(base, 0), row_bytes);
       kblk[0] = load_block<FMT>(kb, off + (uint32_t)((j & 1) * F::BB));
     } else {
@@ -516,7 +618,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     }
   };
   auto load_v = [&](int base) {
-    if constexpr (kStageV && D == 64) {
+    if constexpr (STREAM) {
+      fetch_run(v_rs, base, vst);
+    } else if constexpr (kStageV && D == 64) {
       const uint32_t off = __umul24(v_rowof(base, 0), row_bytes);
       vblk_raw[0] = load_block<FMT>(vb, off + (uint32_t)(((r >> 2) & 1) * F::BB));
     } else {
@@ -582,12 +686,12 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       // the four lane groups hold the four quarters of the block
       part += __shfl_xor(part, 16, 64);
       part += __shfl_xor(part, 32, 64);
-      if constexpr (TOKCOL) part = __shfl(part, j, 64);  // the sums of head j, whose logits this lane keeps
+      if constexpr (TOKCOL) part = __shfl(part, 4 * j, 64);  // the sums of head j, whose logits this lane keeps
       qsum[kk] = part;
       if constexpr (FMT == kFmtQ2_0) {
         biased += __shfl_xor(biased, 16, 64);
         biased += __shfl_xor(biased, 32, 64);
-        if constexpr (TOKCOL) biased = __shfl(biased, j, 64);
+        if constexpr (TOKCOL) biased = __shfl(biased, 4 * j, 64);
         qinit[kk] = -biased;
       } else {
         qinit[kk] = -(CD::kBias + CD::kZero) * part;
@@ -616,9 +720,6 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
   // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
   // then the merge area.
-  extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
-  const int stage_row = p.chunk + 4;
-  const int staged_heads = p.stage_scores ? p.group : 0;
   __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
   // Lanes that park nothing write here: the sink's stage when the logits are staged (the sink is off
   // then), else the start of the dynamic area (the merge uses it after the loop only).
@@ -626,6 +727,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   float *spare = p.stage_scores ? &logit_stage[0][0] : dyn_lds;
   const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
   int base_last = -(1 << 30);
+  __shared__ uint32_t v_strip[kWaves][VL][(kStageV && !STREAM) ? 64 * 4 + 4 * 4 : 1];  // the staged V rows' code words, wave by wave
 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
     half4_t pa[TW];
@@ -633,12 +735,18 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       // ---- logits: token base + 16 tw + r, head j ------------------------------------------------
       float sc[TW];
       RawPiece<FMT> both[4];  // head_dim 64: lane group g held block g % 2 of tile g / 2
-      if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
+      if constexpr (STREAM) {
+        park_run(k_tile, kst);
+        load_k(base + kWaves * TILE);  // the dwords are parked: request the wave's next tile
+      } else if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
         sc[tw] = 0.0f;
         RawPiece<FMT> kpc[KK];
-        if constexpr (D == 64) {
+        if constexpr (STREAM) {
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) kpc[kk] = k_piece(tw, kk);
+        } else if constexpr (D == 64) {
           kpc[0] = both[2 * tw];
           kpc[1] = both[2 * tw + 1];
         } else {
@@ -659,13 +767,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q, times the
           // token's scale for this block, which the lane holds itself
           const half2_t dm = __builtin_bit_cast(half2_t, kpc[kk].hdr);
-          const float mine = row_pick(dot) + qinit[kk];
+          const float mine = dot[0] + qinit[kk];
           if constexpr (F::kHasMin) sc[tw] = fmaf((float)dm[0], mine, fmaf((float)dm[1], qsum[kk], sc[tw]));
           else sc[tw] = fmaf((float)dm[0], mine, sc[tw]);
         }
       }
       if constexpr (D != 64) __builtin_amdgcn_sched_barrier(0);  // (see the other arm)
-      load_k(base + kWaves * TILE);
+      if constexpr (!STREAM) load_k(base + kWaves * TILE);
       load_idx_k(base + 2 * kWaves * TILE);
       float mt = kNegInf;
 #pragma unroll
@@ -732,7 +840,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       wave_lds_fence();  // the previous iteration's reads are done
       p_strip[wave][j][r] = __builtin_bit_cast(uint32_t, pk);
       wave_lds_fence();
-      const u32x4_t w = *(const u32x4_t *)&p_strip[wave][rh][4 * j];
+      const u32x4_t w = *(const u32x4_t *)&p_strip[wave][ph][4 * j];
       typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
@@ -743,12 +851,18 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     // ---- logits ---------------------------------------------------------------------------------
     float4_t s[TW];
     RawPiece<FMT> both[4];  // head_dim 64: lane group g held block g % 2 of tile g / 2
-    if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
+    if constexpr (STREAM) {
+        park_run(k_tile, kst);
+        load_k(base + kWaves * TILE);  // the dwords are parked: request the wave's next tile
+      } else if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       s[tw] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
       RawPiece<FMT> kpc[KK];
-      if constexpr (D == 64) {
+      if constexpr (STREAM) {
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) kpc[kk] = k_piece(tw, kk);
+        } else if constexpr (D == 64) {
         kpc[0] = both[2 * tw];
         kpc[1] = both[2 * tw + 1];
       } else {
@@ -797,7 +911,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     // faster (q2_0 at 128: 146 against 173 us, q4_0 at 256: 137 against 146 us, 32K tokens), the
     // head_dim 64 kernels slower (q4_0: 86 against 82 us).
     if constexpr (D != 64) __builtin_amdgcn_sched_barrier(0);
-    load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
+    if constexpr (!STREAM) load_k(base + kWaves * TILE);  // the K registers are free again: request the wave's next tile
     load_idx_k(base + 2 * kWaves * TILE);
     if constexpr (SOFTCAP) {
       // cap * tanh(logit / cap) on the natural-unit logit (flash_attn_f32_f16.cl:563-565), back to log2 units
@@ -871,13 +985,18 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     }
 
     // ---- O += P . V -----------------------------------------------------------------------------
-#pragma unroll
-    for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-      for (int sg = 0; sg < VSEG; ++sg) {
+    if constexpr (STREAM) {
+      park_run(v_tile, vst);
+      load_v(base + kWaves * TILE);
+    }
+    // The operands of tile tw, V piece sg: bv[c] = channel slot c of the lane's four tokens, hv = their
+    // d (or m) for the header term.
+    auto v_operands = [&](int tw, int sg, half4_t (&bv)[VCH], half4_t &hv) {
         RawPiece<FMT> vpc[4];  // the lane's piece of tokens 4j .. 4j+3
-        if constexpr (kStageV) {
-          __shared__ uint32_t v_strip[kWaves][VL][64 * 4 + 4 * 4];
+        if constexpr (STREAM) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) vpc[e] = v_piece(tw, sg, e);
+        } else if constexpr (kStageV) {
           constexpr bool kShared = D == 64;  // one request serves both tiles
           const RawBlock<FMT> &mine = vblk_raw[kShared ? 0 : tw * VSEG + sg];
           uint32_t *strip = v_strip[wave][kShared ? 0 : tw * VSEG + sg];
@@ -935,18 +1054,25 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           const uint32_t h01 = __builtin_amdgcn_perm(vpc[1].hdr, vpc[0].hdr, sel);
           const uint32_t h23 = __builtin_amdgcn_perm(vpc[3].hdr, vpc[2].hdr, sel);
           typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-          const half4_t hv = __builtin_bit_cast(half4_t, u32x2_t{h01, h23});
-          h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+          hv = __builtin_bit_cast(half4_t, u32x2_t{h01, h23});
         }
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {
-          half4_t bv;
-          if constexpr (kPairV) bv = half4_t{vpair[0][c][0], vpair[0][c][1], vpair[1][c][0], vpair[1][c][1]};
-          else bv = half4_t{vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
-          o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv, o_acc[sg * VCH + c], 0, 0, 0);
+          if constexpr (kPairV) bv[c] = half4_t{vpair[0][c][0], vpair[0][c][1], vpair[1][c][0], vpair[1][c][1]};
+          else bv[c] = half4_t{vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
         }
+    };
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int sg = 0; sg < VSEG; ++sg) {
+        half4_t bv[VCH], hv = {};
+        v_operands(tw, sg, bv, hv);
+        if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < VCH; ++c) o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv[c], o_acc[sg * VCH + c], 0, 0, 0);
       }
-    load_v(base + kWaves * TILE);
+    if constexpr (!STREAM) load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
   if (p.stage_scores) {
@@ -1019,26 +1145,39 @@ template <int FMT, int D>
 int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
   constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
   constexpr int tile_rows = kWaves * 16 * TW;
+  const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
+  const bool tokcol = p.group <= 4;
+  // Packed rows without an index list are streamed (see the kernel); the slabs must start on a dword.
+  const int64_t head_blocks = ((int64_t)p.kv_bs | (int64_t)p.head_stride) / 32;
+  // (Measured per arm: q8_0 +10 % either way, q2_0 +10 % and q4_0 +3 % with tokens as columns; the
+  // tokens-as-rows arm of the 4-bit formats has no registers left for it and ran 3-5 % slower.)
+  const bool stream_rows = !indexed && p.row_stride == D && (((uintptr_t)p.k | (uintptr_t)p.v) & 3) == 0 &&
+                           (head_blocks * BlockFmt<FMT>::BB) % 4 == 0 && (FMT == kFmtQ8_0 || tokcol);
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
-  // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips).
-  constexpr int kStageBytes = 48 * 1024;
+  // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips or the
+  // streamed tiles' LDS copies).
+  constexpr int kTileCopies = 2 * kWaves * (((16 * TW * (D / 32) * BlockFmt<FMT>::BB / 4 + 63) / 64) * 64 + 4) * 4;
+  constexpr int kStageBytes = (kTileCopies > 24 * 1024) ? 32 * 1024 : 48 * 1024;
   constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * BlockShape<D>::MAXH * (D + 4)) * sizeof(float);
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
-  const int wgs_per_cu = argus_wgs_per_cu(ctx, decode_blocks_kernel<FMT, D, TW, false, false, false>, 64 * kWaves,
-                                          max_chunk > 0 ? (size_t)kStageBytes : merge_bytes);
+  auto pick = [&](auto tc, auto st) {
+    constexpr bool TC = decltype(tc)::value, ST = decltype(st)::value;
+    if constexpr (ST && (FMT == kFmtQ8_0 || TC)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
+    else return cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, TC, false> : decode_blocks_kernel<FMT, D, TW, true, false, TC, false>)
+                    : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, TC, false> : decode_blocks_kernel<FMT, D, TW, false, false, TC, false>);
+  };
+  auto kern = stream_rows ? (tokcol ? pick(std::true_type{}, std::true_type{}) : pick(std::false_type{}, std::true_type{}))
+                          : (tokcol ? pick(std::true_type{}, std::false_type{}) : pick(std::false_type{}, std::false_type{}));
+  // dynamic LDS: staged logits or spare slots, then (streamed rows) the tile copies; the merge reuses it
+  constexpr size_t spare_bytes = 64 * kWaves * TW * 16;
+  const size_t tile_bytes = stream_rows ? (size_t)kTileCopies : 0;
+  const int wgs_per_cu = argus_wgs_per_cu(ctx, kern, 64 * kWaves,
+                                          max_chunk > 0 ? (size_t)kStageBytes + tile_bytes : std::max(merge_bytes, spare_bytes + tile_bytes));
   choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   p.direct = 0;
   p.stage_scores = p.scores && p.chunk <= max_chunk;
-  const size_t lds_bytes = std::max(merge_bytes, p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : (size_t)0);
-  const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-  const bool tokcol = p.group <= 4;
-  auto pick = [&](auto tc) {
-    constexpr bool TC = decltype(tc)::value;
-    return cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, TC> : decode_blocks_kernel<FMT, D, TW, true, false, TC>)
-               : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, TC> : decode_blocks_kernel<FMT, D, TW, false, false, TC>);
-  };
-  auto kern = tokcol ? pick(std::true_type{}) : pick(std::false_type{});
-  ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + 1024));
+  const size_t lds_bytes = std::max(merge_bytes, (p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : spare_bytes) + tile_bytes);
+  ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + kTileCopies + 1024));
   const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
   ctx->plan = argus_hip_decode_plan{p.nsplit, p.chunk, wgs_per_cu, (int32_t)lds_bytes, 2, 2, p.stage_scores};

@@ -168,7 +168,10 @@ __global__ __launch_bounds__(64 * WPG * NG, (WPG * NG == 4 && D <= 128) ? ((D ==
   constexpr int CH = NG * BT * D / 8 / NT;   // 16-byte chunks per thread per iteration
   static_assert(CH >= 1 && CH * NT * 8 == NG * BT * D, "tile chunks must divide over the threads");
   constexpr int kLdsAhead = 4;               // MFMA operand reads kept in flight
-  constexpr int kVAhead = (D <= 64) ? 4 : 3;
+#ifndef PF_VAHEAD64
+#define PF_VAHEAD64 4
+#endif
+  constexpr int kVAhead = (D <= 64) ? PF_VAHEAD64 : 3;
 #ifndef PF_VALU_MASK
 #define PF_VALU_MASK 0x402
 #endif
