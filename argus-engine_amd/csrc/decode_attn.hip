@@ -438,7 +438,7 @@ static int attention_gen_impl(argus_hip_ctx *ctx, const argus_hip_attention_gen_
     return dispatch_dim<DescRow>(ctx, p, D, a->batch, want_scores, stream);
   }
   if (blocks) return launch_decode_blocks(ctx, p, D, kv_dtype, a->batch, stream);
-  if (!force_valu && decode_mfma_supported(p, D, kv_dtype)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
+  if (!force_valu && decode_mfma_supported(p, D, kv_dtype, a->batch)) return launch_decode_mfma(ctx, p, D, a->batch, stream);
   switch (kv_dtype) {
     case ARGUS_HIP_F16: return dispatch_dim<_Float16>(ctx, p, D, a->batch, want_scores, stream);
     case ARGUS_HIP_F32: return dispatch_dim<float>(ctx, p, D, a->batch, want_scores, stream);

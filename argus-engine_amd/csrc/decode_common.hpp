@@ -501,7 +501,7 @@ inline void choose_splits(DecodeParams &p, int pairs, int tile_rows, int64_t slo
 }
 
 // Matrix-core variant (decode_mfma.hip): F16 cache, contiguous slots, no soft-cap.
-bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype);
+bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype, int batch);
 int launch_decode_mfma(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hipStream_t stream);
 // Block-quantised caches (decode_blocks.hip): ARGUS_HIP_Q4_0 / Q4_1 / Q8_0, dequantised in registers.
 int launch_decode_blocks(argus_hip_ctx *ctx, DecodeParams &p, int D, int kv_dtype, int batch, hipStream_t stream);

@@ -384,7 +384,7 @@ int launch_mfma(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stre
 
 }  // namespace
 
-bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
+bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype, int batch) {
   if (kv_dtype != ARGUS_HIP_F16 || p.len < 64) return false;
   // rows are addressed with 32-bit byte offsets from the head's first row, a few tiles past the end;
   // an index list may name any slot of the cache (slot x row bytes is a 24-bit multiply)
@@ -394,9 +394,13 @@ bool decode_mfma_supported(const DecodeParams &p, int D, int kv_dtype) {
   if (!score_rows_addressable(p)) return false;
   if (D == 64 || D == 128) return p.group <= 16;
   // head_dim 256: one 64-row tile per workgroup costs more set-up (Q split over 256 channels) than it
-  // saves; measured against the vector-ALU kernel it only pays for long rows and wider groups
-  // (Hq8/Hkv4, L 2048: 30 us vs 17 us; L 32768: equal).
-  return D == 256 && p.group >= 4 && p.group <= 8 && p.len >= 8192;
+  // saves on short calls; measured against the vector-ALU kernel it pays for long rows with wider
+  // groups (Hq8/Hkv4, L 2048: 30 us vs 17 us; L 32768: equal) and, with two to three heads per KV
+  // head, once the call attends enough rows in total (Hq8/Hkv4, L 2048, scores and soft cap: 17.0 vs
+  // 14.9 us at 8 sequences, 80 vs 101 us at 64; the lines cross near 13 sequences).
+  if (D != 256 || p.group > 8) return false;
+  if (p.group >= 4) return p.len >= 8192;
+  return (int64_t)batch * p.n_heads_kv * p.len >= 128 * 1024;
 }
 
 int launch_decode_mfma(argus_hip_ctx *ctx, DecodeParams &p, int D, int batch, hipStream_t stream) {

@@ -312,3 +312,34 @@ def test_statistics_form_on_the_other_decode_kernels_and_the_fallback_row():
     assert np.allclose(host(sc)[..., :L], 1.0 / L)
     assert not host(lg)[..., :L].any() and np.array_equal(host(st).reshape(-1, 2), np.tile([0.0, float(L)], (hq, 1)))
     assert ctx().attention_gen(dev(q), dev(f16(k32)), dev(f16(v32)), out, hkv, L, cap, score_stats=st, check=False) == A.ERR_INVALID
+
+
+@pytest.mark.gpu
+def test_config5_batch16_runs_on_the_matrix_core_arm():
+    # Two query heads per KV head at head_dim 256: a call that attends 128K rows or more (16 sequences
+    # x 4 KV heads x 2048 slots) goes to the matrix-core kernel; below that the vector-ALU kernel is
+    # faster and keeps the call.  Same checks as the flow above: outputs, per-position scores (soft
+    # cap 50), and the opt-in logits + (max, sum) form against the probability form.
+    import torch
+    hq, hkv, d, cap, L, batch, softcap = 8, 4, 256, 4096, 2048, 16, 50.0
+    q = normal((batch, hq, d), 7)
+    kc = np.zeros((batch, hkv, cap, d), np.float16)
+    vc = np.zeros((batch, hkv, cap, d), np.float16)
+    kc[:, :, :L] = f16(normal((batch, hkv, L, d), 8))
+    vc[:, :, :L] = f16(normal((batch, hkv, L, d), 9))
+    out, sc, out2, lg, st = _decode_both_forms(q, kc, vc, hkv, L, cap, batch, softcap)
+    assert ctx().last_decode_plan()["kernel"] == 1, ctx().last_decode_plan()
+    assert torch.equal(out, out2)
+    m, l = st[..., 0:1], st[..., 1:2]
+    assert torch.allclose(torch.exp(lg[..., :L] - m) / l, sc[..., :L], rtol=1e-5, atol=0)
+    got, gsc = host(out), host(sc)
+    for b in (0, 7, 15):
+        ref, p = O.attention_gen(q[b], kc[b], vc[b], hkv, L, cap, scores=True, scores_stride=cap, softcap=softcap)
+        check_attention_out(got[b], ref, "seq %d" % b)
+        check_scores(gsc[b, :, :L], p[:, :L], "seq %d" % b)
+    # the same shape at 8 sequences stays on the vector-ALU kernel
+    out8 = torch.empty((8, hq, d), device="cuda")
+    ctx().attention_gen(dev(q[:8]), dev(kc[:8]), dev(vc[:8]), out8, hkv, L, cap, batch=8, kv_batch_stride=hkv * cap * d, softcap=softcap)
+    assert ctx().last_decode_plan()["kernel"] == 0, ctx().last_decode_plan()
+    for b in (0, 7):
+        check_attention_out(host(out8)[b], O.attention_gen(q[b], kc[b], vc[b], hkv, L, cap, softcap=softcap), "seq %d of 8" % b)
