@@ -283,30 +283,39 @@ __device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p, uint32_t
 // one word, bytes 2, 3 in another -- and the four shifts of piece_codes then bring out one nibble
 // position of both tokens at a time: byte 0 low, byte 1 low, byte 0 high, byte 1 high from the first
 // word are slots 0, 2, 4, 6, the same from the second word slots 1, 3, 5, 7.
-template <int FMT, int N>
+// SCALED = false leaves the operands 64 + code (the caller scales the other MFMA operand instead).
+template <int FMT, int N, bool SCALED>
 __device__ __forceinline__ void scaled_pair(const RawPiece<FMT> &a, const RawPiece<FMT> &b, uint32_t upper, half2_t (&out)[N]) {
   static_assert((FMT == kFmtQ4_0 || FMT == kFmtQ4_1) && (N == 8 || N == 4), "nibble formats; whole or half pieces");
-  const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b.hdr, a.hdr, 0x05040100u));  // {d_a, d_b}
-  const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};                               // exact
+  half2_t dd = {}, nb = {};
+  if constexpr (SCALED) {
+    dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b.hdr, a.hdr, 0x05040100u));  // {d_a, d_b}
+    nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};                               // exact
+  }
+  auto value = [&](half2_t code) { return SCALED ? __builtin_elementwise_fma(code, dd, nb) : code; };
   uint32_t mask = 0x00f000f0u, exponent = 0x54005400u;
   asm("" : "+v"(mask), "+v"(exponent));  // keep both in vector registers
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     uint32_t w = __builtin_amdgcn_perm(b.code[0], a.code[0], h ? 0x07060302u : 0x05040100u);
-    // Half pieces (head_dim 64, N = 4): the lane's half is the low or the high nibbles (`upper`),
-    // brought down by a per-lane shift; slots 0..3 are bytes 0, 2, 1, 3 of that half.
-    if constexpr (N == 4) w >>= 4u * upper;
-    out[0 + h] = __builtin_elementwise_fma(nibbles(w << 4, mask, exponent), dd, nb);
-    out[2 + h] = __builtin_elementwise_fma(nibbles(w >> 4, mask, exponent), dd, nb);
-    if constexpr (N == 8) {
-      out[4 + h] = __builtin_elementwise_fma(nibbles(w, mask, exponent), dd, nb);
-      out[6 + h] = __builtin_elementwise_fma(nibbles(w >> 8, mask, exponent), dd, nb);
+    if constexpr (N == 4) {
+      // Half pieces (head_dim 64): the lane's half is the low or the high nibbles (`upper`); a
+      // per-lane shift brings byte 0's to bits 4..7, and byte 1's follow 8 bits further up.  Slots
+      // 0..3 are bytes 0, 2, 1, 3 of that half.
+      w <<= 4u - 4u * upper;
+      out[0 + h] = value(nibbles(w, mask, exponent));
+      out[2 + h] = value(nibbles(w >> 8, mask, exponent));
+    } else {
+      out[0 + h] = value(nibbles(w << 4, mask, exponent));
+      out[2 + h] = value(nibbles(w >> 4, mask, exponent));
+      out[4 + h] = value(nibbles(w, mask, exponent));
+      out[6 + h] = value(nibbles(w >> 8, mask, exponent));
     }
   }
 }
 
 // Half a piece (head_dim 64): the element held by slot s of the half `upper` of code index x, and
-// its 4 values d * code.  q4: `upper` selects the high nibbles, brought down by a per-lane shift so
+// its 4 values d * code.  q4: `upper` selects the high nibbles, lined up by a per-lane shift so
 // that both halves run the same instructions; q8: the piece's one code dword is already the half;
 // q2_0: `sel` is the lane's q2_byte_selector (the half is one byte: four fields).
 template <int FMT>
@@ -314,29 +323,46 @@ __host__ __device__ constexpr int half_slot_elem(int x, int upper, int s) {
   if (FMT == kFmtQ8_0 || FMT == kFmtQ2_0) return 8 * x + 4 * upper + s;
   return 16 * upper + 4 * x + (s == 1 ? 2 : (s == 2 ? 1 : s));  // 0, 2, 1, 3
 }
+// The operand of half slot s is half_slot_bias(s) + code when SCALED is false.
 template <int FMT>
+__host__ __device__ constexpr float half_slot_bias(int s) {
+  return (FMT == kFmtQ8_0) ? 0.0f : ((FMT == kFmtQ2_0 && (s & 1)) ? 16.0f : 64.0f);
+}
+template <int FMT, bool SCALED>
 __device__ __forceinline__ half4_t scaled_half(const RawPiece<FMT> &p, uint32_t upper, uint32_t sel) {
-  const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u));  // {d, d}
+  const half2_t dd = SCALED ? __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u)) : half2_t{};  // {d, d}
   half2_t v[2];
   if constexpr (FMT == kFmtQ2_0) {
     const uint32_t w = __builtin_amdgcn_perm(0u, p.code[0], sel);  // [byte, 0, byte, 0]
     uint32_t mask = 0x00c00030u, exponent = 0x4c005400u;           // low half: bits 4..5 (64 + n), high half: bits 6..7 (16 + n)
     asm("" : "+v"(mask), "+v"(exponent));
     const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-16.0f};  // exact
-    v[0] = __builtin_elementwise_fma(nibbles(w << 4, mask, exponent), dd, nb);  // fields 0, 1
-    v[1] = __builtin_elementwise_fma(nibbles(w, mask, exponent), dd, nb);       // fields 2, 3
+    v[0] = nibbles(w << 4, mask, exponent);  // fields 0, 1
+    v[1] = nibbles(w, mask, exponent);       // fields 2, 3
+    if constexpr (SCALED) {
+      v[0] = __builtin_elementwise_fma(v[0], dd, nb);
+      v[1] = __builtin_elementwise_fma(v[1], dd, nb);
+    }
   } else if constexpr (FMT == kFmtQ8_0) {
     const half2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
     const uint32_t u = p.code[0] ^ 0x80808080u;
-    v[0] = (bytes_lo(u) + off) * dd;
-    v[1] = (bytes_hi(u) + off) * dd;
+    v[0] = bytes_lo(u) + off;
+    v[1] = bytes_hi(u) + off;
+    if constexpr (SCALED) {
+      v[0] = v[0] * dd;
+      v[1] = v[1] * dd;
+    }
   } else {
-    const uint32_t w = p.code[0] >> (4u * upper);
+    const uint32_t w = p.code[0] << (4u - 4u * upper);  // the half's nibbles of bytes 0, 2 at bits 4..7
     uint32_t mask = 0x00f000f0u, exponent = 0x54005400u;
     asm("" : "+v"(mask), "+v"(exponent));
     const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
-    v[0] = __builtin_elementwise_fma(nibbles(w << 4, mask, exponent), dd, nb);  // bytes 0, 2
-    v[1] = __builtin_elementwise_fma(nibbles(w >> 4, mask, exponent), dd, nb);  // bytes 1, 3
+    v[0] = nibbles(w, mask, exponent);       // bytes 0, 2
+    v[1] = nibbles(w >> 8, mask, exponent);  // bytes 1, 3
+    if constexpr (SCALED) {
+      v[0] = __builtin_elementwise_fma(v[0], dd, nb);
+      v[1] = __builtin_elementwise_fma(v[1], dd, nb);
+    }
   }
   return half4_t{v[0][0], v[0][1], v[1][0], v[1][1]};
 }
@@ -714,9 +740,19 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // sum over tokens of p * d (q4_0: times -8 it is the zero-point term of the lane's channels) or
   // of p * m (q4_1: the minimum term), per V piece; one more MFMA column each
   constexpr bool kHdrTerm = FMT != kFmtQ8_0;
-  float4_t h_acc[VSEG];
+  // Tokens as columns: the sixteen rows of the P operand are four heads (row % 4) times four copies,
+  // and copy row / 4 is multiplied by the scale d of the block that output columns 4 (row / 4) ..
+  // + 3 belong to (head_dim 64: two blocks, copies row / 4 % 2).  The V operand is then the bare
+  // code, bias + n, with no arithmetic per value; column c of the result is right in the rows of
+  // its own block's copy, and the merge reads it from there.  h_acc sums the scaled weights (times
+  // -(bias + zero point) it takes the bias back out), m_acc the plain weights times the minimum.
+  constexpr bool kScaleP = TOKCOL;
+  constexpr bool kMinTerm = kScaleP && F::kHasMin;
+  float4_t h_acc[VSEG], m_acc[kMinTerm ? VSEG : 1];
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int sg = 0; sg < (kMinTerm ? VSEG : 1); ++sg) m_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
   // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
   // then the merge area.
@@ -833,6 +869,12 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           for (int sg = 0; sg < VSEG; ++sg)
 #pragma unroll
             for (int i = 0; i < 4; ++i) h_acc[sg][i] *= al[i];
+        }
+        if constexpr (kMinTerm) {
+#pragma unroll
+          for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) m_acc[sg][i] *= al[i];
         }
       }
       // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of head r % 4
@@ -990,8 +1032,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       load_v(base + kWaves * TILE);
     }
     // The operands of tile tw, V piece sg: bv[c] = channel slot c of the lane's four tokens, hv = their
-    // d (or m) for the header term.
-    auto v_operands = [&](int tw, int sg, half4_t (&bv)[VCH], half4_t &hv) {
+    // d (or m) for the header term; with the scales on the P side: bv[c] = the bare codes, dv = the
+    // tokens' d, hv = their m.
+    auto v_operands = [&](int tw, int sg, half4_t (&bv)[VCH], half4_t &hv, half4_t &dv) {
         RawPiece<FMT> vpc[4];  // the lane's piece of tokens 4j .. 4j+3
         if constexpr (STREAM) {
 #pragma unroll
@@ -1039,22 +1082,28 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         vrow_t vrow[4];
         half2_t vpair[2][VCH];
         if constexpr (kPairV) {
-          scaled_pair<FMT, VCH>(vpc[0], vpc[1], (uint32_t)(r >> 3), vpair[0]);
-          scaled_pair<FMT, VCH>(vpc[2], vpc[3], (uint32_t)(r >> 3), vpair[1]);
+          scaled_pair<FMT, VCH, !kScaleP>(vpc[0], vpc[1], (uint32_t)(r >> 3), vpair[0]);
+          scaled_pair<FMT, VCH, !kScaleP>(vpc[2], vpc[3], (uint32_t)(r >> 3), vpair[1]);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if constexpr (D == 64) vrow[e] = scaled_half<FMT>(vpc[e], (uint32_t)(r >> 3), v_half_sel);
+            if constexpr (D == 64) vrow[e] = scaled_half<FMT, !kScaleP>(vpc[e], (uint32_t)(r >> 3), v_half_sel);
+            else if constexpr (kScaleP) vrow[e] = code_operand<FMT>(vpc[e], v_sel);
             else vrow[e] = scaled_codes<FMT>(vpc[e], v_sel);
           }
         }
-        if constexpr (kHdrTerm) {
+        typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+        if constexpr (kHdrTerm && (!kScaleP || F::kHasMin)) {
           // d (q4_0: low halves of the headers) or m (q4_1, q2_0: high halves) of the lane's four tokens
           constexpr uint32_t sel = F::kHasMin ? 0x07060302u : 0x05040100u;
           const uint32_t h01 = __builtin_amdgcn_perm(vpc[1].hdr, vpc[0].hdr, sel);
           const uint32_t h23 = __builtin_amdgcn_perm(vpc[3].hdr, vpc[2].hdr, sel);
-          typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
           hv = __builtin_bit_cast(half4_t, u32x2_t{h01, h23});
+        }
+        if constexpr (kScaleP) {
+          const uint32_t d01 = __builtin_amdgcn_perm(vpc[1].hdr, vpc[0].hdr, 0x05040100u);
+          const uint32_t d23 = __builtin_amdgcn_perm(vpc[3].hdr, vpc[2].hdr, 0x05040100u);
+          dv = __builtin_bit_cast(half4_t, u32x2_t{d01, d23});
         }
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {
@@ -1066,11 +1115,19 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
       for (int sg = 0; sg < VSEG; ++sg) {
-        half4_t bv[VCH], hv = {};
-        v_operands(tw, sg, bv, hv);
-        if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+        half4_t bv[VCH], hv = {}, dv = {};
+        v_operands(tw, sg, bv, hv, dv);
+        half4_t pv = pa[tw];
+        if constexpr (kScaleP) {
+          pv = pa[tw] * dv;
+          const half4_t ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
+          if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, ones, h_acc[sg], 0, 0, 0);
+          if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, m_acc[sg], 0, 0, 0);
+        } else if constexpr (kHdrTerm) {
+          h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+        }
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], bv[c], o_acc[sg * VCH + c], 0, 0, 0);
+        for (int c = 0; c < VCH; ++c) o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, bv[c], o_acc[sg * VCH + c], 0, 0, 0);
       }
     if constexpr (!STREAM) load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
@@ -1082,7 +1139,20 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     __syncthreads();  // the other waves' spare slots lie in the merge area
   }
 
-  if constexpr (kHdrTerm) {
+  if constexpr (kScaleP && kHdrTerm) {
+#pragma unroll
+    for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+      for (int c = 0; c < VCH; ++c) {
+        const float bias = (D == 64) ? half_slot_bias<FMT>(c) : CD::slot_bias(c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float o = fmaf(-(bias + CD::kZero), h_acc[sg][i], o_acc[sg * VCH + c][i]);
+          if constexpr (kMinTerm) o += m_acc[sg][i];
+          o_acc[sg * VCH + c][i] = o;
+        }
+      }
+  } else if constexpr (kHdrTerm) {
     constexpr float kTerm = (FMT == kFmtQ4_0) ? -CD::kZero : 1.0f;
 #pragma unroll
     for (int sg = 0; sg < VSEG; ++sg)
@@ -1099,6 +1169,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
   }
+  const int own_copy = (D == 64) ? ((r >> 2) & 1) : (r >> 2);  // the P copy scaled for this lane's output columns
   float (*lds_m)[16] = (float (*)[16])dyn_lds;
   float (*lds_l)[16] = lds_m + kWaves;
   float (*lds_acc)[SH::MAXH][D + 4] = (float (*)[SH::MAXH][D + 4])(dyn_lds + 2 * kWaves * 16);
@@ -1113,7 +1184,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       const int ch = 32 * vblk[sg] + ((D == 64) ? half_slot_elem<FMT>(r & 3, r >> 3, c) : slot_elem<FMT>(r & 3, c));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (TOKCOL ? j == 0 : 4 * j + i < SH::MAXH) lds_acc[wave][4 * j + i][ch] = o_acc[sg * VCH + c][i];  // (TOKCOL: rows 4j + i repeat head i)
+        if (TOKCOL ? j == own_copy : 4 * j + i < SH::MAXH) lds_acc[wave][TOKCOL ? i : 4 * j + i][ch] = o_acc[sg * VCH + c][i];  // (TOKCOL: row 4j + i is head i scaled for block j)
     }
   __syncthreads();
 

@@ -149,6 +149,36 @@ def test_every_group_width_with_and_without_scores(fmt, d):
             run_case(fmt, 2 * g, 2, d, L, cap=L + 5, seed=g + L + d + 1, scores=not ((g + L) & 1))
 
 
+@pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (14, 2, 64), (32, 8, 128), (16, 2, 128), (8, 4, 256)])
+def test_value_scales_from_tiny_to_large(fmt, hq, hkv, d):
+    # Groups of up to four heads carry a V block's scale on the attention weights instead of on its
+    # codes (the product of a weight and a scale is rounded to f16 before the matrix multiply), wider
+    # groups scale the codes: V scales (and minima) spread over 2^-12 .. 2^4 times the usual ones
+    # pin both against the oracle, relative to the largest output.
+    import argus_hip as A
+    desc, name = FORMATS[fmt]
+    L = 1500
+    rows = hkv * L
+    bb = O.desc_block_bytes(desc)
+    k_raw = random_blocks(desc, rows * d // 32, 31)
+    v_raw = random_blocks(desc, rows * d // 32, 32).reshape(-1, bb).copy()
+    gain = np.exp2(np.random.default_rng(33).integers(-12, 5, size=v_raw.shape[0])).astype(np.float32)
+    hdr = v_raw[:, :4].copy().view(np.float16).astype(np.float32)  # (d, m or the first code bytes)
+    n_hdr = 2 if desc[2] == O.SCALE_F16_MIN else 1
+    scaled = (hdr[:, :n_hdr] * gain[:, None]).astype(np.float16)
+    v_raw[:, :2 * n_hdr] = scaled.view(np.uint8).reshape(-1, 2 * n_hdr)
+    v_raw = v_raw.reshape(-1)
+    q = normal((hq, d), 30)
+    out = dev(np.zeros((hq, d), np.float32))
+    ctx().attention_gen(dev(q), dev(k_raw), dev(v_raw), out, hkv, L, L, kv_dtype=getattr(A, name))
+    ref = O.attention_gen_blocks(q, k_raw, v_raw, desc, hkv, L, L)
+    got = host(out)
+    assert np.all(np.isfinite(got))
+    err = np.abs(got.astype(np.float64) - ref) / np.abs(ref).max()
+    assert err.max() <= 2e-3 and err.mean() <= 1e-3, "%s Hq%d Hkv%d d%d: max %g mean %g of the largest output" % (fmt, hq, hkv, d, err.max(), err.mean())
+
+
 @pytest.mark.parametrize("fmt,hq,hkv,d,L", [("q4_0", 16, 8, 256, 2048), ("q8_0", 8, 4, 256, 1000), ("q4_1", 32, 8, 128, 1500), ("q4_0", 14, 2, 64, 777),
                                             ("q2_0", 32, 8, 128, 900)])
 def test_soft_cap_on_block_caches(fmt, hq, hkv, d, L):
