@@ -421,6 +421,16 @@ struct BlockShape {
   static constexpr int MAXH = (D == 256) ? 8 : 16;        // query heads per KV head (bounds the merge LDS)
 };
 
+// The wave-private LDS copy of a streamed tile (see the kernel): requests of kLW dwords per lane,
+// NLD of them per tile, and the dwords one copy takes.
+template <int FMT, int D, int TW>
+struct StreamCopy {
+  static constexpr int kLW = 2;
+  static constexpr int kRowDwords = (D / 32) * BlockFmt<FMT>::BB / 4;
+  static constexpr int NLD = (16 * TW * kRowDwords + 64 * kLW - 1) / (64 * kLW);
+  static constexpr int kDwords = NLD * 64 * kLW + 4;  // the last request may run past the tile; a piece's second dword past a row
+};
+
 // Waves per SIMD the register allocation aims at: 4 at head_dim 64 (128 registers), 3 at 128 (168;
 // q8_0 would spill there and stays at 2), 2 at 256.  Without the bound most instantiations came out a
 // few registers on one or the other side of a step depending on unrelated edits (q4_0 at 128: 165 or
@@ -497,11 +507,16 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   constexpr int RBY = KK * F::BB;                  // bytes per packed row
   static_assert(RBY % 4 == 0, "rows are whole dwords");
   constexpr int RD = RBY / 4;                      // dwords per row
-  constexpr int NLD = (TILE * RD + 63) / 64;       // wave-wide dword requests per tile
-  uint32_t kst[STREAM ? NLD : 1], vst[STREAM ? NLD : 1];
+  // A request fetches LW dwords per lane, 256 LW contiguous bytes per wave.  Measured at 1, 2 and 4
+  // dwords: 2 was within 1 % of the best for every format (q8_0 +3 % over 1); 4 makes the copies
+  // bigger, and with staged scores that leaves room for fewer workgroups (-6 %).
+  using SC = StreamCopy<FMT, D, TW>;
+  constexpr int LW = SC::kLW, NLD = SC::NLD;
+  static_assert(SC::kRowDwords == RD, "launcher and kernel agree on the row");
+  uint32_t kst[STREAM ? NLD * LW : 1], vst[STREAM ? NLD * LW : 1];
   // The copies live in the dynamic area behind whatever the token loop keeps there (the staged
   // logits, or the spare slots of lanes that park nothing); the merge at the end reuses all of it.
-  constexpr int kTileDw = NLD * 64 + 4;  // the last request may run past the tile; a piece's second dword past a row
+  constexpr int kTileDw = SC::kDwords;
   extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
   const int stage_row = p.chunk + 4;
   const int staged_heads = p.stage_scores ? p.group : 0;
@@ -511,15 +526,34 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   const uint32_t run_bytes = (uint32_t)min((int64_t)p.len * RBY, (int64_t)0xffffffffll);
   const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void *)kb, 0, STREAM ? run_bytes : 0u, kBufferFlags);
   const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc((void *)vb, 0, STREAM ? run_bytes : 0u, kBufferFlags);
-  auto fetch_run = [&](__amdgpu_buffer_rsrc_t rs, int base, uint32_t (&st)[STREAM ? NLD : 1]) {
+  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+  auto fetch_run = [&](__amdgpu_buffer_rsrc_t rs, int base, uint32_t (&st)[STREAM ? NLD * LW : 1]) {
     const uint32_t off = (uint32_t)min(base, p.len) * (uint32_t)RBY;  // scalar; past the end everything reads as zero
 #pragma unroll
-    for (int c = 0; c < NLD; ++c) st[c] = __builtin_amdgcn_raw_buffer_load_b32(rs, 4u * (uint32_t)lane + 256u * (uint32_t)c, off, 0);
+    for (int c = 0; c < NLD; ++c) {
+      const uint32_t vo = (4u * LW) * (uint32_t)lane + (256u * LW) * (uint32_t)c;
+      if constexpr (LW == 4) {
+        const u32x4_t v = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, vo, off, 0));
+#pragma unroll
+        for (int w = 0; w < 4; ++w) st[4 * c + w] = v[w];
+      } else if constexpr (LW == 2) {
+        const u32x2_t v = __builtin_bit_cast(u32x2_t, __builtin_amdgcn_raw_buffer_load_b64(rs, vo, off, 0));
+        st[2 * c] = v[0];
+        st[2 * c + 1] = v[1];
+      } else {
+        st[c] = __builtin_amdgcn_raw_buffer_load_b32(rs, vo, off, 0);
+      }
+    }
   };
-  auto park_run = [&](uint32_t *tile, const uint32_t (&st)[STREAM ? NLD : 1]) {
+  auto park_run = [&](uint32_t *tile, const uint32_t (&st)[STREAM ? NLD * LW : 1]) {
     wave_lds_fence();  // the reads of the tile before are done
 #pragma unroll
-    for (int c = 0; c < NLD; ++c) tile[64 * c + lane] = st[c];
+    for (int c = 0; c < NLD; ++c) {
+      uint32_t *dst = tile + LW * (64 * c + lane);
+      if constexpr (LW == 4) *(u32x4_t *)dst = u32x4_t{st[4 * c], st[4 * c + 1], st[4 * c + 2], st[4 * c + 3]};
+      else if constexpr (LW == 2) *(u32x2_t *)dst = u32x2_t{st[2 * c], st[2 * c + 1]};
+      else *dst = st[c];
+    }
     wave_lds_fence();
   };
   // Piece (code index x, CW dwords) of block blk of a parked row.  With a 2-byte header the code
@@ -684,7 +718,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   load_idx_v(base0 + kWaves * TILE);
   __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the query's
 
-  // ---- Q operand: lane (j, h = r), block kk: the elements slot_elem(j, 0..7), log2 domain, hi + lo
+  // ---- Q operand: lane (j, h = r), block kk: the elements slot_elem(j, 0..7), log2 domain, hi + lo.
+  // Tokens as columns: row r is head r / 4, and of a head's four rows the first carries the high
+  // parts and the second the low parts (the other two are zero), so one MFMA yields both partial
+  // dot products, in result registers 0 and 1 of the head's lane group.
   half8_t qh[KK], ql[KK];
   float qsum[KK];   // sum of the scaled query over block kk: the minimum term
   float qinit[KK];  // what a block's MFMA accumulator starts from: -sum over the block of (slot bias + zero point) * q
@@ -706,8 +743,12 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         if constexpr (FMT == kFmtQ2_0) biased = fmaf(CD::slot_bias(s), x, biased);
         _Float16 hi, lo;
         split_f16(x, hi, lo);
-        qh[kk][s] = hi;
-        ql[kk][s] = lo;
+        if constexpr (TOKCOL) {
+          qh[kk][s] = (ph == 0) ? hi : ((ph == 1) ? lo : (_Float16)0.0f);
+        } else {
+          qh[kk][s] = hi;
+          ql[kk][s] = lo;
+        }
       }
       // the four lane groups hold the four quarters of the block
       part += __shfl_xor(part, 16, 64);
@@ -799,11 +840,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           const half8_t kb_op = code_operand<FMT>(kpc[kk], k_sel);
           float4_t dot = {0.0f, 0.0f, 0.0f, 0.0f};
           dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[kk], kb_op, dot, 0, 0, 0);
-          dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql[kk], kb_op, dot, 0, 0, 0);
           // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q, times the
           // token's scale for this block, which the lane holds itself
           const half2_t dm = __builtin_bit_cast(half2_t, kpc[kk].hdr);
-          const float mine = dot[0] + qinit[kk];
+          const float mine = (dot[0] + qinit[kk]) + dot[1];
           if constexpr (F::kHasMin) sc[tw] = fmaf((float)dm[0], mine, fmaf((float)dm[1], qsum[kk], sc[tw]));
           else sc[tw] = fmaf((float)dm[0], mine, sc[tw]);
         }
@@ -883,7 +923,6 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       p_strip[wave][j][r] = __builtin_bit_cast(uint32_t, pk);
       wave_lds_fence();
       const u32x4_t w = *(const u32x4_t *)&p_strip[wave][ph][4 * j];
-      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
         const uint32_t sel = tw ? 0x07060302u : 0x05040100u;
@@ -1092,7 +1131,6 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
             else vrow[e] = scaled_codes<FMT>(vpc[e], v_sel);
           }
         }
-        typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
         if constexpr (kHdrTerm && (!kScaleP || F::kHasMin)) {
           // d (q4_0: low halves of the headers) or m (q4_1, q2_0: high halves) of the lane's four tokens
           constexpr uint32_t sel = F::kHasMin ? 0x07060302u : 0x05040100u;
@@ -1111,24 +1149,50 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           else bv[c] = half4_t{vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
         }
     };
-#pragma unroll
-    for (int tw = 0; tw < TW; ++tw)
+    const half4_t ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
+    if constexpr (TW == 2 && TOKCOL && D == 128) {
+      // Both tiles in one MFMA of 32 tokens (it holds the matrix core no longer than one of 16):
+      // contraction slots 0..3 of a lane are its four tokens of the first tile, 4..7 of the second.
+      // (The tokens-as-rows arm has no registers for the operands of two tiles at once; head_dim 64
+      // ran 2 % slower this way.)
+      auto both = [](half4_t a, half4_t b) { return half8_t{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]}; };
 #pragma unroll
       for (int sg = 0; sg < VSEG; ++sg) {
-        half4_t bv[VCH], hv = {}, dv = {};
-        v_operands(tw, sg, bv, hv, dv);
-        half4_t pv = pa[tw];
+        half4_t bv0[VCH], bv1[VCH], hv0 = {}, hv1 = {}, dv0 = {}, dv1 = {};
+        v_operands(0, sg, bv0, hv0, dv0);
+        v_operands(1, sg, bv1, hv1, dv1);
+        const half8_t pw = both(pa[0], pa[1]);
+        half8_t pv = pw;
         if constexpr (kScaleP) {
-          pv = pa[tw] * dv;
-          const half4_t ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
-          if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, ones, h_acc[sg], 0, 0, 0);
-          if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, m_acc[sg], 0, 0, 0);
+          pv = both(pa[0] * dv0, pa[1] * dv1);
+          if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv, both(ones, ones), h_acc[sg], 0, 0, 0);
+          if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pw, both(hv0, hv1), m_acc[sg], 0, 0, 0);
         } else if constexpr (kHdrTerm) {
-          h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+          h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pw, both(hv0, hv1), h_acc[sg], 0, 0, 0);
         }
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, bv[c], o_acc[sg * VCH + c], 0, 0, 0);
+        for (int c = 0; c < VCH; ++c)
+          o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv, both(bv0[c], bv1[c]), o_acc[sg * VCH + c], 0, 0, 0);
       }
+    } else {
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+        for (int sg = 0; sg < VSEG; ++sg) {
+          half4_t bv[VCH], hv = {}, dv = {};
+          v_operands(tw, sg, bv, hv, dv);
+          half4_t pv = pa[tw];
+          if constexpr (kScaleP) {
+            pv = pa[tw] * dv;
+            if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, ones, h_acc[sg], 0, 0, 0);
+            if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, m_acc[sg], 0, 0, 0);
+          } else if constexpr (kHdrTerm) {
+            h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+          }
+#pragma unroll
+          for (int c = 0; c < VCH; ++c) o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, bv[c], o_acc[sg * VCH + c], 0, 0, 0);
+        }
+    }
     if constexpr (!STREAM) load_v(base + kWaves * TILE);
     load_idx_v(base + 2 * kWaves * TILE);
   }
@@ -1172,7 +1236,8 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   const int own_copy = (D == 64) ? ((r >> 2) & 1) : (r >> 2);  // the P copy scaled for this lane's output columns
   float (*lds_m)[16] = (float (*)[16])dyn_lds;
   float (*lds_l)[16] = lds_m + kWaves;
-  float (*lds_acc)[SH::MAXH][D + 4] = (float (*)[SH::MAXH][D + 4])(dyn_lds + 2 * kWaves * 16);
+  constexpr int MH = TOKCOL ? 4 : SH::MAXH;  // heads a workgroup merges (tokens as columns: groups of up to four)
+  float (*lds_acc)[MH][D + 4] = (float (*)[MH][D + 4])(dyn_lds + 2 * kWaves * 16);
   if (TOKCOL ? r == 0 : j == 0) {
     lds_m[wave][TOKCOL ? j : r] = m_run;
     lds_l[wave][TOKCOL ? j : r] = l_run;
@@ -1184,7 +1249,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       const int ch = 32 * vblk[sg] + ((D == 64) ? half_slot_elem<FMT>(r & 3, r >> 3, c) : slot_elem<FMT>(r & 3, c));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (TOKCOL ? j == own_copy : 4 * j + i < SH::MAXH) lds_acc[wave][TOKCOL ? i : 4 * j + i][ch] = o_acc[sg * VCH + c][i];  // (TOKCOL: row 4j + i is head i scaled for block j)
+        if (TOKCOL ? j == own_copy : 4 * j + i < MH) lds_acc[wave][TOKCOL ? i : 4 * j + i][ch] = o_acc[sg * VCH + c][i];  // (TOKCOL: row 4j + i is head i scaled for block j)
     }
   __syncthreads();
 
@@ -1227,9 +1292,9 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
   // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips or the
   // streamed tiles' LDS copies).
-  constexpr int kTileCopies = 2 * kWaves * (((16 * TW * (D / 32) * BlockFmt<FMT>::BB / 4 + 63) / 64) * 64 + 4) * 4;
+  constexpr int kTileCopies = 2 * kWaves * StreamCopy<FMT, D, TW>::kDwords * 4;
   constexpr int kStageBytes = (kTileCopies > 24 * 1024) ? 32 * 1024 : 48 * 1024;
-  constexpr size_t merge_bytes = (2 * kWaves * 16 + kWaves * BlockShape<D>::MAXH * (D + 4)) * sizeof(float);
+  const size_t merge_bytes = (2 * kWaves * 16 + kWaves * (tokcol ? 4 : BlockShape<D>::MAXH) * (D + 4)) * sizeof(float);
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
   auto pick = [&](auto tc, auto st) {
     constexpr bool TC = decltype(tc)::value, ST = decltype(st)::value;
