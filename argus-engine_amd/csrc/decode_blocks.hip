@@ -1286,9 +1286,10 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   // Packed rows without an index list are streamed (see the kernel); the slabs must start on a dword.
   const int64_t head_blocks = ((int64_t)p.kv_bs | (int64_t)p.head_stride) / 32;
   // (Measured per arm: q8_0 +10 % either way, q2_0 +10 % and q4_0 +3 % with tokens as columns; the
-  // tokens-as-rows arm of the 4-bit formats has no registers left for it and ran 3-5 % slower.)
+  // tokens-as-rows arm of the 4-bit formats has no registers left for it at head_dim 128 and 256 and
+  // ran 3-5 % slower, at 64 it has and runs 3 % faster.)
   const bool stream_rows = !indexed && p.row_stride == D && (((uintptr_t)p.k | (uintptr_t)p.v) & 3) == 0 &&
-                           (head_blocks * BlockFmt<FMT>::BB) % 4 == 0 && (FMT == kFmtQ8_0 || tokcol);
+                           (head_blocks * BlockFmt<FMT>::BB) % 4 == 0 && (FMT == kFmtQ8_0 || tokcol || D == 64);
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
   // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips or the
   // streamed tiles' LDS copies).
@@ -1298,7 +1299,7 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
   auto pick = [&](auto tc, auto st) {
     constexpr bool TC = decltype(tc)::value, ST = decltype(st)::value;
-    if constexpr (ST && (FMT == kFmtQ8_0 || TC)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
+    if constexpr (ST && (FMT == kFmtQ8_0 || TC || D == 64)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
     else return cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, TC, false> : decode_blocks_kernel<FMT, D, TW, true, false, TC, false>)
                     : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, TC, false> : decode_blocks_kernel<FMT, D, TW, false, false, TC, false>);
   };
