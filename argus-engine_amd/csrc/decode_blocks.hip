@@ -446,6 +446,10 @@ struct StreamCopy {
 // softmax runs once per logit instead of once per operand column, a head's maximum is a reduction
 // inside one 16-lane row, and the probabilities reach the P operand's layout (lane (j, r): tokens
 // 4j..4j+3 of head r % 4) through 256 bytes of LDS per wave.
+// TOKCOL = 2 (head_dim 64, five to eight heads per KV head): the query rows are head r / 2, high part
+// in the even row and low part in the odd one, so lane group g keeps the two heads 2g and 2g + 1 (HL
+// = 2 logits per lane and tile); the P operand has head r % 4 + 4 (r / 8) in row r, scaled for block
+// r / 4 % 2 -- with two blocks per row the sixteen rows are exactly eight heads times two blocks.
 //
 // STREAM (rows packed back to back, no index list): a wave's tile is one contiguous run of bytes.
 // The per-lane block requests of the other path put a header and 16 or 32 code bytes at an 18- or
@@ -454,7 +458,7 @@ struct StreamCopy {
 // TCP_TOTAL_CACHE_ACCESSES against TCP_TCC_READ_REQ).  Here the lanes fetch consecutive dwords of
 // the run (one access per 64 bytes), park them in a wave-private LDS copy of the tile, and every lane
 // then reads the pieces of its MFMA operands straight from there: no trades between lanes at all.
-template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, bool TOKCOL, bool STREAM>
+template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, int TOKCOL, bool STREAM>
 __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
@@ -471,8 +475,11 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // Head whose query this lane's operand row (or column) carries.  TOKCOL: rows 4g..4g+3 all carry
   // head g, so the four registers of a result lane in lane group g all hold head g's logit and no
   // register has to be picked; the P operand of the output MFMAs has head r % 4 in row r.
-  const int rh = TOKCOL ? (r >> 2) : r;
-  const int ph = r & 3;
+  constexpr int HL = (TOKCOL == 2) ? 2 : 1;  // heads a lane keeps logits of
+  static_assert(TOKCOL != 2 || D == 64, "two heads per lane: the P copies are two blocks times eight heads");
+  const int rh = (TOKCOL == 2) ? (r >> 1) : (TOKCOL ? (r >> 2) : r);
+  const int ph = (TOKCOL == 2) ? (r & 1) : (r & 3);                  // which part of the query the row carries
+  const int pa_head = (TOKCOL == 2) ? (r & 3) + 4 * (r >> 3) : (r & 3);  // head in row r of the P operand
   static_assert(!(STREAM && INDEXED), "an index list gathers rows: they are read block by block");
 
   const int t_begin = split * p.chunk;
@@ -731,8 +738,8 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // parts and the second the low parts (the other two are zero), so one MFMA yields both partial
   // dot products, in result registers 0 and 1 of the head's lane group.
   half8_t qh[KK], ql[KK];
-  float qsum[KK];   // sum of the scaled query over block kk: the minimum term
-  float qinit[KK];  // what a block's MFMA accumulator starts from: -sum over the block of (slot bias + zero point) * q
+  float qsum[KK][HL];   // sum of the scaled query over block kk: the minimum term (tokens as columns: of each head the lane keeps)
+  float qinit[KK][HL];  // what a block's MFMA accumulator starts from: -sum over the block of (slot bias + zero point) * q
   {
     const float c = p.scale * 1.4426950408889634f;
     const int h = kvh * G + min(rh, G - 1);
@@ -761,15 +768,18 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       // the four lane groups hold the four quarters of the block
       part += __shfl_xor(part, 16, 64);
       part += __shfl_xor(part, 32, 64);
-      if constexpr (TOKCOL) part = __shfl(part, 4 * j, 64);  // the sums of head j, whose logits this lane keeps
-      qsum[kk] = part;
       if constexpr (FMT == kFmtQ2_0) {
         biased += __shfl_xor(biased, 16, 64);
         biased += __shfl_xor(biased, 32, 64);
-        if constexpr (TOKCOL) biased = __shfl(biased, 4 * j, 64);
-        qinit[kk] = -biased;
-      } else {
-        qinit[kk] = -(CD::kBias + CD::kZero) * part;
+      }
+#pragma unroll
+      for (int u = 0; u < HL; ++u) {
+        // tokens as columns: the sums of the heads whose logits this lane keeps, from a lane whose row is theirs
+        const int src = (TOKCOL == 2) ? 4 * j + 2 * u : 4 * j;
+        const float head_part = TOKCOL ? __shfl(part, src, 64) : part;
+        qsum[kk][u] = head_part;
+        if constexpr (FMT == kFmtQ2_0) qinit[kk][u] = -(TOKCOL ? __shfl(biased, src, 64) : biased);
+        else qinit[kk][u] = -(CD::kBias + CD::kZero) * head_part;
       }
     }
   }
@@ -802,7 +812,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   for (int sg = 0; sg < VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
   for (int sg = 0; sg < (kMinTerm ? VSEG : 1); ++sg) m_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  float m_run = kNegInf, l_run = 0.0f;  // per (lane = head r); l is this lane group's partial sum
+  float m_run[HL], l_run[HL];  // per (lane = head r; tokens as columns: the HL heads of the lane group); l is this lane group's partial sum
+#pragma unroll
+  for (int u = 0; u < HL; ++u) m_run[u] = kNegInf, l_run[u] = 0.0f;
   // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
   // then the merge area.
   __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
@@ -817,8 +829,8 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
     half4_t pa[TW];
     if constexpr (TOKCOL) {
-      // ---- logits: token base + 16 tw + r, head j ------------------------------------------------
-      float sc[TW];
+      // ---- logits: token base + 16 tw + r, head j (HL = 2: heads 2j and 2j + 1) -----------------
+      float sc[TW][HL];
       RawPiece<FMT> both[4];  // head_dim 64: lane group g held block g % 2 of tile g / 2
       if constexpr (STREAM) {
         park_run(k_tile, kst);
@@ -826,7 +838,8 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       } else if constexpr (D == 64) block_to_pieces<FMT>(kblk[0], both);
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
-        sc[tw] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < HL; ++u) sc[tw][u] = 0.0f;
         RawPiece<FMT> kpc[KK];
         if constexpr (STREAM) {
 #pragma unroll
@@ -851,63 +864,82 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q, times the
           // token's scale for this block, which the lane holds itself
           const half2_t dm = __builtin_bit_cast(half2_t, kpc[kk].hdr);
-          const float mine = (dot[0] + qinit[kk]) + dot[1];
-          if constexpr (F::kHasMin) sc[tw] = fmaf((float)dm[0], mine, fmaf((float)dm[1], qsum[kk], sc[tw]));
-          else sc[tw] = fmaf((float)dm[0], mine, sc[tw]);
+#pragma unroll
+          for (int u = 0; u < HL; ++u) {
+            // high and low parts: registers 0 and 1 (two heads per lane: 2u and 2u + 1)
+            const float mine = (dot[2 * u] + qinit[kk][u]) + dot[2 * u + 1];
+            if constexpr (F::kHasMin) sc[tw][u] = fmaf((float)dm[0], mine, fmaf((float)dm[1], qsum[kk][u], sc[tw][u]));
+            else sc[tw][u] = fmaf((float)dm[0], mine, sc[tw][u]);
+          }
         }
       }
       if constexpr (D != 64) __builtin_amdgcn_sched_barrier(0);  // (see the other arm)
       if constexpr (!STREAM) load_k(base + kWaves * TILE);
       load_idx_k(base + 2 * kWaves * TILE);
-      float mt = kNegInf;
+      float mt[HL];
 #pragma unroll
-      for (int tw = 0; tw < TW; ++tw) {
-        if constexpr (SOFTCAP) {
-          const float sv = sc[tw];
-          const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * kLog2e;
-          sc[tw] = (sv != sv) ? kNegInf : capped;
+      for (int u = 0; u < HL; ++u) {
+        mt[u] = kNegInf;
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          if constexpr (SOFTCAP) {
+            const float sv = sc[tw][u];
+            const float capped = softcap_tanh(sv * kLn2, p.softcap, inv_cap) * kLog2e;
+            sc[tw][u] = (sv != sv) ? kNegInf : capped;
+          }
+          if (base + 16 * tw + r >= t_end) sc[tw][u] = kNegInf;
+          sc[tw][u] = fmaxf(sc[tw][u], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
+          mt[u] = fmaxf(mt[u], sc[tw][u]);
         }
-        if (base + 16 * tw + r >= t_end) sc[tw] = kNegInf;
-        sc[tw] = fmaxf(sc[tw], kNegInf);  // NaN logit counts as -inf (common.rs:790-795)
-        mt = fmaxf(mt, sc[tw]);
       }
       // Emitted logits: parked in the chunk's LDS rows (lanes with nothing to park write to a spare
       // slot of their own), or stored through the sink's bounds-checked descriptor with an offset
       // that drops the store.  Under a uniform branch: calls without scores run 2 % faster that way
       // than with the stores always issued and dropped.
       if (p.scores) {  // uniform
-        const bool parks = j < staged_heads;
-        float *dst = parks ? dyn_lds + j * stage_row + (base - t_begin) + r : spare + 4 * TW * (int)threadIdx.x;
-        const uint32_t row_off = (uint32_t)(((int64_t)j * p.score_stride + r) * 4);
 #pragma unroll
-        for (int tw = 0; tw < TW; ++tw) {
-          const float logit = sc[tw] * kLn2;
-          dst[parks ? 16 * tw : tw] = logit;
-          const bool writes = sink.on && j < G && base + 16 * tw + r < t_end;
-          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, logit), sink.rsrc,
-                                                writes ? row_off + 4u * (uint32_t)(base + 16 * tw) : LogitSink<TW>::kDropped, 0u, 2);
+        for (int u = 0; u < HL; ++u) {
+          const int hj = HL * j + u;  // the head within the group
+          const bool parks = hj < staged_heads;
+          float *dst = parks ? dyn_lds + hj * stage_row + (base - t_begin) + r : spare + 4 * TW * (int)threadIdx.x + TW * u;
+          const uint32_t row_off = (uint32_t)(((int64_t)hj * p.score_stride + r) * 4);
+#pragma unroll
+          for (int tw = 0; tw < TW; ++tw) {
+            const float logit = sc[tw][u] * kLn2;
+            dst[parks ? 16 * tw : tw] = logit;
+            const bool writes = sink.on && hj < G && base + 16 * tw + r < t_end;
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, logit), sink.rsrc,
+                                                  writes ? row_off + 4u * (uint32_t)(base + 16 * tw) : LogitSink<TW>::kDropped, 0u, 2);
+          }
         }
       }
       // ---- online softmax: a head's tokens are the 16 lanes of one row ---------------------------
-      mt = group_allreduce_max<16>(mt);
-      const float m_new = fmaxf(m_run, mt);
-      const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-      m_run = m_new;
-      half2_t pk = {(_Float16)0.0f, (_Float16)0.0f};
-      float lsum = 0.0f;
+      float alpha[HL];
+      half2_t pk[HL];
+      bool moved = false;
 #pragma unroll
-      for (int tw = 0; tw < TW; ++tw) {
-        const float e = __builtin_amdgcn_exp2f(sc[tw] - m_ref);  // the row sum takes the unrounded weight
-        lsum += e;
-        pk[tw] = (_Float16)e;
+      for (int u = 0; u < HL; ++u) {
+        const float m_new = fmaxf(m_run[u], group_allreduce_max<16>(mt[u]));
+        const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
+        alpha[u] = __builtin_amdgcn_exp2f(m_run[u] - m_ref);
+        moved = moved || alpha[u] != 1.0f;
+        m_run[u] = m_new;
+        pk[u] = half2_t{(_Float16)0.0f, (_Float16)0.0f};
+        float lsum = 0.0f;
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          const float e = __builtin_amdgcn_exp2f(sc[tw][u] - m_ref);  // the row sum takes the unrounded weight
+          lsum += e;
+          pk[u][tw] = (_Float16)e;
+        }
+        l_run[u] = l_run[u] * alpha[u] + lsum;
       }
-      l_run = l_run * alpha + lsum;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-        // O accumulator register i belongs to head i, whose factor every lane of row i holds
+      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+        // O accumulator register i belongs to head i, whose factor every lane of row i holds (two heads
+        // per lane: to head i + 4 (j / 2), kept as slot i % 2 by lane group 2 (j / 2) + i / 2)
         float al[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 16 * i, 64);
+        for (int i = 0; i < 4; ++i) al[i] = (HL == 2) ? __shfl(alpha[i & 1], 16 * (2 * (j >> 1) + (i >> 1)), 64) : __shfl(alpha[0], 16 * i, 64);
 #pragma unroll
         for (int a = 0; a < NACC; ++a)
 #pragma unroll
@@ -925,12 +957,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
             for (int i = 0; i < 4; ++i) m_acc[sg][i] *= al[i];
         }
       }
-      // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of head r % 4
-      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][4][16];  // 64 words: writes and reads each touch every bank once
+      // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of the head of its row
+      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][4 * HL][16];  // 64 words per four heads: writes and reads each touch every bank once
       wave_lds_fence();  // the previous iteration's reads are done
-      p_strip[wave][j][r] = __builtin_bit_cast(uint32_t, pk);
+#pragma unroll
+      for (int u = 0; u < HL; ++u) p_strip[wave][HL * j + u][r] = __builtin_bit_cast(uint32_t, pk[u]);
       wave_lds_fence();
-      const u32x4_t w = *(const u32x4_t *)&p_strip[wave][ph][4 * j];
+      const u32x4_t w = *(const u32x4_t *)&p_strip[wave][pa_head][4 * j];
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
         const uint32_t sel = tw ? 0x07060302u : 0x05040100u;
@@ -971,7 +1004,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           const int kk = 2 * kp + u;
           const half8_t ka = code_operand<FMT>(kpc[kk], k_sel);
           // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q
-          const float c0 = qinit[kk];
+          const float c0 = qinit[kk][0];
           dot[u] = float4_t{c0, c0, c0, c0};
           dot[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qh[kk], dot[u], 0, 0, 0);
           dot[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, ql[kk], dot[u], 0, 0, 0);
@@ -983,7 +1016,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const half2_t dm = __builtin_bit_cast(half2_t, __builtin_amdgcn_ds_bpermute(hdr_src[i], (int)kpc[2 * kp + u].hdr));
-              s[tw][i] = fmaf((float)dm[0], dot[u][i], fmaf((float)dm[1], qsum[2 * kp + u], s[tw][i]));
+              s[tw][i] = fmaf((float)dm[0], dot[u][i], fmaf((float)dm[1], qsum[2 * kp + u][0], s[tw][i]));
             }
         } else {
           // scales of two blocks travel together
@@ -1037,10 +1070,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 
     // ---- online softmax: the running max of a head is shared by the four lane groups -----------
     mt = rows_allreduce_max(mt);
-    const float m_new = fmaxf(m_run, mt);
+    const float m_new = fmaxf(m_run[0], mt);
     const float m_ref = (m_new == kNegInf) ? 0.0f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-    m_run = m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run[0] - m_ref);
+    m_run[0] = m_new;
     float lsum = 0.0f;
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
@@ -1053,7 +1086,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         pa[tw][i] = (_Float16)e;
       }
     }
-    l_run = l_run * alpha + lsum;
+    l_run[0] = l_run[0] * alpha + lsum;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
       // O accumulator register i of lane group j belongs to head 4j + i: fetch that head's factor.
       float al[4];
@@ -1236,19 +1269,23 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 
   // ---- merge: lane groups (row sum), then the waves through LDS ---------------------------------
   if constexpr (TOKCOL) {
-    l_run = group_allreduce_sum<16>(l_run);  // lane group j holds head j
+#pragma unroll
+    for (int u = 0; u < HL; ++u) l_run[u] = group_allreduce_sum<16>(l_run[u]);  // lane group j holds head j (heads 2j, 2j + 1)
   } else {
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run[0] += __shfl_xor(l_run[0], 16, 64);
+    l_run[0] += __shfl_xor(l_run[0], 32, 64);
   }
   const int own_copy = (D == 64) ? ((r >> 2) & 1) : (r >> 2);  // the P copy scaled for this lane's output columns
   float (*lds_m)[16] = (float (*)[16])dyn_lds;
   float (*lds_l)[16] = lds_m + kWaves;
-  constexpr int MH = TOKCOL ? 4 : SH::MAXH;  // heads a workgroup merges (tokens as columns: groups of up to four)
+  constexpr int MH = TOKCOL ? 4 * HL : SH::MAXH;  // heads a workgroup merges (tokens as columns: groups of up to four or eight)
   float (*lds_acc)[MH][D + 4] = (float (*)[MH][D + 4])(dyn_lds + 2 * kWaves * 16);
   if (TOKCOL ? r == 0 : j == 0) {
-    lds_m[wave][TOKCOL ? j : r] = m_run;
-    lds_l[wave][TOKCOL ? j : r] = l_run;
+#pragma unroll
+    for (int u = 0; u < HL; ++u) {
+      lds_m[wave][TOKCOL ? HL * j + u : r] = m_run[u];
+      lds_l[wave][TOKCOL ? HL * j + u : r] = l_run[u];
+    }
   }
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg)
@@ -1257,7 +1294,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       const int ch = 32 * vblk[sg] + ((D == 64) ? half_slot_elem<FMT>(r & 3, r >> 3, c) : slot_elem<FMT>(r & 3, c));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (TOKCOL ? j == own_copy : 4 * j + i < MH) lds_acc[wave][TOKCOL ? i : 4 * j + i][ch] = o_acc[sg * VCH + c][i];  // (TOKCOL: row 4j + i is head i scaled for block j)
+        // (tokens as columns: row 4j + i is head i scaled for block j; two heads per lane: head i + 4 (j / 2) scaled for block j % 2)
+        if ((TOKCOL == 2) ? (j & 1) == own_copy : (TOKCOL ? j == own_copy : 4 * j + i < MH))
+          lds_acc[wave][(TOKCOL == 2) ? i + 4 * (j >> 1) : (TOKCOL ? i : 4 * j + i)][ch] = o_acc[sg * VCH + c][i];
     }
   __syncthreads();
 
@@ -1290,7 +1329,8 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
   constexpr int tile_rows = kWaves * 16 * TW;
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-  const bool tokcol = p.group <= 4;
+  const bool wide = D == 64 && p.group > 4 && p.group <= 8;  // two heads per lane (see the kernel)
+  const bool tokcol = p.group <= 4 || wide;
   // Packed rows without an index list are streamed (see the kernel); the slabs must start on a dword.
   const int64_t head_blocks = ((int64_t)p.kv_bs | (int64_t)p.head_stride) / 32;
   // (Measured per arm: q8_0 +10 % either way, q2_0 +10 % and q4_0 +3 % with tokens as columns; the
@@ -1306,16 +1346,20 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   // streamed tiles' LDS copies).
   constexpr int kTileCopies = 2 * kWaves * StreamCopy<FMT, D, TW>::kDwords * 4;
   constexpr int kStageBytes = (kTileCopies > 24 * 1024) ? 32 * 1024 : 48 * 1024;
-  const size_t merge_bytes = (2 * kWaves * 16 + kWaves * (tokcol ? 4 : BlockShape<D>::MAXH) * (D + 4)) * sizeof(float);
+  const size_t merge_bytes = (2 * kWaves * 16 + kWaves * (tokcol ? (wide ? 8 : 4) : BlockShape<D>::MAXH) * (D + 4)) * sizeof(float);
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
   auto pick = [&](auto tc, auto st) {
-    constexpr bool TC = decltype(tc)::value, ST = decltype(st)::value;
-    if constexpr (ST && (FMT == kFmtQ8_0 || TC || D == 64)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
+    constexpr int TC = decltype(tc)::value;
+    constexpr bool ST = decltype(st)::value;
+    if constexpr (ST && (FMT == kFmtQ8_0 || TC != 0 || D == 64)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
     else return cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, TC, false> : decode_blocks_kernel<FMT, D, TW, true, false, TC, false>)
                     : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, TC, false> : decode_blocks_kernel<FMT, D, TW, false, false, TC, false>);
   };
-  auto kern = stream_rows ? (tokcol ? pick(std::true_type{}, std::true_type{}) : pick(std::false_type{}, std::true_type{}))
-                          : (tokcol ? pick(std::true_type{}, std::false_type{}) : pick(std::false_type{}, std::false_type{}));
+  typedef std::integral_constant<int, 0> Rows;
+  typedef std::integral_constant<int, 1> Cols;
+  typedef std::integral_constant<int, (D == 64) ? 2 : 1> Cols2;  // (only head_dim 64 has the arm; `wide` is false elsewhere)
+  auto kern = stream_rows ? (wide ? pick(Cols2{}, std::true_type{}) : tokcol ? pick(Cols{}, std::true_type{}) : pick(Rows{}, std::true_type{}))
+                          : (wide ? pick(Cols2{}, std::false_type{}) : tokcol ? pick(Cols{}, std::false_type{}) : pick(Rows{}, std::false_type{}));
   // dynamic LDS: staged logits or spare slots, then (streamed rows) the tile copies; the merge reuses it
   constexpr size_t spare_bytes = 64 * kWaves * TW * 16;
   const size_t tile_bytes = stream_rows ? (size_t)kTileCopies : 0;
