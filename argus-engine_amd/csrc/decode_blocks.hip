@@ -450,6 +450,7 @@ struct StreamCopy {
 // in the even row and low part in the odd one, so lane group g keeps the two heads 2g and 2g + 1 (HL
 // = 2 logits per lane and tile); the P operand has head r % 4 + 4 (r / 8) in row r, scaled for block
 // r / 4 % 2 -- with two blocks per row the sixteen rows are exactly eight heads times two blocks.
+// At head_dim 128 (four blocks per row) the output MFMAs run twice, for heads 0..3 and 4..7.
 //
 // STREAM (rows packed back to back, no index list): a wave's tile is one contiguous run of bytes.
 // The per-lane block requests of the other path put a header and 16 or 32 code bytes at an 18- or
@@ -459,7 +460,7 @@ struct StreamCopy {
 // the run (one access per 64 bytes), park them in a wave-private LDS copy of the tile, and every lane
 // then reads the pieces of its MFMA operands straight from there: no trades between lanes at all.
 template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, int TOKCOL, bool STREAM>
-__global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0 || TOKCOL == 2) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
   using SH = BlockShape<D>;
   using CD = Codec<FMT>;
@@ -476,10 +477,14 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // head g, so the four registers of a result lane in lane group g all hold head g's logit and no
   // register has to be picked; the P operand of the output MFMAs has head r % 4 in row r.
   constexpr int HL = (TOKCOL == 2) ? 2 : 1;  // heads a lane keeps logits of
-  static_assert(TOKCOL != 2 || D == 64, "two heads per lane: the P copies are two blocks times eight heads");
+  static_assert(TOKCOL != 2 || D == 64 || D == 128, "two heads per lane: head_dim 64 and 128");
+  // P operands of the output MFMAs: one set of sixteen rows, or (two heads per lane at head_dim 128,
+  // where a row's four blocks leave room for four heads only) two sets, heads 0..3 and 4..7, over the
+  // same V operands and with accumulators of their own.
+  constexpr int NQ = (TOKCOL == 2 && D == 128) ? 2 : 1;
   const int rh = (TOKCOL == 2) ? (r >> 1) : (TOKCOL ? (r >> 2) : r);
   const int ph = (TOKCOL == 2) ? (r & 1) : (r & 3);                  // which part of the query the row carries
-  const int pa_head = (TOKCOL == 2) ? (r & 3) + 4 * (r >> 3) : (r & 3);  // head in row r of the P operand
+  const int pa_head = (TOKCOL == 2 && D == 64) ? (r & 3) + 4 * (r >> 3) : (r & 3);  // head in row r of the P operand (set q: + 4 q)
   static_assert(!(STREAM && INDEXED), "an index list gathers rows: they are read block by block");
 
   const int t_begin = split * p.chunk;
@@ -793,9 +798,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
   for (int i = 0; i < 4; ++i) hdr_src[i] = 4 * (20 * j + i);  // ds_bpermute byte address
 
-  float4_t o_acc[NACC];
+  float4_t o_acc[NQ * NACC];  // (set q at q * NACC)
 #pragma unroll
-  for (int a = 0; a < NACC; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int a = 0; a < NQ * NACC; ++a) o_acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   // sum over tokens of p * d (q4_0: times -8 it is the zero-point term of the lane's channels) or
   // of p * m (q4_1: the minimum term), per V piece; one more MFMA column each
   constexpr bool kHdrTerm = FMT != kFmtQ8_0;
@@ -807,11 +812,11 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // -(bias + zero point) it takes the bias back out), m_acc the plain weights times the minimum.
   constexpr bool kScaleP = TOKCOL;
   constexpr bool kMinTerm = kScaleP && F::kHasMin;
-  float4_t h_acc[VSEG], m_acc[kMinTerm ? VSEG : 1];
+  float4_t h_acc[NQ * VSEG], m_acc[kMinTerm ? NQ * VSEG : 1];  // (set q at q * VSEG)
 #pragma unroll
-  for (int sg = 0; sg < VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int sg = 0; sg < NQ * VSEG; ++sg) h_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int sg = 0; sg < (kMinTerm ? VSEG : 1); ++sg) m_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int sg = 0; sg < (kMinTerm ? NQ * VSEG : 1); ++sg) m_acc[sg] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run[HL], l_run[HL];  // per (lane = head r; tokens as columns: the HL heads of the lane group); l is this lane group's partial sum
 #pragma unroll
   for (int u = 0; u < HL; ++u) m_run[u] = kNegInf, l_run[u] = 0.0f;
@@ -827,7 +832,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   __shared__ uint32_t v_strip[kWaves][VL][(kStageV && !STREAM) ? 64 * 4 + 4 * 4 : 1];  // the staged V rows' code words, wave by wave
 
   for (int base = base0; base < t_end; base += kWaves * TILE) {
-    half4_t pa[TW];
+    half4_t pa[NQ][TW];
     if constexpr (TOKCOL) {
       // ---- logits: token base + 16 tw + r, head j (HL = 2: heads 2j and 2j + 1) -----------------
       float sc[TW][HL];
@@ -937,24 +942,29 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       if (__builtin_amdgcn_ballot_w64(moved) != 0) {
         // O accumulator register i belongs to head i, whose factor every lane of row i holds (two heads
         // per lane: to head i + 4 (j / 2), kept as slot i % 2 by lane group 2 (j / 2) + i / 2)
-        float al[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) al[i] = (HL == 2) ? __shfl(alpha[i & 1], 16 * (2 * (j >> 1) + (i >> 1)), 64) : __shfl(alpha[0], 16 * i, 64);
+        for (int q = 0; q < NQ; ++q) {
+          // (two sets: register i of set q is head 4q + i, slot i % 2 of lane group 2q + i / 2)
+          float al[4];
 #pragma unroll
-        for (int a = 0; a < NACC; ++a)
+          for (int i = 0; i < 4; ++i)
+            al[i] = (HL == 2) ? __shfl(alpha[i & 1], 16 * (2 * (NQ == 2 ? q : (j >> 1)) + (i >> 1)), 64) : __shfl(alpha[0], 16 * i, 64);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o_acc[a][i] *= al[i];
-        if constexpr (kHdrTerm) {
+          for (int a = 0; a < NACC; ++a)
 #pragma unroll
-          for (int sg = 0; sg < VSEG; ++sg)
+            for (int i = 0; i < 4; ++i) o_acc[q * NACC + a][i] *= al[i];
+          if constexpr (kHdrTerm) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) h_acc[sg][i] *= al[i];
-        }
-        if constexpr (kMinTerm) {
+            for (int sg = 0; sg < VSEG; ++sg)
 #pragma unroll
-          for (int sg = 0; sg < VSEG; ++sg)
+              for (int i = 0; i < 4; ++i) h_acc[q * VSEG + sg][i] *= al[i];
+          }
+          if constexpr (kMinTerm) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) m_acc[sg][i] *= al[i];
+            for (int sg = 0; sg < VSEG; ++sg)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) m_acc[q * VSEG + sg][i] *= al[i];
+          }
         }
       }
       // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of the head of its row
@@ -963,11 +973,14 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
       for (int u = 0; u < HL; ++u) p_strip[wave][HL * j + u][r] = __builtin_bit_cast(uint32_t, pk[u]);
       wave_lds_fence();
-      const u32x4_t w = *(const u32x4_t *)&p_strip[wave][pa_head][4 * j];
 #pragma unroll
-      for (int tw = 0; tw < TW; ++tw) {
-        const uint32_t sel = tw ? 0x07060302u : 0x05040100u;
-        pa[tw] = __builtin_bit_cast(half4_t, u32x2_t{__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel)});
+      for (int q = 0; q < NQ; ++q) {
+        const u32x4_t w = *(const u32x4_t *)&p_strip[wave][pa_head + 4 * q][4 * j];
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          const uint32_t sel = tw ? 0x07060302u : 0x05040100u;
+          pa[q][tw] = __builtin_bit_cast(half4_t, u32x2_t{__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel)});
+        }
       }
     } else {
     // ---- logits ---------------------------------------------------------------------------------
@@ -1083,7 +1096,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         // a handful of tokens the f16 roundings of the weights (2^-12 each) would not average out.
         const float e = __builtin_amdgcn_exp2f(s[tw][i] - m_ref);
         lsum += e;
-        pa[tw][i] = (_Float16)e;
+        pa[0][tw][i] = (_Float16)e;
       }
     }
     l_run[0] = l_run[0] * alpha + lsum;
@@ -1202,18 +1215,21 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         half4_t bv0[VCH], bv1[VCH], hv0 = {}, hv1 = {}, dv0 = {}, dv1 = {};
         v_operands(0, sg, bv0, hv0, dv0);
         v_operands(1, sg, bv1, hv1, dv1);
-        const half8_t pw = both(pa[0], pa[1]);
-        half8_t pv = pw;
-        if constexpr (kScaleP) {
-          pv = both(pa[0] * dv0, pa[1] * dv1);
-          if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv, both(ones, ones), h_acc[sg], 0, 0, 0);
-          if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pw, both(hv0, hv1), m_acc[sg], 0, 0, 0);
-        } else if constexpr (kHdrTerm) {
-          h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pw, both(hv0, hv1), h_acc[sg], 0, 0, 0);
-        }
 #pragma unroll
-        for (int c = 0; c < VCH; ++c)
-          o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv, both(bv0[c], bv1[c]), o_acc[sg * VCH + c], 0, 0, 0);
+        for (int q = 0; q < NQ; ++q) {
+          const half8_t pw = both(pa[q][0], pa[q][1]);
+          half8_t pv = pw;
+          if constexpr (kScaleP) {
+            pv = both(pa[q][0] * dv0, pa[q][1] * dv1);
+            if constexpr (kHdrTerm) h_acc[q * VSEG + sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv, both(ones, ones), h_acc[q * VSEG + sg], 0, 0, 0);
+            if constexpr (kMinTerm) m_acc[q * VSEG + sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pw, both(hv0, hv1), m_acc[q * VSEG + sg], 0, 0, 0);
+          } else if constexpr (kHdrTerm) {
+            h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pw, both(hv0, hv1), h_acc[sg], 0, 0, 0);
+          }
+#pragma unroll
+          for (int c = 0; c < VCH; ++c)
+            o_acc[q * NACC + sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pv, both(bv0[c], bv1[c]), o_acc[q * NACC + sg * VCH + c], 0, 0, 0);
+        }
       }
     } else {
 #pragma unroll
@@ -1222,13 +1238,14 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         for (int sg = 0; sg < VSEG; ++sg) {
           half4_t bv[VCH], hv = {}, dv = {};
           v_operands(tw, sg, bv, hv, dv);
-          half4_t pv = pa[tw];
+          static_assert(NQ == 1 || (TW == 2 && D == 128), "two sets of P operands come with the 32-token MFMAs");
+          half4_t pv = pa[0][tw];
           if constexpr (kScaleP) {
-            pv = pa[tw] * dv;
+            pv = pa[0][tw] * dv;
             if constexpr (kHdrTerm) h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, ones, h_acc[sg], 0, 0, 0);
-            if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, m_acc[sg], 0, 0, 0);
+            if constexpr (kMinTerm) m_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[0][tw], hv, m_acc[sg], 0, 0, 0);
           } else if constexpr (kHdrTerm) {
-            h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[tw], hv, h_acc[sg], 0, 0, 0);
+            h_acc[sg] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[0][tw], hv, h_acc[sg], 0, 0, 0);
           }
 #pragma unroll
           for (int c = 0; c < VCH; ++c) o_acc[sg * VCH + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(pv, bv[c], o_acc[sg * VCH + c], 0, 0, 0);
@@ -1246,17 +1263,19 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 
   if constexpr (kScaleP && kHdrTerm) {
 #pragma unroll
-    for (int sg = 0; sg < VSEG; ++sg)
+    for (int q = 0; q < NQ; ++q)
 #pragma unroll
-      for (int c = 0; c < VCH; ++c) {
-        const float bias = (D == 64) ? half_slot_bias<FMT>(c) : CD::slot_bias(c);
+      for (int sg = 0; sg < VSEG; ++sg)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float o = fmaf(-(bias + CD::kZero), h_acc[sg][i], o_acc[sg * VCH + c][i]);
-          if constexpr (kMinTerm) o += m_acc[sg][i];
-          o_acc[sg * VCH + c][i] = o;
+        for (int c = 0; c < VCH; ++c) {
+          const float bias = (D == 64) ? half_slot_bias<FMT>(c) : CD::slot_bias(c);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float o = fmaf(-(bias + CD::kZero), h_acc[q * VSEG + sg][i], o_acc[q * NACC + sg * VCH + c][i]);
+            if constexpr (kMinTerm) o += m_acc[q * VSEG + sg][i];
+            o_acc[q * NACC + sg * VCH + c][i] = o;
+          }
         }
-      }
   } else if constexpr (kHdrTerm) {
     constexpr float kTerm = (FMT == kFmtQ4_0) ? -CD::kZero : 1.0f;
 #pragma unroll
@@ -1294,9 +1313,12 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
       const int ch = 32 * vblk[sg] + ((D == 64) ? half_slot_elem<FMT>(r & 3, r >> 3, c) : slot_elem<FMT>(r & 3, c));
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        // (tokens as columns: row 4j + i is head i scaled for block j; two heads per lane: head i + 4 (j / 2) scaled for block j % 2)
-        if ((TOKCOL == 2) ? (j & 1) == own_copy : (TOKCOL ? j == own_copy : 4 * j + i < MH))
-          lds_acc[wave][(TOKCOL == 2) ? i + 4 * (j >> 1) : (TOKCOL ? i : 4 * j + i)][ch] = o_acc[sg * VCH + c][i];
+        // (tokens as columns: row 4j + i is head i scaled for block j; two heads per lane at head_dim 64:
+        // head i + 4 (j / 2) scaled for block j % 2, at 128: set q holds head 4q + i)
+#pragma unroll
+        for (int q = 0; q < NQ; ++q)
+          if ((TOKCOL == 2 && D == 64) ? (j & 1) == own_copy : (TOKCOL ? j == own_copy : 4 * j + i < MH))
+            lds_acc[wave][(TOKCOL == 2 && D == 64) ? i + 4 * (j >> 1) : (TOKCOL ? 4 * q + i : 4 * j + i)][ch] = o_acc[q * NACC + sg * VCH + c][i];
     }
   __syncthreads();
 
@@ -1329,7 +1351,7 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
   constexpr int tile_rows = kWaves * 16 * TW;
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-  const bool wide = D == 64 && p.group > 4 && p.group <= 8;  // two heads per lane (see the kernel)
+  const bool wide = (D == 64 || D == 128) && p.group > 4 && p.group <= 8;  // two heads per lane (see the kernel)
   const bool tokcol = p.group <= 4 || wide;
   // Packed rows without an index list are streamed (see the kernel); the slabs must start on a dword.
   const int64_t head_blocks = ((int64_t)p.kv_bs | (int64_t)p.head_stride) / 32;
@@ -1357,7 +1379,7 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   };
   typedef std::integral_constant<int, 0> Rows;
   typedef std::integral_constant<int, 1> Cols;
-  typedef std::integral_constant<int, (D == 64) ? 2 : 1> Cols2;  // (only head_dim 64 has the arm; `wide` is false elsewhere)
+  typedef std::integral_constant<int, (D == 64 || D == 128) ? 2 : 1> Cols2;  // (head_dim 256 has no such arm; `wide` is false there)
   auto kern = stream_rows ? (wide ? pick(Cols2{}, std::true_type{}) : tokcol ? pick(Cols{}, std::true_type{}) : pick(Rows{}, std::true_type{}))
                           : (wide ? pick(Cols2{}, std::false_type{}) : tokcol ? pick(Cols{}, std::false_type{}) : pick(Rows{}, std::false_type{}));
   // dynamic LDS: staged logits or spare slots, then (streamed rows) the tile copies; the merge reuses it

@@ -141,9 +141,10 @@ def test_ragged_lengths_at_every_head_dim(fmt, d):
 @pytest.mark.parametrize("d", [64, 128, 256])
 def test_every_group_width_with_and_without_scores(fmt, d):
     # Up to four query heads per KV head the kernel keeps one head per lane group (the logits MFMA
-    # has the tokens in its columns); wider groups keep the heads in the columns.  Every head must
-    # get its own logits in both, with the scores emitted or not, over ragged and multi-tile rows.
-    for g in (1, 2, 3, 4, 5, 8):
+    # has the tokens in its columns), five to eight at head_dim 64 and 128 two heads per lane group;
+    # wider groups keep the heads in the columns.  Every head must get its own logits in each, with
+    # the scores emitted or not, over ragged and multi-tile rows.
+    for g in (1, 2, 3, 4, 5, 6, 7, 8) + ((9, 16) if d != 256 else ()):  # (head_dim 256 takes groups of up to 8)
         for L in (97, 1300):
             run_case(fmt, 2 * g, 2, d, L, cap=L + 5, seed=g + L + d, scores=bool((g + L) & 1))
             run_case(fmt, 2 * g, 2, d, L, cap=L + 5, seed=g + L + d + 1, scores=not ((g + L) & 1))
@@ -188,7 +189,8 @@ def test_soft_cap_on_block_caches(fmt, hq, hkv, d, L):
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "q4_1", "q8_0", "q2_0"])
-@pytest.mark.parametrize("hq,hkv,d,L,cap", [(14, 2, 64, 700, 1500), (32, 8, 128, 1000, 4096), (8, 4, 256, 333, 800), (8, 2, 128, 9000, 20000)])
+@pytest.mark.parametrize("hq,hkv,d,L,cap", [(14, 2, 64, 700, 1500), (32, 8, 128, 1000, 4096), (8, 4, 256, 333, 800), (8, 2, 128, 9000, 20000),
+                                            (16, 2, 128, 700, 1500), (14, 2, 128, 2100, 2500)])
 def test_index_list_over_block_caches(fmt, hq, hkv, d, L, cap):
     # Post-eviction addressing: token t lives in slot kv_index[t] (any order, here shuffled), and the
     # result is the attention over the gathered rows.
