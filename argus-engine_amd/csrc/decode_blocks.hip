@@ -1351,7 +1351,9 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
   constexpr int tile_rows = kWaves * 16 * TW;
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
-  const bool wide = (D == 64 || D == 128) && p.group > 4 && p.group <= 8;  // two heads per lane (see the kernel)
+  // Two heads per lane (see the kernel).  At head_dim 128 only without scores: with them the arm's
+  // single-float logit stores (two per lane and tile) make it 8-16 % slower than the tokens-as-rows arm.
+  const bool wide = (D == 64 || (D == 128 && p.scores == nullptr)) && p.group > 4 && p.group <= 8;
   const bool tokcol = p.group <= 4 || wide;
   // Packed rows without an index list are streamed (see the kernel); the slabs must start on a dword.
   const int64_t head_blocks = ((int64_t)p.kv_bs | (int64_t)p.head_stride) / 32;
