@@ -401,7 +401,13 @@ struct BlockFallback {
     }
     if (p.scores) {
       float *srow = p.scores + (int64_t)b * p.score_bs + (int64_t)h * p.score_stride;
-      for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = u;
+      // (logits + statistics form: exp(0 - 0) / len is the same uniform weight)
+      for (int t = threadIdx.x; t < p.len; t += blockDim.x) srow[t] = p.score_stats ? 0.0f : u;
+      if (p.score_stats && threadIdx.x == 0) {
+        float *st = p.score_stats + (int64_t)b * p.stats_bs + (int64_t)h * 2;
+        st[0] = 0.0f;
+        st[1] = (float)p.len;
+      }
     }
     return true;
   }

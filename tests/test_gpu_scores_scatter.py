@@ -310,6 +310,13 @@ def test_statistics_form_on_the_other_decode_kernels_and_the_fallback_row():
     out, sc, out2, lg, st = _decode_both_forms(qn, f16(k32), f16(v32), hkv, L, cap, 1)
     assert torch.equal(out, out2)
     assert np.allclose(host(sc)[..., :L], 1.0 / L)
+    # the same row over the block cache, in both forms
+    qnd = dev(qn)
+    ctx().attention_gen(qnd, kd, vd, o1, hkv, L, cap, scores=s1, score_stride=cap, kv_dtype=A.Q4_0)
+    ctx().attention_gen(qnd, kd, vd, o2, hkv, L, cap, scores=s2, score_stride=cap, kv_dtype=A.Q4_0, score_stats=t2)
+    assert torch.equal(o1, o2) and bool(torch.isfinite(o1).all())
+    assert np.allclose(host(s1)[..., :L], 1.0 / L)
+    assert np.allclose(host(torch.exp(s2[..., :L] - t2[..., 0:1]) / t2[..., 1:2]), 1.0 / L)
     assert not host(lg)[..., :L].any() and np.array_equal(host(st).reshape(-1, 2), np.tile([0.0, float(L)], (hq, 1)))
     assert ctx().attention_gen(dev(q), dev(f16(k32)), dev(f16(v32)), out, hkv, L, cap, score_stats=st, check=False) == A.ERR_INVALID
 
