@@ -169,7 +169,7 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
     return r
 
 
-def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1, scores=False):
+def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1, scores=False, stats=False):
     """Decode attention over a block-quantised cache (q4_0 / q8_0 / q2_0 rows of 18- / 34- / 12-byte blocks):
     synthetic blocks (random codes, f16 scales sized for N(0,1)-like values); algorithmic bytes are
     the attended block rows of K and V plus Q and out."""
@@ -194,13 +194,14 @@ def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1,
     q = torch.randn((batch, hq, d), generator=g, device="cuda", dtype=torch.float32)
     out = torch.empty((batch, hq, d), device="cuda", dtype=torch.float32)
     sc = torch.empty((batch, hq, L), device="cuda", dtype=torch.float32) if scores else None
+    st = torch.empty((batch, hq, 2), device="cuda", dtype=torch.float32) if (scores and stats) else None
     state = {"i": 0}
 
     def step():
         i = state["i"] % rotate
         state["i"] += 1
         ctx.attention_gen(q, ks[i], vs[i], out, hkv, L, L, batch=batch, kv_batch_stride=hkv * L * d, kv_dtype=kv_dtype,
-                          scores=sc, score_stride=L if scores else 0)
+                          scores=sc, score_stride=L if scores else 0, score_stats=st)
 
     wall, kernel_ms, tail_ms = measure(ctx, step, steps, warmup)
     nbytes = batch * (2 * hkv * L * row_bytes + 2 * hq * d * 4 + (hq * L * 4 if scores else 0))
@@ -621,8 +622,10 @@ def main():
             "head_dim 64 (Llama-3.2-1B head shape), 32 caches per launch, 183 MB")
         add("cfg3_q4_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q4_0 rows attended in-kernel, 604 MB of blocks")
-        add("cfg3_q4_0_blocks_L32768_b16_scores", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew, scores=True),
-            "q4_0 rows with scores emitted (67 MB of logits per call)")
+        add("cfg3_q4_0_blocks_L32768_b16_scores", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew, scores=True, stats=True),
+            "q4_0 rows with scores emitted as logits + (max, sum) per row (67 MB per call)")
+        add("cfg3_q4_0_blocks_L32768_b16_scores_as_probabilities", bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 16, es, ew, scores=True),
+            "the trait's form: combine_us is the pass that rewrites the 67 MB of logits as probabilities")
         add("cfg3_q8_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q8_0", 32, 8, 128, 32768, 16, es, ew),
             "--kv-format q8_0 rows attended in-kernel, 1141 MB of blocks")
         add("cfg3_q2_0_blocks_L32768_b16", bench_decode_blocks(ctx, "q2_0", 32, 8, 128, 32768, 16, es, ew),
