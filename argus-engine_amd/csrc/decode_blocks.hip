@@ -9,12 +9,14 @@
 // byte i, element 16 + i in the high nibble; q8_0: x = d * c, c = int8; q2_0: [f16 d][f16 m][8 code
 // bytes], x = d * n + m, element 4i + k in bits 2k, 2k+1 of code byte i (dtype_layout.rs:146-166).
 //
-// Same data flow as decode_mfma.hip.  Rows are requested one whole block per lane (contiguous 16 or
-// 32 code bytes, so a request touches each cache line once) and the lanes then trade dwords
-// (v_permlane swaps for K, a wave-private LDS strip for 4-bit V rows) until each holds the 4 (q4) or
-// 8 (q8) code bytes of its MFMA operand, which it turns into 8 f16 values: q8 bytes go under the
-// exponent of 1024 with v_perm and a packed subtract leaves the exact integer; q4 nibbles are
-// masked into the mantissa of 64 + n.
+// Same data flow as decode_mfma.hip.  Packed rows read without an index list are streamed: a wave
+// fetches its tile as one contiguous run, parks it in a private LDS copy and every lane reads the
+// pieces of its operands from there (STREAM, see the kernel).  Otherwise rows are requested one
+// whole block per lane (contiguous 16 or 32 code bytes, so a request touches each cache line once)
+// and the lanes then trade dwords (v_permlane swaps for K, a wave-private LDS strip for 4-bit V
+// rows).  Either way each lane ends up with the 4 (q4) or 8 (q8) code bytes of its MFMA operand,
+// which it turns into 8 f16 values: q8 bytes go under the exponent of 1024 with v_perm and a packed
+// subtract leaves the exact integer; q4 nibbles are masked into the mantissa of 64 + n.
 //   S^T[token][head] = sum over blocks kk of d_kk(token) * (C_kk . Q_kk^T)
 //       v_mfma_f32_16x16x32_f16 per 32-element block with A = the integer codes n - 8 (q4_0), n
 //       (q4_1) or c (q8_0) -- lane (j, r) = token r, code bytes 4j..4j+3 of block kk, i.e. elements
@@ -23,13 +25,16 @@
 //       result: the result lane (j, h) holds tokens 4j..4j+3, whose scales sit in lanes 20j + i of
 //       the wave and are fetched with ds_bpermute (q4_1 adds m_kk(token) * sum of Q_kk).  Logits
 //       therefore carry no f16 rounding of d * (n - 8), and the emitted scores keep the 1e-4 bar.
-//       With at most four query heads per KV head the two operands change places (TOKCOL, see the
-//       kernel): S[head][token], the result lane (j, n) holds token n for the heads 0..3, lane
-//       group j keeps head j and applies the scales of its own token.
-//   O[head][channel] = P . V     v_mfma_f32_16x16x16_f16
+//       With at most four query heads per KV head (eight at head_dim 64, and at 128 when no scores
+//       are emitted) the two operands change places (TOKCOL, see the kernel): S[head][token], the
+//       result lane (j, n) holds token n, lane group j keeps head j (heads 2j, 2j + 1) and applies
+//       the scales of its own token; the query's hi and lo parts are two rows of the one operand.
+//   O[head][channel] = P . V     v_mfma_f32_16x16x16_f16 (16x16x32 over two tiles at head_dim 128, TOKCOL)
 //       B: lane (j, r) loads, for tokens 4j..4j+3, code bytes 4(r%4).. of block r/4, dequantises
 //       them to f16 (one rounding, 2^-12 relative: far below the 2e-3 output bar) and gets
 //       8 channels x 4 tokens; the per-channel operands are the 4x8 transpose of that.
+//       TOKCOL: the V operand is the bare code and the block scale multiplies the P operand instead,
+//       whose spare rows hold one copy of the weights per block of output columns.
 // Partials and the combine pass are those of the other decode kernels (decode_common.hpp).
 #include "decode_common.hpp"
 
@@ -442,17 +447,18 @@ struct StreamCopy {
 };
 
 // Waves per SIMD the register allocation aims at: 4 at head_dim 64 (128 registers), 3 at 128 (168;
-// q8_0 would spill there and stays at 2), 2 at 256.  Without the bound most instantiations came out a
+// q8_0 would spill there and stays at 2, as does the arm with two sets of output accumulators), 2 at 256.  Without the bound most instantiations came out a
 // few registers on one or the other side of a step depending on unrelated edits (q4_0 at 128: 165 or
 // 170 registers; q8_0 at 256: 256 or 257).
-// TOKCOL (at most four query heads per KV head): the logits MFMA takes the
-// query as its row operand, head r / 4 in row r, and the codes as its column operand, so result lane
-// (g, n) holds token n of the tile for head g in each of its four registers (rows 4g..4g+3).  Lane
-// group g keeps head g: the token's block scales are the lane's own (no exchange), the
+// TOKCOL = 1 (at most four query heads per KV head): the logits MFMA takes the
+// query as its row operand, head r / 4 in row r (its high part in the first of a head's four rows,
+// its low part in the second, zeros in the others), and the codes as its column operand, so result
+// lane (g, n) holds token n of the tile for head g (the two partial dot products in registers 0 and
+// 1).  Lane group g keeps head g: the token's block scales are the lane's own (no exchange), the
 // softmax runs once per logit instead of once per operand column, a head's maximum is a reduction
 // inside one 16-lane row, and the probabilities reach the P operand's layout (lane (j, r): tokens
 // 4j..4j+3 of head r % 4) through 256 bytes of LDS per wave.
-// TOKCOL = 2 (head_dim 64, five to eight heads per KV head): the query rows are head r / 2, high part
+// TOKCOL = 2 (head_dim 64 and 128, five to eight heads per KV head): the query rows are head r / 2, high part
 // in the even row and low part in the odd one, so lane group g keeps the two heads 2g and 2g + 1 (HL
 // = 2 logits per lane and tile); the P operand has head r % 4 + 4 (r / 8) in row r, scaled for block
 // r / 4 % 2 -- with two blocks per row the sixteen rows are exactly eight heads times two blocks.
@@ -462,9 +468,9 @@ struct StreamCopy {
 // The per-lane block requests of the other path put a header and 16 or 32 code bytes at an 18- or
 // 34-byte stride under every lane, which the texture path serves lane by lane: the q4_0 kernel made
 // as many L1 accesses as the F16 kernel for 3.6 times fewer bytes (17 per 128-byte line, counter
-// TCP_TOTAL_CACHE_ACCESSES against TCP_TCC_READ_REQ).  Here the lanes fetch consecutive dwords of
-// the run (one access per 64 bytes), park them in a wave-private LDS copy of the tile, and every lane
-// then reads the pieces of its MFMA operands straight from there: no trades between lanes at all.
+// TCP_TOTAL_CACHE_ACCESSES against TCP_TCC_READ_REQ).  Here the lanes fetch consecutive 8-byte pieces
+// of the run, park them in a wave-private LDS copy of the tile, and every lane then reads the pieces
+// of its MFMA operands straight from there: no trades between lanes at all.
 template <int FMT, int D, int TW, bool SOFTCAP, bool INDEXED, int TOKCOL, bool STREAM>
 __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == kFmtQ8_0 || TOKCOL == 2) ? 2 : 3) : 2) void decode_blocks_kernel(const DecodeParams p) {
   using F = BlockFmt<FMT>;
