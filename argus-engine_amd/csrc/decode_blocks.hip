@@ -517,7 +517,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // block_to_pieces).  A wave-wide request covers 16 rows x 4 blocks: one 16-token tile at
   // head_dim 128, half of one at 256 (two requests per tile), both tiles of an iteration at 64
   // (lane group j takes block j % 2 of tile j / 2).
-  static_assert(D != 64 || TW == 2, "head_dim 64 pairs the two tiles of an iteration in one request");
+  static_assert(D != 64 || TW == 2 || (TW == 4 && TOKCOL && STREAM), "head_dim 64 pairs the two tiles of an iteration in one request; streamed, tokens as columns: four tiles");
   constexpr int KQ = (D == 64) ? 1 : KK / 4;        // requests per tile (head_dim 64: per iteration)
   constexpr int KL = (D == 64) ? 1 : TW * KQ;
   RawBlock<FMT> kblk[KL];
@@ -548,7 +548,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
   const int stage_row = p.chunk + 4;
   const int staged_heads = p.stage_scores ? p.group : 0;
-  constexpr int kSpareFloats = 64 * kWaves * TW * 4;  // 16 TW bytes per lane
+  // Spare slots of lanes that park no logit: 4 TW floats per lane (tokens as columns: HL TW).
+  constexpr int kSparePerLane = TOKCOL ? HL * TW : 4 * TW;
+  constexpr int kSpareFloats = 64 * kWaves * kSparePerLane;
   uint32_t *const tiles = (uint32_t *)(dyn_lds + (p.stage_scores ? staged_heads * stage_row : kSpareFloats));
   uint32_t *const k_tile = tiles + wave * kTileDw, *const v_tile = tiles + (kWaves + wave) * kTileDw;
   const uint32_t run_bytes = (uint32_t)min((int64_t)p.len * RBY, (int64_t)0xffffffffll);
@@ -834,12 +836,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   for (int u = 0; u < HL; ++u) m_run[u] = kNegInf, l_run[u] = 0.0f;
   // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
   // then the merge area.
-  __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][LogitSink<TW>::kStageFloats];
+  using Sink = LogitSink<(TW > 2) ? 2 : TW>;  // (the tokens-as-columns arm only takes its descriptor from it)
+  __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][Sink::kStageFloats];
   // Lanes that park nothing write here: the sink's stage when the logits are staged (the sink is off
   // then), else the start of the dynamic area (the merge uses it after the loop only).
-  static_assert(sizeof(logit_stage) >= 64 * kWaves * TW * 16, "spare slots of 16 TW bytes per lane");
+  static_assert(sizeof(logit_stage) >= kSpareFloats * sizeof(float), "room for every lane's spare slots");
   float *spare = p.stage_scores ? &logit_stage[0][0] : dyn_lds;
-  const LogitSink<TW> sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
+  const Sink sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
   int base_last = -(1 << 30);
   __shared__ uint32_t v_strip[kWaves][VL][(kStageV && !STREAM) ? 64 * 4 + 4 * 4 : 1];  // the staged V rows' code words, wave by wave
 
@@ -918,7 +921,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         for (int u = 0; u < HL; ++u) {
           const int hj = HL * j + u;  // the head within the group
           const bool parks = hj < staged_heads;
-          float *dst = parks ? dyn_lds + hj * stage_row + (base - t_begin) + r : spare + 4 * TW * (int)threadIdx.x + TW * u;
+          float *dst = parks ? dyn_lds + hj * stage_row + (base - t_begin) + r : spare + kSparePerLane * (int)threadIdx.x + TW * u;
           const uint32_t row_off = (uint32_t)(((int64_t)hj * p.score_stride + r) * 4);
 #pragma unroll
           for (int tw = 0; tw < TW; ++tw) {
@@ -926,13 +929,14 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
             dst[parks ? 16 * tw : tw] = logit;
             const bool writes = sink.on && hj < G && base + 16 * tw + r < t_end;
             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, logit), sink.rsrc,
-                                                  writes ? row_off + 4u * (uint32_t)(base + 16 * tw) : LogitSink<TW>::kDropped, 0u, 2);
+                                                  writes ? row_off + 4u * (uint32_t)(base + 16 * tw) : Sink::kDropped, 0u, 2);
           }
         }
       }
       // ---- online softmax: a head's tokens are the 16 lanes of one row ---------------------------
       float alpha[HL];
-      half2_t pk[HL];
+      constexpr int NPD = (TW + 1) / 2;  // dwords that hold a token column's TW weights (two per dword)
+      half2_t pk[HL][NPD];
       bool moved = false;
 #pragma unroll
       for (int u = 0; u < HL; ++u) {
@@ -941,13 +945,14 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         alpha[u] = __builtin_amdgcn_exp2f(m_run[u] - m_ref);
         moved = moved || alpha[u] != 1.0f;
         m_run[u] = m_new;
-        pk[u] = half2_t{(_Float16)0.0f, (_Float16)0.0f};
+#pragma unroll
+        for (int d2 = 0; d2 < NPD; ++d2) pk[u][d2] = half2_t{(_Float16)0.0f, (_Float16)0.0f};
         float lsum = 0.0f;
 #pragma unroll
         for (int tw = 0; tw < TW; ++tw) {
           const float e = __builtin_amdgcn_exp2f(sc[tw][u] - m_ref);  // the row sum takes the unrounded weight
           lsum += e;
-          pk[u][tw] = (_Float16)e;
+          pk[u][tw >> 1][tw & 1] = (_Float16)e;
         }
         l_run[u] = l_run[u] * alpha[u] + lsum;
       }
@@ -980,20 +985,27 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         }
       }
       // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of the head of its row
-      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][4 * HL][16];  // 64 words per four heads: writes and reads each touch every bank once
+      __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][NPD][4 * HL][16];  // 64 words per four heads: writes and reads each touch every bank once
       wave_lds_fence();  // the previous iteration's reads are done
 #pragma unroll
-      for (int u = 0; u < HL; ++u) p_strip[wave][HL * j + u][r] = __builtin_bit_cast(uint32_t, pk[u]);
+      for (int u = 0; u < HL; ++u)
+#pragma unroll
+        for (int d2 = 0; d2 < NPD; ++d2) p_strip[wave][d2][HL * j + u][r] = __builtin_bit_cast(uint32_t, pk[u][d2]);
       wave_lds_fence();
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        const u32x4_t w = *(const u32x4_t *)&p_strip[wave][pa_head + 4 * q][4 * j];
+      for (int q = 0; q < NQ; ++q)
 #pragma unroll
-        for (int tw = 0; tw < TW; ++tw) {
-          const uint32_t sel = tw ? 0x07060302u : 0x05040100u;
-          pa[q][tw] = __builtin_bit_cast(half4_t, u32x2_t{__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel)});
+        for (int d2 = 0; d2 < NPD; ++d2) {
+          const u32x4_t w = *(const u32x4_t *)&p_strip[wave][d2][pa_head + 4 * q][4 * j];
+#pragma unroll
+          for (int h2 = 0; h2 < 2; ++h2) {
+            const int tw = 2 * d2 + h2;
+            if (tw < TW) {
+              const uint32_t sel = h2 ? 0x07060302u : 0x05040100u;
+              pa[q][tw] = __builtin_bit_cast(half4_t, u32x2_t{__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel)});
+            }
+          }
         }
-      }
     } else {
     // ---- logits ---------------------------------------------------------------------------------
     float4_t s[TW];
@@ -1361,7 +1373,9 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 template <int FMT, int D>
 int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t stream) {
   constexpr int TW = (D == 256) ? 1 : 2;  // head_dim 256 at two tiles needs every register (one wave per SIMD)
-  constexpr int tile_rows = kWaves * 16 * TW;
+  // Head_dim 64, rows streamed, tokens as columns: four tiles (64 tokens) per wave iteration -- its
+  // rows are half as long, and the softmax and the exchanges of an iteration cost the same.
+  constexpr int TW64 = 4;
   const bool cap = p.softcap > 0.0f, indexed = p.kv_index != nullptr;
   // Two heads per lane (see the kernel).  At head_dim 128 only without scores: with them the arm's
   // single-float logit stores (two per lane and tile) make it 8-16 % slower than the tokens-as-rows arm.
@@ -1380,14 +1394,17 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   // With scores the chunks are kept short enough for a workgroup's logits to wait in LDS until its
   // token loop is over (kStageBytes; two workgroups per CU still fit beside the V strips or the
   // streamed tiles' LDS copies).
-  constexpr int kTileCopies = 2 * kWaves * StreamCopy<FMT, D, TW>::kDwords * 4;
-  constexpr int kStageBytes = (kTileCopies > 24 * 1024) ? 32 * 1024 : 48 * 1024;
+  const bool four_tiles = D == 64 && tokcol && stream_rows;
+  const int tile_rows = kWaves * 16 * (four_tiles ? TW64 : TW);
+  const int kTileCopies = 2 * kWaves * (four_tiles ? StreamCopy<FMT, D, TW64>::kDwords : StreamCopy<FMT, D, TW>::kDwords) * 4;
+  const int kStageBytes = (kTileCopies > 24 * 1024) ? 32 * 1024 : 48 * 1024;
   const size_t merge_bytes = (2 * kWaves * 16 + kWaves * (tokcol ? (wide ? 8 : 4) : BlockShape<D>::MAXH) * (D + 4)) * sizeof(float);
   const int max_chunk = staged_chunk_limit(ctx, p, kStageBytes, tile_rows);
   auto pick = [&](auto tc, auto st) {
     constexpr int TC = decltype(tc)::value;
     constexpr bool ST = decltype(st)::value;
-    if constexpr (ST && (FMT == kFmtQ8_0 || TC != 0 || D == 64)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
+    if constexpr (ST && D == 64 && TC != 0) return cap ? decode_blocks_kernel<FMT, D, TW64, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW64, false, false, TC, true>;
+    else if constexpr (ST && (FMT == kFmtQ8_0 || TC != 0 || D == 64)) return cap ? decode_blocks_kernel<FMT, D, TW, true, false, TC, true> : decode_blocks_kernel<FMT, D, TW, false, false, TC, true>;
     else return cap ? (indexed ? decode_blocks_kernel<FMT, D, TW, true, true, TC, false> : decode_blocks_kernel<FMT, D, TW, true, false, TC, false>)
                     : (indexed ? decode_blocks_kernel<FMT, D, TW, false, true, TC, false> : decode_blocks_kernel<FMT, D, TW, false, false, TC, false>);
   };
@@ -1397,7 +1414,8 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   auto kern = stream_rows ? (wide ? pick(Cols2{}, std::true_type{}) : tokcol ? pick(Cols{}, std::true_type{}) : pick(Rows{}, std::true_type{}))
                           : (wide ? pick(Cols2{}, std::false_type{}) : tokcol ? pick(Cols{}, std::false_type{}) : pick(Rows{}, std::false_type{}));
   // dynamic LDS: staged logits or spare slots, then (streamed rows) the tile copies; the merge reuses it
-  constexpr size_t spare_bytes = 64 * kWaves * TW * 16;
+  // (the spare slots of lanes that park no logit: 4 TW floats per lane, tokens as columns HL TW)
+  const size_t spare_bytes = 64 * kWaves * sizeof(float) * (tokcol ? (wide ? 2 : 1) * (four_tiles ? TW64 : TW) : 4 * TW);
   const size_t tile_bytes = stream_rows ? (size_t)kTileCopies : 0;
   const int wgs_per_cu = argus_wgs_per_cu(ctx, kern, 64 * kWaves,
                                           max_chunk > 0 ? (size_t)kStageBytes + tile_bytes : std::max(merge_bytes, spare_bytes + tile_bytes));
