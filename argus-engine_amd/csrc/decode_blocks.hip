@@ -551,7 +551,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // Spare slots of lanes that park no logit: 4 TW floats per lane (tokens as columns: HL TW).
   constexpr int kSparePerLane = TOKCOL ? HL * TW : 4 * TW;
   constexpr int kSpareFloats = 64 * kWaves * kSparePerLane;
-  uint32_t *const tiles = (uint32_t *)(dyn_lds + (p.stage_scores ? staged_heads * stage_row : kSpareFloats));
+  // Tokens as columns: [staged logits][spare slots][tile copies]; tokens as rows: [staged logits, or
+  // the spare slots][tile copies] (with staged logits its spare slots are the sink's static stage).
+  const int spare_at = (TOKCOL && p.stage_scores) ? staged_heads * stage_row : 0;  // floats
+  uint32_t *const tiles = (uint32_t *)(dyn_lds + (TOKCOL ? spare_at + kSpareFloats : (p.stage_scores ? staged_heads * stage_row : kSpareFloats)));
   uint32_t *const k_tile = tiles + wave * kTileDw, *const v_tile = tiles + (kWaves + wave) * kTileDw;
   const uint32_t run_bytes = (uint32_t)min((int64_t)p.len * RBY, (int64_t)0xffffffffll);
   const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void *)kb, 0, STREAM ? run_bytes : 0u, kBufferFlags);
@@ -837,12 +840,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // Dynamic LDS: the chunk's logits when they are staged (p.stage_scores: G rows of chunk + 4 floats),
   // then the merge area.
   using Sink = LogitSink<(TW > 2) ? 2 : TW>;  // (the tokens-as-columns arm only takes its descriptor from it)
-  __shared__ __attribute__((aligned(16))) float logit_stage[kWaves][Sink::kStageFloats];
-  // Lanes that park nothing write here: the sink's stage when the logits are staged (the sink is off
-  // then), else the start of the dynamic area (the merge uses it after the loop only).
-  static_assert(sizeof(logit_stage) >= kSpareFloats * sizeof(float), "room for every lane's spare slots");
-  float *spare = p.stage_scores ? &logit_stage[0][0] : dyn_lds;
-  const Sink sink(p, logit_stage[wave], b, kvh * G, G, lane, t_end);
+  constexpr bool kSinkStage = !TOKCOL;  // (the tokens-as-columns arms store single logits: no static LDS for the sink)
+  __shared__ __attribute__((aligned(16))) float logit_stage[kSinkStage ? kWaves : 1][kSinkStage ? Sink::kStageFloats : 4];
+  // Lanes that park nothing write to spare slots: in the dynamic area (see `tiles`), or, tokens as
+  // rows with staged logits, in the sink's stage (the sink is off then).
+  static_assert(!kSinkStage || sizeof(logit_stage) >= kSpareFloats * sizeof(float), "room for every lane's spare slots");
+  float *spare = TOKCOL ? dyn_lds + spare_at : (p.stage_scores ? &logit_stage[0][0] : dyn_lds);
+  const Sink sink(p, logit_stage[kSinkStage ? wave : 0], b, kvh * G, G, lane, t_end);
   int base_last = -(1 << 30);
   __shared__ uint32_t v_strip[kWaves][VL][(kStageV && !STREAM) ? 64 * 4 + 4 * 4 : 1];  // the staged V rows' code words, wave by wave
 
@@ -1417,13 +1421,14 @@ int launch_blocks(argus_hip_ctx *ctx, DecodeParams &p, int batch, hipStream_t st
   // (the spare slots of lanes that park no logit: 4 TW floats per lane, tokens as columns HL TW)
   const size_t spare_bytes = 64 * kWaves * sizeof(float) * (tokcol ? (wide ? 2 : 1) * (four_tiles ? TW64 : TW) : 4 * TW);
   const size_t tile_bytes = stream_rows ? (size_t)kTileCopies : 0;
+  const size_t staged_spare = tokcol ? spare_bytes : 0;  // tokens as columns keep their spare slots behind the staged logits
   const int wgs_per_cu = argus_wgs_per_cu(ctx, kern, 64 * kWaves,
-                                          max_chunk > 0 ? (size_t)kStageBytes + tile_bytes : std::max(merge_bytes, spare_bytes + tile_bytes));
+                                          max_chunk > 0 ? (size_t)kStageBytes + staged_spare + tile_bytes : std::max(merge_bytes, spare_bytes + tile_bytes));
   choose_splits(p, batch * p.n_heads_kv, tile_rows, (int64_t)ctx->compute_units * wgs_per_cu, max_chunk);
   p.direct = 0;
   p.stage_scores = p.scores && p.chunk <= max_chunk;
-  const size_t lds_bytes = std::max(merge_bytes, (p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) : spare_bytes) + tile_bytes);
-  ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + kTileCopies + 1024));
+  const size_t lds_bytes = std::max(merge_bytes, (p.stage_scores ? (size_t)p.group * (p.chunk + 4) * sizeof(float) + staged_spare : spare_bytes) + tile_bytes);
+  ARGUS_HIP_CHECK(ctx, argus_raise_lds_limit(ctx, kern, kStageBytes + kTileCopies + (int)spare_bytes + 1024));
   const int rc = reserve_partials(ctx, p, batch, D);
   if (rc != ARGUS_HIP_OK) return rc;
   ctx->plan = argus_hip_decode_plan{p.nsplit, p.chunk, wgs_per_cu, (int32_t)lds_bytes, 2, 2, p.stage_scores};
