@@ -40,6 +40,7 @@ struct PrefillParams {
   int32_t n_heads_q, n_heads_kv, group;
   int32_t seq_len, cache_len, q_start, capacity, batch, window;
   int32_t n_qtiles, group_chunks;  // grid decomposition
+  int32_t unpaired;                // one query tile per workgroup, longest first (else the pair n-1-j, j)
   int32_t q_f16, out_f16;
   // F32 caches take two passes over the same kernel: V rounded to f16 first, then (v_residual) the
   // rounding's remainder v - f16(v), whose output is added to the first pass's (accumulate).
@@ -199,8 +200,8 @@ __global__ __launch_bounds__(64 * WPG * NG, (WPG * NG == 4 && D <= 128) ? ((D ==
   // Causal work grows linearly with the query tile index, so each workgroup takes the pair
   // (n_qtiles-1-jt, jt): every workgroup then carries the same number of key tiles.
   for (int pass = 0; pass < 2; ++pass) {
-  const int qt = pass == 0 ? (p.n_qtiles - 1 - jt) : jt;
-  if (pass == 1 && qt == p.n_qtiles - 1 - jt) break;
+  const int qt = (pass == 0 || p.unpaired) ? (p.n_qtiles - 1 - jt) : jt;
+  if (pass == 1 && (p.unpaired || qt == p.n_qtiles - 1 - jt)) break;
   const int qb = qt * QPW + wq / HPW;
   const int r0 = qb * 32;            // first query row of this wave
   const int row = r0 + ln;           // this lane's query row
@@ -756,7 +757,14 @@ int launch_ng(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
   constexpr int QPW = WPG / HPW;
   p.n_qtiles = (p.seq_len + 32 * QPW - 1) / (32 * QPW);
   p.group_chunks = p.group / (HPW * NH);
-  const int64_t wgs = (int64_t)p.batch * p.n_heads_kv * p.group_chunks * ((p.n_qtiles + 1) / 2);
+  // Workgroups take the query tiles in pairs (n-1-j, j) of equal total length, which balances a grid
+  // that is resident all at once.  A grid of four or more workgroups per CU is balanced by the order
+  // of dispatch instead: one tile per workgroup, longest first, and a workgroup's start-up runs beside
+  // its neighbours' loops (d 64, 16K tokens: 1,045 against 1,065-1,085 us; at 512 workgroups and
+  // below the pairs are 2-3 % faster).
+  const int64_t paired = (int64_t)p.batch * p.n_heads_kv * p.group_chunks * ((p.n_qtiles + 1) / 2);
+  p.unpaired = paired >= 4 * (int64_t)ctx->compute_units;
+  const int64_t wgs = p.unpaired ? (int64_t)p.batch * p.n_heads_kv * p.group_chunks * p.n_qtiles : paired;
   if (wgs > 0x7fffffff) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: grid too large");
   // two buffers of NG tile pairs; the merge of the KV groups reuses the space
   size_t lds_bytes = 2 * NG * (size_t)TL::HALFS * sizeof(_Float16);

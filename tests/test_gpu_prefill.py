@@ -110,6 +110,18 @@ def test_grid_that_fills_the_device_with_four_wave_workgroups(d):
     check_attention_out(got, O.prefill_attention(q.astype(np.float32), k, v, hkv, s, s))
 
 
+@pytest.mark.parametrize("hq,hkv,d,s,b", [(32, 32, 64, 512, 16), (32, 8, 64, 512, 32), (16, 16, 128, 384, 32)])
+def test_grid_of_four_workgroups_per_cu_takes_one_query_tile_each(hq, hkv, d, s, b):
+    # From 1024 workgroups on (256 CUs) the launcher stops pairing query tiles (n-1-j, j) and gives
+    # every workgroup one tile, longest first: many short sequences, ragged last tiles included.
+    q = f16(normal((b, s - 5, hq, d), 17))
+    k = f16(normal((b, hkv, s, d), 18))
+    v = f16(normal((b, hkv, s, d), 19))
+    rc, got = run_prefill(q, k, v, hkv, s - 5, s)
+    assert rc == 1
+    check_attention_out(got, O.prefill_attention(q.astype(np.float32), k, v, hkv, s - 5, s))
+
+
 def test_batched_prefill_with_capacity_and_offset():
     b, s, hq, hkv, d, cap, csl = 3, 150, 8, 2, 128, 400, 333
     q = normal((b, s, hq, d), 1)
