@@ -319,6 +319,34 @@ __device__ __forceinline__ void scaled_pair(const RawPiece<FMT> &a, const RawPie
   }
 }
 
+// The same for q2_0 (four 2-bit fields per byte): byte h of both tokens' pieces goes into one word
+// as [byte of a, 0, byte of b, 0] (`sel[h]`: the lane's v_perm selectors over {a's code dword, b's}),
+// and the two masks of piece_codes bring out one field of both tokens at a time: field f of byte h
+// is slot 2f + h of a whole piece (N = 8, two bytes) or slot f of a half piece (N = 4, one byte,
+// sel[0]).  Values are d * code (SCALED) or the operands slot bias + code.
+template <int N, bool SCALED>
+__device__ __forceinline__ void scaled_pair_q2(const RawPiece<kFmtQ2_0> &a, const RawPiece<kFmtQ2_0> &b, const uint32_t (&sel)[2], half2_t (&out)[N]) {
+  static_assert(N == 8 || N == 4, "whole or half pieces");
+  half2_t dd = {}, nb_a = {}, nb_b = {};
+  if constexpr (SCALED) {
+    dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b.hdr, a.hdr, 0x05040100u));  // {d_a, d_b}
+    nb_a = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};                            // exact
+    nb_b = dd * half2_t{(_Float16)-16.0f, (_Float16)-16.0f};
+  }
+  uint32_t mask_a = 0x00300030u, exp_a = 0x54005400u, mask_b = 0x00c000c0u, exp_b = 0x4c004c00u;
+  asm("" : "+v"(mask_a), "+v"(exp_a), "+v"(mask_b), "+v"(exp_b));
+  auto value = [&](half2_t code, half2_t nb) { return SCALED ? __builtin_elementwise_fma(code, dd, nb) : code; };
+  constexpr int NB = N / 4;  // bytes of the piece
+#pragma unroll
+  for (int h = 0; h < NB; ++h) {
+    const uint32_t w = __builtin_amdgcn_perm(b.code[0], a.code[0], sel[h]), w4 = w << 4;
+    out[0 * NB + h] = value(nibbles(w4, mask_a, exp_a), nb_a);  // field 0 -> bits 4..5: 64 + n
+    out[1 * NB + h] = value(nibbles(w4, mask_b, exp_b), nb_b);  // field 1 -> bits 6..7: 16 + n
+    out[2 * NB + h] = value(nibbles(w, mask_a, exp_a), nb_a);   // field 2
+    out[3 * NB + h] = value(nibbles(w, mask_b, exp_b), nb_b);   // field 3
+  }
+}
+
 // Half a piece (head_dim 64): the element held by slot s of the half `upper` of code index x, and
 // its 4 values d * code.  q4: `upper` selects the high nibbles, lined up by a per-lane shift so
 // that both halves run the same instructions; q8: the piece's one code dword is already the half;
@@ -812,6 +840,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // and for head_dim 64 which byte of the dword is its half piece
   const uint32_t k_sel = q2_half_selector(j & 1), v_sel = q2_half_selector(r & 1);
   const uint32_t v_half_sel = q2_byte_selector(2 * (r & 1) + (r >> 3));
+  // q2_0 V pieces of two tokens side by side (scaled_pair_q2): byte h of the lane's piece in both code dwords
+  uint32_t v_pair_sel[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint32_t at = (D == 64) ? (uint32_t)(2 * (r & 1) + (r >> 3)) : (uint32_t)(2 * (r & 1) + h);
+    v_pair_sel[h] = 0x0c000c00u | at | ((4u + at) << 16);
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) hdr_src[i] = 4 * (20 * j + i);  // ds_bpermute byte address
 
@@ -1198,11 +1233,14 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         // interleave the code words of two tokens before the nibbles come out (scaled_pair), so a
         // register holds one channel of two tokens and no value is moved afterwards; the others
         // dequantise token by token and transpose.
-        constexpr bool kPairV = FMT == kFmtQ4_0 || FMT == kFmtQ4_1;
+        constexpr bool kPairV = FMT == kFmtQ4_0 || FMT == kFmtQ4_1 || FMT == kFmtQ2_0;
         typedef _Float16 vrow_t __attribute__((ext_vector_type(VCH)));
         vrow_t vrow[4];
         half2_t vpair[2][VCH];
-        if constexpr (kPairV) {
+        if constexpr (FMT == kFmtQ2_0) {
+          scaled_pair_q2<VCH, !kScaleP>(vpc[0], vpc[1], v_pair_sel, vpair[0]);
+          scaled_pair_q2<VCH, !kScaleP>(vpc[2], vpc[3], v_pair_sel, vpair[1]);
+        } else if constexpr (kPairV) {
           scaled_pair<FMT, VCH, !kScaleP>(vpc[0], vpc[1], (uint32_t)(r >> 3), vpair[0]);
           scaled_pair<FMT, VCH, !kScaleP>(vpc[2], vpc[3], (uint32_t)(r >> 3), vpair[1]);
         } else {
