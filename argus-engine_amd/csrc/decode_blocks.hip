@@ -216,10 +216,8 @@ __device__ __forceinline__ half2_t nibbles(uint32_t word, uint32_t mask, uint32_
   return __builtin_bit_cast(half2_t, (word & mask) | exponent);
 }
 
-// v_perm selectors that spread one 16-bit half of a dword as [byte, 0, next byte, 0] (q2_0 pieces),
-// and one byte as [byte, 0, byte, 0] (q2_0 half pieces).
+// v_perm selector that spreads one 16-bit half of a dword as [byte, 0, next byte, 0] (q2_0 pieces).
 __device__ __forceinline__ uint32_t q2_half_selector(int half) { return half ? 0x0c030c02u : 0x0c010c00u; }
-__device__ __forceinline__ uint32_t q2_byte_selector(int byte) { return 0x0c000c00u | (uint32_t)byte | ((uint32_t)byte << 16); }
 
 // The 8 codes of a piece as exact f16 numbers Codec::slot_bias + code.  `sel` (q2_0 only): the
 // lane's q2_half_selector.
@@ -258,28 +256,6 @@ template <int FMT>
 __device__ __forceinline__ half8_t code_operand(const RawPiece<FMT> &p, uint32_t sel) {
   half2_t v[4];
   piece_codes<FMT>(p, v, sel);
-  return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
-}
-
-// The 8 values of a piece without zero point and minimum, d * code, rounded once to f16.
-template <int FMT>
-__device__ __forceinline__ half8_t scaled_codes(const RawPiece<FMT> &p, uint32_t sel) {
-  const half2_t dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u));  // {d, d}
-  half2_t v[4];
-  piece_codes<FMT>(p, v, sel);
-  if constexpr (FMT == kFmtQ8_0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = v[i] * dd;
-  } else if constexpr (FMT == kFmtQ2_0) {
-    const half2_t nb_a = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
-    const half2_t nb_b = dd * half2_t{(_Float16)-16.0f, (_Float16)-16.0f};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = __builtin_elementwise_fma(v[i], dd, (i & 1) ? nb_b : nb_a);
-  } else {
-    const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = __builtin_elementwise_fma(v[i], dd, nb);
-  }
   return half8_t{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
 }
 
@@ -347,59 +323,43 @@ __device__ __forceinline__ void scaled_pair_q2(const RawPiece<kFmtQ2_0> &a, cons
   }
 }
 
-// Half a piece (head_dim 64): the element held by slot s of the half `upper` of code index x, and
-// its 4 values d * code.  q4: `upper` selects the high nibbles, lined up by a per-lane shift so
-// that both halves run the same instructions; q8: the piece's one code dword is already the half;
-// q2_0: `sel` is the lane's q2_byte_selector (the half is one byte: four fields).
+// The same for q8_0: bytes 0, 1 (2, 3) of both tokens' code words go into one word as [a's, b's,
+// a's, b's], and the two byte spreads of piece_codes then yield one channel of both tokens each.
+// N = 8: two code words per token; N = 4 (head_dim 64): the half piece's one word.
+template <int N, bool SCALED>
+__device__ __forceinline__ void scaled_pair_q8(const RawPiece<kFmtQ8_0> &a, const RawPiece<kFmtQ8_0> &b, half2_t (&out)[N]) {
+  static_assert(N == 8 || N == 4, "whole or half pieces");
+  const half2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+  half2_t dd = {};
+  if constexpr (SCALED) dd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b.hdr, a.hdr, 0x05040100u));  // {d_a, d_b}
+#pragma unroll
+  for (int w = 0; w < N / 4; ++w)
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t u = __builtin_amdgcn_perm(b.code[w], a.code[w], k ? 0x07030602u : 0x05010400u) ^ 0x80808080u;
+      half2_t lo = bytes_lo(u) + off, hi = bytes_hi(u) + off;
+      if constexpr (SCALED) {
+        lo = lo * dd;
+        hi = hi * dd;
+      }
+      out[4 * w + 2 * k] = lo;
+      out[4 * w + 2 * k + 1] = hi;
+    }
+}
+
+// Half a piece (head_dim 64, where 8 lanes would cover the two blocks of a row twice over): the
+// element held by slot s of the half `upper` of code index x.  q4: `upper` selects the high nibbles;
+// q8: the piece's second code word; q2_0: its second byte.
 template <int FMT>
 __host__ __device__ constexpr int half_slot_elem(int x, int upper, int s) {
   if (FMT == kFmtQ8_0 || FMT == kFmtQ2_0) return 8 * x + 4 * upper + s;
   return 16 * upper + 4 * x + (s == 1 ? 2 : (s == 2 ? 1 : s));  // 0, 2, 1, 3
 }
-// The operand of half slot s is half_slot_bias(s) + code when SCALED is false.
+// The operand of half slot s is half_slot_bias(s) + code.
 template <int FMT>
 __host__ __device__ constexpr float half_slot_bias(int s) {
   return (FMT == kFmtQ8_0) ? 0.0f : ((FMT == kFmtQ2_0 && (s & 1)) ? 16.0f : 64.0f);
 }
-template <int FMT, bool SCALED>
-__device__ __forceinline__ half4_t scaled_half(const RawPiece<FMT> &p, uint32_t upper, uint32_t sel) {
-  const half2_t dd = SCALED ? __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, p.hdr, 0x01000100u)) : half2_t{};  // {d, d}
-  half2_t v[2];
-  if constexpr (FMT == kFmtQ2_0) {
-    const uint32_t w = __builtin_amdgcn_perm(0u, p.code[0], sel);  // [byte, 0, byte, 0]
-    uint32_t mask = 0x00c00030u, exponent = 0x4c005400u;           // low half: bits 4..5 (64 + n), high half: bits 6..7 (16 + n)
-    asm("" : "+v"(mask), "+v"(exponent));
-    const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-16.0f};  // exact
-    v[0] = nibbles(w << 4, mask, exponent);  // fields 0, 1
-    v[1] = nibbles(w, mask, exponent);       // fields 2, 3
-    if constexpr (SCALED) {
-      v[0] = __builtin_elementwise_fma(v[0], dd, nb);
-      v[1] = __builtin_elementwise_fma(v[1], dd, nb);
-    }
-  } else if constexpr (FMT == kFmtQ8_0) {
-    const half2_t off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
-    const uint32_t u = p.code[0] ^ 0x80808080u;
-    v[0] = bytes_lo(u) + off;
-    v[1] = bytes_hi(u) + off;
-    if constexpr (SCALED) {
-      v[0] = v[0] * dd;
-      v[1] = v[1] * dd;
-    }
-  } else {
-    const uint32_t w = p.code[0] << (4u - 4u * upper);  // the half's nibbles of bytes 0, 2 at bits 4..7
-    uint32_t mask = 0x00f000f0u, exponent = 0x54005400u;
-    asm("" : "+v"(mask), "+v"(exponent));
-    const half2_t nb = dd * half2_t{(_Float16)-64.0f, (_Float16)-64.0f};  // exact
-    v[0] = nibbles(w, mask, exponent);       // bytes 0, 2
-    v[1] = nibbles(w >> 8, mask, exponent);  // bytes 1, 3
-    if constexpr (SCALED) {
-      v[0] = __builtin_elementwise_fma(v[0], dd, nb);
-      v[1] = __builtin_elementwise_fma(v[1], dd, nb);
-    }
-  }
-  return half4_t{v[0][0], v[0][1], v[1][0], v[1][1]};
-}
-
 // One element of a block as f32 (rare paths only).
 template <int FMT>
 __device__ float block_elem(const uint8_t *blk, int e) {
@@ -836,11 +796,10 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
   // Result lane (j, h) of a logits MFMA holds tokens 4j..4j+3; their block headers were loaded by
   // lanes 16j + (4j + i) (token = lane % 16).
   int hdr_src[4];
-  // q2_0: which 16-bit half of a code dword is this lane's piece (K: code index j; V: code index r % 4),
-  // and for head_dim 64 which byte of the dword is its half piece
-  const uint32_t k_sel = q2_half_selector(j & 1), v_sel = q2_half_selector(r & 1);
-  const uint32_t v_half_sel = q2_byte_selector(2 * (r & 1) + (r >> 3));
-  // q2_0 V pieces of two tokens side by side (scaled_pair_q2): byte h of the lane's piece in both code dwords
+  // q2_0: which 16-bit half of a code dword is this lane's K piece (code index j)
+  const uint32_t k_sel = q2_half_selector(j & 1);
+  // q2_0 V pieces of two tokens side by side (scaled_pair_q2): byte h of the lane's piece (code index
+  // r % 4; head_dim 64: the one byte of its half piece) in both code dwords
   uint32_t v_pair_sel[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -1229,27 +1188,19 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
           for (int e = 0; e < 4; ++e) vpc[e] = vraw[tw][sg][e];
         }
-        // The V operand of channel c wants the four tokens' values side by side.  The 4-bit formats
-        // interleave the code words of two tokens before the nibbles come out (scaled_pair), so a
-        // register holds one channel of two tokens and no value is moved afterwards; the others
-        // dequantise token by token and transpose.
-        constexpr bool kPairV = FMT == kFmtQ4_0 || FMT == kFmtQ4_1 || FMT == kFmtQ2_0;
-        typedef _Float16 vrow_t __attribute__((ext_vector_type(VCH)));
-        vrow_t vrow[4];
+        // The V operand of channel c wants the four tokens' values side by side: the code words of two
+        // tokens are interleaved before the codes come out (scaled_pair*), so a register holds one
+        // channel of two tokens and no value is moved afterwards.
         half2_t vpair[2][VCH];
         if constexpr (FMT == kFmtQ2_0) {
           scaled_pair_q2<VCH, !kScaleP>(vpc[0], vpc[1], v_pair_sel, vpair[0]);
           scaled_pair_q2<VCH, !kScaleP>(vpc[2], vpc[3], v_pair_sel, vpair[1]);
-        } else if constexpr (kPairV) {
+        } else if constexpr (FMT == kFmtQ8_0) {
+          scaled_pair_q8<VCH, !kScaleP>(vpc[0], vpc[1], vpair[0]);
+          scaled_pair_q8<VCH, !kScaleP>(vpc[2], vpc[3], vpair[1]);
+        } else {
           scaled_pair<FMT, VCH, !kScaleP>(vpc[0], vpc[1], (uint32_t)(r >> 3), vpair[0]);
           scaled_pair<FMT, VCH, !kScaleP>(vpc[2], vpc[3], (uint32_t)(r >> 3), vpair[1]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if constexpr (D == 64) vrow[e] = scaled_half<FMT, !kScaleP>(vpc[e], (uint32_t)(r >> 3), v_half_sel);
-            else if constexpr (kScaleP) vrow[e] = code_operand<FMT>(vpc[e], v_sel);
-            else vrow[e] = scaled_codes<FMT>(vpc[e], v_sel);
-          }
         }
         if constexpr (kHdrTerm && (!kScaleP || F::kHasMin)) {
           // d (q4_0: low halves of the headers) or m (q4_1, q2_0: high halves) of the lane's four tokens
@@ -1264,10 +1215,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
           dv = __builtin_bit_cast(half4_t, u32x2_t{d01, d23});
         }
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) {
-          if constexpr (kPairV) bv[c] = half4_t{vpair[0][c][0], vpair[0][c][1], vpair[1][c][0], vpair[1][c][1]};
-          else bv[c] = half4_t{vrow[0][c], vrow[1][c], vrow[2][c], vrow[3][c]};
-        }
+        for (int c = 0; c < VCH; ++c) bv[c] = half4_t{vpair[0][c][0], vpair[0][c][1], vpair[1][c][0], vpair[1][c][1]};
     };
     const half4_t ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
     if constexpr (TW == 2 && TOKCOL && D == 128) {
