@@ -412,7 +412,7 @@ def cpu_baseline_decode(hq, hkv, d, L, budget_s=12.0):
 # scaled by what the same counters read for a plain 1 GiB copy (x2.000 and x1.000).  Counters cannot
 # be read from inside this process, so the figure is the one of the profile run named beside it in
 # the output (`traffic_source`), not a measurement of this run.
-DECODE_TRAFFIC_BYTES = 2_161_393_081
+DECODE_TRAFFIC_BYTES = 2_161_394_139
 DECODE_TRAFFIC_SOURCE = "profiles/decode_mfma_cfg3_L32768_b16_hbm_traffic.md"
 
 
