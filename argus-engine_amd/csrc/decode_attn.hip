@@ -119,16 +119,32 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecodeParams p)
     constexpr bool FULL = decltype(full_tag)::value;
     vec_t kr[U], vr[U];
     bool valid[U];
+    int64_t slot[U];
+    int tc[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = base + u * RPW + grp;
       valid[u] = FULL || t < t_end;
-      const int tc = valid[u] ? t : (t_end - 1);
+      tc[u] = valid[u] ? t : (t_end - 1);
+    }
+    if (use_idx) {  // uniform
+      // The list entries of all U rows are requested together and before the rows: read one by one
+      // between the rows, every entry's wait also waited for the rows requested before it.
+      uint32_t entry[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) entry[u] = (uint32_t)idx[tc[u]];
       // a slot outside the cache (stale or negative list entry) is clamped to the last one: the rows
       // are fetched with plain loads, which nothing else bounds
-      const int64_t slot = use_idx ? (int64_t)min((uint32_t)idx[tc], (uint32_t)(p.slot_bound - 1)) : (int64_t)(p.kv_start + tc);
-      kr[u] = load_row_piece<KV_T>(p, p.k, head_elem, slot, c0);
-      vr[u] = load_row_piece<KV_T>(p, p.v, head_elem, slot, c0);
+#pragma unroll
+      for (int u = 0; u < U; ++u) slot[u] = (int64_t)min(entry[u], (uint32_t)(p.slot_bound - 1));
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) slot[u] = (int64_t)(p.kv_start + tc[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      kr[u] = load_row_piece<KV_T>(p, p.k, head_elem, slot[u], c0);
+      vr[u] = load_row_piece<KV_T>(p, p.v, head_elem, slot[u], c0);
     }
 
     float s[U][GT];
