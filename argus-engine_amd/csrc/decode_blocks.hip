@@ -623,7 +623,17 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     }
   };
   // V piece of token 4j + e of tile tw: block vblk[sg], code index r % 4 (head_dim 64, q8_0: the
-  // lane's half of the piece, one dword); the lane's offsets into a row are fixed
+  // lane's half of the piece, one dword); the lane's offsets into a row are fixed.
+  // Tokens as columns: the contraction slots of the output MFMAs may hold the tile's tokens in any
+  // order as long as the P operand follows, and P passes through LDS anyway.  Slot 4j + e is token
+  // j + 4e at head_dim 64: one read instruction (fixed e) then takes four neighbouring rows, whose
+  // dwords lie side by side in the copy, instead of four rows 4 RD dwords apart (36 dwords for q4_0:
+  // lane groups 0 and 1 four banks apart; q4_0 +3..7 % with four heads per KV head and +1..3 % with
+  // seven, q4_1 +1..2 %, q2_0 and q8_0 alike).
+  // Rows of head_dim 128 span more than half the banks, two lane groups collide wherever their rows
+  // lie, and the counters agree: q4_0 the same conflict cycles either way, q8_0 a third more and q2_0
+  // 3 % slower with neighbouring rows.
+  constexpr bool kSpreadV = TOKCOL != 0 && STREAM && D == 64;
   uint32_t v_blk_byte[VSEG], v_code_dw[VSEG], v_sh[VSEG];
 #pragma unroll
   for (int sg = 0; sg < VSEG; ++sg) {
@@ -637,7 +647,7 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     v_sh[sg] = a & 3u;
   }
   auto v_piece = [&](int tw, int sg, int e) {
-    const uint32_t *row = v_tile + (16 * tw + 4 * j + e) * RD;
+    const uint32_t *row = v_tile + (16 * tw + (kSpreadV ? j + 4 * e : 4 * j + e)) * RD;
     if constexpr (FMT == kFmtQ8_0 && D == 64) {  // half a piece: one code dword
       RawPiece<FMT> pc;
       pc.hdr = *(const uint16_t *)((const uint8_t *)row + v_blk_byte[sg]);
@@ -983,12 +993,13 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
         }
       }
       // (token, head) -> the P operand: lane (j, r) wants tokens 4j..4j+3 of the head of its row
+      // (kSpreadV: tokens j, j + 4, j + 8, j + 12, so token r is written to place 4 (r % 4) + r / 4)
       __shared__ __attribute__((aligned(16))) uint32_t p_strip[kWaves][NPD][4 * HL][16];  // 64 words per four heads: writes and reads each touch every bank once
       wave_lds_fence();  // the previous iteration's reads are done
 #pragma unroll
       for (int u = 0; u < HL; ++u)
 #pragma unroll
-        for (int d2 = 0; d2 < NPD; ++d2) p_strip[wave][d2][HL * j + u][r] = __builtin_bit_cast(uint32_t, pk[u][d2]);
+        for (int d2 = 0; d2 < NPD; ++d2) p_strip[wave][d2][HL * j + u][kSpreadV ? 4 * (r & 3) + (r >> 2) : r] = __builtin_bit_cast(uint32_t, pk[u][d2]);
       wave_lds_fence();
 #pragma unroll
       for (int q = 0; q < NQ; ++q)

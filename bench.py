@@ -170,23 +170,23 @@ def bench_decode(ctx, hq, hkv, d, L, batch, steps, warmup, capacity=None, scores
 
 
 def bench_decode_blocks(ctx, fmt, hq, hkv, d, L, batch, steps, warmup, rotate=1, scores=False, stats=False):
-    """Decode attention over a block-quantised cache (q4_0 / q8_0 / q2_0 rows of 18- / 34- / 12-byte blocks):
+    """Decode attention over a block-quantised cache (q4_0 / q4_1 / q8_0 / q2_0 rows of 18- / 20- / 34- / 12-byte blocks):
     synthetic blocks (random codes, f16 scales sized for N(0,1)-like values); algorithmic bytes are
     the attended block rows of K and V plus Q and out."""
     import torch
     import argus_hip as A
-    bb = {"q4_0": 18, "q8_0": 34, "q2_0": 12}[fmt]
-    kv_dtype = {"q4_0": A.Q4_0, "q8_0": A.Q8_0, "q2_0": A.Q2_0}[fmt]
+    bb = {"q4_0": 18, "q4_1": 20, "q8_0": 34, "q2_0": 12}[fmt]
+    kv_dtype = {"q4_0": A.Q4_0, "q4_1": A.Q4_1, "q8_0": A.Q8_0, "q2_0": A.Q2_0}[fmt]
     row_bytes = d // 32 * bb
     g = torch.Generator(device="cuda").manual_seed(11)
 
     def blocks():
         raw = torch.randint(0, 256, (batch * hkv * L * d // 32, bb), generator=g, device="cuda", dtype=torch.uint8)
-        lo, hi = {"q4_0": (0.1, 0.3), "q8_0": (0.005, 0.02), "q2_0": (0.8, 1.6)}[fmt]
+        lo, hi = {"q4_0": (0.1, 0.3), "q4_1": (0.1, 0.3), "q8_0": (0.005, 0.02), "q2_0": (0.8, 1.6)}[fmt]
         scale = (torch.rand(raw.shape[0], generator=g, device="cuda") * (hi - lo) + lo).half()
         raw[:, 0:2] = scale.view(torch.uint8).reshape(-1, 2)
-        if fmt == "q2_0":  # [f16 d][f16 m]: minimum at -1.5 d
-            raw[:, 2:4] = (scale.float() * -1.5).half().view(torch.uint8).reshape(-1, 2)
+        if fmt in ("q2_0", "q4_1"):  # [f16 d][f16 m]: minimum at half the code range below zero
+            raw[:, 2:4] = (scale.float() * (-1.5 if fmt == "q2_0" else -7.5)).half().view(torch.uint8).reshape(-1, 2)
         return raw.reshape(-1)
 
     ks = [blocks() for _ in range(rotate)]
