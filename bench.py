@@ -487,7 +487,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="primary",
                     choices=["primary", "decode_b1", "prefill", "prefill_d128", "kivi_q4", "kivi_q8", "cfg5", "q4_0", "q4_0_b1", "primary_scores_stats",
-                             "q8_0", "copy_calib", "aux", "layers", "primary_scores", "cfg5_b64", "prefill_d64_16k"],
+                             "q8_0", "q4_0_d64", "copy_calib", "aux", "layers", "primary_scores", "cfg5_b64", "prefill_d64_16k"],
                     help="run one secondary workload alone (for profiling) instead of the primary line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -533,6 +533,8 @@ def main():
             res = bench_prefill(ctx, args.steps, args.warmup, hq=32, hkv=8, d=64, s=16384)
         elif w in ("q4_0", "q8_0"):
             res = bench_decode_blocks(ctx, w, 32, 8, 128, 32768, 16, args.steps, args.warmup)
+        elif w == "q4_0_d64":
+            res = bench_decode_blocks(ctx, "q4_0", 14, 2, 64, 32768, 64, args.steps, args.warmup)
         elif w == "q4_0_b1":
             res = bench_decode_blocks(ctx, "q4_0", 32, 8, 128, 32768, 1, args.steps, args.warmup, rotate=8)
         elif w == "cfg5":
