@@ -45,6 +45,14 @@ namespace argus_decode {
 namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+// LDS as 32-bit addresses (the streamed tile copies are read through lane bases kept as integers)
+typedef const __attribute__((address_space(3))) uint32_t *lds_u32_ptr;
+typedef const __attribute__((address_space(3))) uint16_t *lds_u16_ptr;
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+__device__ __forceinline__ uint32_t lds_dword(uint32_t addr) { return *(lds_u32_ptr)(uintptr_t)addr; }
+__device__ __forceinline__ uint32_t lds_half(uint32_t addr) { return *(lds_u16_ptr)(uintptr_t)addr; }
 typedef uint32_t u32_a2 __attribute__((aligned(2)));  // code words sit at 2-byte boundaries (18- and 34-byte blocks)
 
 enum { kFmtQ4_0 = 0, kFmtQ4_1 = 1, kFmtQ8_0 = 2, kFmtQ2_0 = 3 };
@@ -581,46 +589,57 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     }
     wave_lds_fence();
   };
-  // Piece (code index x, CW dwords) of block blk of a parked row.  With a 2-byte header the code
-  // words of every other block straddle dwords: `sh` = 2 there, 0 where they are aligned.
-  auto parked_piece = [&](const uint32_t *row, uint32_t blk_byte, uint32_t code_dw, uint32_t sh) {
-    RawPiece<FMT> pc;
-    if constexpr (F::HDR == 4) {
-      pc.hdr = row[blk_byte / 4];
-#pragma unroll
-      for (int w = 0; w < F::CW; ++w) pc.code[w] = row[code_dw + w];
-    } else {
-      pc.hdr = *(const uint16_t *)((const uint8_t *)row + blk_byte);
-      uint32_t d[F::CW + 1];
-#pragma unroll
-      for (int w = 0; w <= F::CW; ++w) d[w] = row[code_dw + w];
-#pragma unroll
-      for (int w = 0; w < F::CW; ++w) pc.code[w] = __builtin_amdgcn_alignbyte(d[w + 1], d[w], sh);
-    }
-    return pc;
+  // Reads of a parked tile.  The two-dword reads (ds_read2_b32) carry their constant offset in an
+  // 8-bit field of dwords, so a lane base reaches 1020 bytes; left to itself the compiler covers the
+  // rest of the copy with an address add in front of every read (30 a wave iteration at head_dim 64,
+  // where the vector ALU is the limit).  The lane bases are therefore kept as integers the compiler
+  // cannot re-derive, one per group of kTilesPerBase tiles, and every read adds a constant that fits.
+  constexpr int kRowsAhead = (TOKCOL != 0 && STREAM && D == 64) ? 12 : 3;  // furthest row of a V read past the lane's first (see kSpreadV)
+  // (K: a row's blocks lie up to a row further on; V: the base points at the lane's code dword already)
+  constexpr auto reads_fit = [](int tiles) {
+    return 16 * (tiles - 1) * RBY + RBY <= 1020 && (16 * (tiles - 1) + kRowsAhead) * RBY + 4 * F::CW <= 1020;
   };
+  // Where it pays: head_dim 64 (q8_0 apart, which is short of registers and not bound by the vector
+  // ALU); elsewhere one base and the compiler's own adds (the pinned bases cost the 128- and
+  // 256-wide kernels 8 to 22 registers and some of them spills).
+  constexpr bool kPinBases = D == 64 && FMT != kFmtQ8_0;
+  constexpr int kTilesPerBase = !kPinBases || reads_fit(TW) ? TW : (TW >= 2 && reads_fit(TW / 2)) ? TW / 2 : 1;
+  constexpr int NB = TW / kTilesPerBase;
+  static_assert(NB * kTilesPerBase == TW, "groups of tiles divide the iteration");
   // K operand piece of token r of tile tw: code index j of block kk (q2_0: the dword that holds half j)
+  uint32_t k_hdr_at = 0, k_code_at[NB] = {};
+  if constexpr (STREAM) {
+    k_hdr_at = lds_address(k_tile) + 4u * (uint32_t)(r * RD);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      k_code_at[nb] = lds_address(k_tile) + 4u * (uint32_t)((16 * kTilesPerBase * nb + r) * RD + ((FMT == kFmtQ2_0) ? (j >> 1) : F::CW * j));
+      if constexpr (kPinBases) asm volatile("" : "+v"(k_code_at[nb]));
+    }
+  }
   auto k_piece = [&](int tw, int kk) {
-    const uint32_t *row = k_tile + (16 * tw + r) * RD;
+    RawPiece<FMT> pc;
     const uint32_t blk = (uint32_t)(kk * F::BB);
+    const uint32_t row = (uint32_t)(16 * (tw % kTilesPerBase) * RBY);  // bytes from the base's first tile
+    const uint32_t code = k_code_at[tw / kTilesPerBase] + row + (blk + (uint32_t)F::HDR) / 4u * 4u;
     if constexpr (F::HDR == 4) {
-      return parked_piece(row, blk, blk / 4 + 1 + ((FMT == kFmtQ2_0) ? (uint32_t)(j >> 1) : (uint32_t)(F::CW * j)), 0u);
+      pc.hdr = lds_dword(k_hdr_at + (uint32_t)(16 * tw * RBY) + blk);
+#pragma unroll
+      for (int w = 0; w < F::CW; ++w) pc.code[w] = lds_dword(code + 4u * (uint32_t)w);
     } else {
-      const uint32_t a = blk + 2u + 4u * (uint32_t)(F::CW * j);  // first code byte; a % 4 is the block's, known at compile time
-      RawPiece<FMT> pc;
-      pc.hdr = *(const uint16_t *)((const uint8_t *)row + blk);
+      pc.hdr = lds_half(k_hdr_at + (uint32_t)(16 * tw * RBY) + blk);
+      // with a 2-byte header the code words of every other block straddle dwords
       if ((kk * F::BB) % 4 == 0) {
         uint32_t d[F::CW + 1];
 #pragma unroll
-        for (int w = 0; w <= F::CW; ++w) d[w] = row[a / 4 + w];
+        for (int w = 0; w <= F::CW; ++w) d[w] = lds_dword(code + 4u * (uint32_t)w);
 #pragma unroll
         for (int w = 0; w < F::CW; ++w) pc.code[w] = __builtin_amdgcn_alignbyte(d[w + 1], d[w], 2u);
       } else {
 #pragma unroll
-        for (int w = 0; w < F::CW; ++w) pc.code[w] = row[a / 4 + w];
+        for (int w = 0; w < F::CW; ++w) pc.code[w] = lds_dword(code + 4u * (uint32_t)w);
       }
-      return pc;
     }
+    return pc;
   };
   // V piece of token 4j + e of tile tw: block vblk[sg], code index r % 4 (head_dim 64, q8_0: the
   // lane's half of the piece, one dword); the lane's offsets into a row are fixed.
@@ -646,17 +665,42 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
     v_code_dw[sg] = a / 4;
     v_sh[sg] = a & 3u;
   }
-  auto v_piece = [&](int tw, int sg, int e) {
-    const uint32_t *row = v_tile + (16 * tw + (kSpreadV ? j + 4 * e : 4 * j + e)) * RD;
-    if constexpr (FMT == kFmtQ8_0 && D == 64) {  // half a piece: one code dword
-      RawPiece<FMT> pc;
-      pc.hdr = *(const uint16_t *)((const uint8_t *)row + v_blk_byte[sg]);
-      pc.code[0] = __builtin_amdgcn_alignbyte(row[v_code_dw[sg] + 1], row[v_code_dw[sg]], v_sh[sg]);
-      pc.code[1] = 0u;
-      return pc;
-    } else {
-      return parked_piece(row, v_blk_byte[sg], v_code_dw[sg], v_sh[sg]);
+  static_assert(kRowsAhead == (kSpreadV ? 12 : 3), "the furthest row of a V read");
+  uint32_t v_hdr_at[VSEG] = {}, v_code_at[NB][VSEG] = {};
+  if constexpr (STREAM) {
+#pragma unroll
+    for (int sg = 0; sg < VSEG; ++sg) {
+      const uint32_t first = lds_address(v_tile) + 4u * (uint32_t)((kSpreadV ? j : 4 * j) * RD);  // the lane's first row of tile 0
+      v_hdr_at[sg] = first + v_blk_byte[sg];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        v_code_at[nb][sg] = first + 4u * (uint32_t)(16 * kTilesPerBase * nb * RD) + 4u * v_code_dw[sg];
+        if constexpr (kPinBases) asm volatile("" : "+v"(v_code_at[nb][sg]));
+      }
     }
+  }
+  auto v_piece = [&](int tw, int sg, int e) {
+    RawPiece<FMT> pc;
+    const uint32_t rows = (uint32_t)(kSpreadV ? 4 * e : e);  // rows past the lane's first
+    const uint32_t code = v_code_at[tw / kTilesPerBase][sg] + (uint32_t)(16 * (tw % kTilesPerBase) * RBY) + rows * (uint32_t)RBY;
+    const uint32_t hdr = v_hdr_at[sg] + (uint32_t)(16 * tw * RBY) + rows * (uint32_t)RBY;
+    if constexpr (F::HDR == 4) {
+      pc.hdr = lds_dword(hdr);
+#pragma unroll
+      for (int w = 0; w < F::CW; ++w) pc.code[w] = lds_dword(code + 4u * (uint32_t)w);
+    } else if constexpr (FMT == kFmtQ8_0 && D == 64) {  // half a piece: one code dword
+      pc.hdr = lds_half(hdr);
+      pc.code[0] = __builtin_amdgcn_alignbyte(lds_dword(code + 4u), lds_dword(code), v_sh[sg]);
+      pc.code[1] = 0u;
+    } else {
+      pc.hdr = lds_half(hdr);
+      uint32_t d[F::CW + 1];
+#pragma unroll
+      for (int w = 0; w <= F::CW; ++w) d[w] = lds_dword(code + 4u * (uint32_t)w);
+#pragma unroll
+      for (int w = 0; w < F::CW; ++w) pc.code[w] = __builtin_amdgcn_alignbyte(d[w + 1], d[w], v_sh[sg]);
+    }
+    return pc;
   };
   // Rows past the chunk re-read its last row (they are masked below), so every request is
   // unconditional and a tile may be asked for before it is known to exist.
@@ -887,15 +931,20 @@ __global__ __launch_bounds__(64 * kWaves, (D == 64) ? 4 : (D == 128) ? ((FMT == 
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
           const half8_t kb_op = code_operand<FMT>(kpc[kk], k_sel);
+          // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q: the second term
+          // is what the accumulator of the high part starts from
+          // (head_dim 64, where the vector ALU is the limit and the two accumulator tuples fit; added
+          // behind the MFMA elsewhere)
+          constexpr bool kStartFromInit = D == 64 && FMT != kFmtQ8_0;
           float4_t dot = {0.0f, 0.0f, 0.0f, 0.0f};
+          if constexpr (kStartFromInit) dot = float4_t{qinit[kk][0], 0.0f, (HL == 2) ? qinit[kk][HL - 1] : 0.0f, 0.0f};
           dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[kk], kb_op, dot, 0, 0, 0);
-          // sum of (code - zero) * q = sum of operand * q - sum of (bias + zero) * q, times the
-          // token's scale for this block, which the lane holds itself
+          // ... times the token's scale for this block, which the lane holds itself
           const half2_t dm = __builtin_bit_cast(half2_t, kpc[kk].hdr);
 #pragma unroll
           for (int u = 0; u < HL; ++u) {
             // high and low parts: registers 0 and 1 (two heads per lane: 2u and 2u + 1)
-            const float mine = (dot[2 * u] + qinit[kk][u]) + dot[2 * u + 1];
+            const float mine = kStartFromInit ? dot[2 * u] + dot[2 * u + 1] : (dot[2 * u] + qinit[kk][u]) + dot[2 * u + 1];
             if constexpr (F::kHasMin) sc[tw][u] = fmaf((float)dm[0], mine, fmaf((float)dm[1], qsum[kk][u], sc[tw][u]));
             else sc[tw][u] = fmaf((float)dm[0], mine, sc[tw][u]);
           }
