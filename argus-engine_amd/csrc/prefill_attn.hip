@@ -684,6 +684,72 @@ __global__ __launch_bounds__(64 * WPG * NG, (WPG * NG == 4 && D <= 128) ? ((D ==
     }
   }
 
+  // ---- merge the KV groups through LDS, normalise and store --------------------------------------
+  // Two groups trade halves: each hands the other (m, l) and one half of its O^T row blocks, merges
+  // the half it keeps and stores it, so both do half the LDS traffic, half the arithmetic and half
+  // the stores of a one-sided merge and neither waits for the other to finish.
+  constexpr bool kTradeHalves = NG == 2 && RB % 2 == 0;
+  if constexpr (kTradeHalves) {
+#pragma unroll
+    for (int n = 0; n < NH; ++n) l_run[n] += __shfl_xor(l_run[n], 32, 64);
+    constexpr int KEEP = RB / 2;  // row blocks a group ends up with
+    float *mrg = (float *)smem;   // [2 senders][WPG query waves][NH][KEEP*16 + 2][64 lanes]
+    constexpr int SLOTS = KEEP * 16 + 2;
+    auto hand_over = [&](auto first_c) {  // row blocks [FIRST, FIRST + KEEP) go to the other group
+      constexpr int FIRST = decltype(first_c)::value;
+#pragma unroll
+      for (int n = 0; n < NH; ++n) {
+        float *dst = mrg + ((kvg * WPG + wq) * NH + n) * SLOTS * 64 + lane;
+#pragma unroll
+        for (int r = 0; r < KEEP; ++r)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) dst[(r * 16 + i) * 64] = o_acc[n][FIRST + r][i];
+        dst[KEEP * 16 * 64] = m_run[n];
+        dst[(KEEP * 16 + 1) * 64] = l_run[n];
+      }
+    };
+    // ... the other group's [FIRST, FIRST + KEEP) are merged into this one's, normalised and stored
+    // (lane = query row, registers = channels)
+    auto take_and_store = [&](auto first_c) {
+      constexpr int FIRST = decltype(first_c)::value;
+#pragma unroll
+      for (int n = 0; n < NH; ++n) {
+        const float *src = mrg + (((1 - kvg) * WPG + wq) * NH + n) * SLOTS * 64 + lane;
+        const float m_o = src[KEEP * 16 * 64], l_o = src[(KEEP * 16 + 1) * 64];
+        const float m_new = fmaxf(m_run[n], m_o);
+        const float m_to = (m_new == kNegInf) ? 0.0f : m_new;
+        const float fa = __builtin_amdgcn_exp2f(m_run[n] - m_to), fb = __builtin_amdgcn_exp2f(m_o - m_to);
+        const float l_all = l_run[n] * fa + l_o * fb;
+        const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+        const int64_t ooff = (((int64_t)b * p.seq_len + row) * p.n_heads_q + h0 + n) * D;
+#pragma unroll
+        for (int r = 0; r < KEEP; ++r)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4) {
+            float4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (o_acc[n][FIRST + r][4 * i4 + e] * fa + src[(r * 16 + 4 * i4 + e) * 64] * fb) * inv;
+            const int d0 = 32 * (FIRST + r) + 8 * i4 + 4 * hl;
+            if (!row_ok) continue;
+            if (p.out_f16) {
+              half4_t oh = {(_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3]};
+              *(half4_t *)((_Float16 *)p.out + ooff + d0) = oh;
+            } else {
+              float4_t *dst = (float4_t *)((float *)p.out + ooff + d0);
+              if (p.accumulate) o += *dst;
+              *dst = o;
+            }
+          }
+      }
+    };
+    typedef std::integral_constant<int, 0> Lower;
+    typedef std::integral_constant<int, KEEP> Upper;
+    if (kvg == 0) hand_over(Upper{});
+    else hand_over(Lower{});
+    __syncthreads();
+    if (kvg == 0) take_and_store(Lower{});
+    else take_and_store(Upper{});
+  } else {
   // ---- merge the KV groups: groups > 0 hand (m, l, O^T) to group 0 through LDS ---------------
 #pragma unroll
   for (int n = 0; n < NH; ++n) l_run[n] += __shfl_xor(l_run[n], 32, 64);
@@ -747,6 +813,7 @@ __global__ __launch_bounds__(64 * WPG * NG, (WPG * NG == 4 && D <= 128) ? ((D ==
     }
   }
   }
+  }
   __syncthreads();  // the merge area is free again before the next pass stages tiles into it
   }  // pass
 }
@@ -768,7 +835,8 @@ int launch_ng(argus_hip_ctx *ctx, PrefillParams &p, hipStream_t stream) {
   if (wgs > 0x7fffffff) return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: grid too large");
   // two buffers of NG tile pairs; the merge of the KV groups reuses the space
   size_t lds_bytes = 2 * NG * (size_t)TL::HALFS * sizeof(_Float16);
-  const size_t merge_bytes = (size_t)(NG - 1) * WPG * NH * (D / 32 * 16 + 2) * 64 * sizeof(float);
+  // (two groups trade halves of their row blocks, each with its (m, l); more hand whole rows to group 0)
+  const size_t merge_bytes = (NG == 2 ? (size_t)2 * WPG * NH * (D / 64 * 16 + 2) : (size_t)(NG - 1) * WPG * NH * (D / 32 * 16 + 2)) * 64 * sizeof(float);
   if (merge_bytes > lds_bytes) lds_bytes = merge_bytes;
   if (lds_bytes > ctx->props.sharedMemPerBlock)
     return argus_fail(ctx, ARGUS_HIP_ERR_UNSUPPORTED, "prefill: %zu bytes of LDS needed, %zu available", lds_bytes,
